@@ -1,0 +1,259 @@
+"""Pins the CPU oracle against things that do not come from the oracle itself: torch's fp64 conv2d,
+hand-computed cases, closed forms and invariants.  The reference holds no golden vectors for this path
+(its tests are differential against a CPU backend that is a separate project)."""
+import numpy as np
+import pytest
+import torch
+
+RNG = np.random.default_rng(0xA70CAD0)
+
+
+def torch_conv(x, w, pad, stride=(1, 1), dilation=(1, 1), groups=1):
+    """NHWC/KRSC fp64 cross-check: Avocado CONVOLUTION mode == torch conv2d (no kernel flip), padding = -offset."""
+    xt = torch.from_numpy(np.ascontiguousarray(x.transpose(0, 3, 1, 2)))
+    wt = torch.from_numpy(np.ascontiguousarray(w.transpose(0, 3, 1, 2)))
+    y = torch.nn.functional.conv2d(xt, wt, None, stride, (-pad[0], -pad[1]), dilation, groups)
+    return y.numpy().transpose(0, 2, 3, 1)
+
+
+@pytest.mark.parametrize("shape", [
+    dict(x=(2, 7, 9, 5), w=(4, 3, 3, 5), pad=(-1, -1)),
+    dict(x=(3, 8, 8, 6), w=(7, 5, 5, 6), pad=(-2, -2)),
+    dict(x=(2, 6, 5, 8), w=(3, 1, 1, 8), pad=(0, 0)),
+    dict(x=(2, 11, 12, 4), w=(6, 3, 3, 4), pad=(-1, -1), stride=(2, 2)),
+    dict(x=(1, 9, 9, 3), w=(2, 3, 3, 3), pad=(-2, -2), dilation=(2, 2)),
+    dict(x=(2, 6, 6, 8), w=(4, 3, 3, 4), pad=(-1, -1), groups=2),
+    dict(x=(2, 6, 7, 3), w=(4, 3, 3, 3), pad=(0, 0)),
+])
+def test_conv_matches_torch_fp64(oracle, shape):
+    x = RNG.standard_normal(shape["x"])
+    w = RNG.standard_normal(shape["w"])
+    kw = {k: v for k, v in shape.items() if k in ("stride", "dilation", "groups")}
+    got = oracle.conv2d(x, w, pad=shape["pad"], **kw)
+    want = torch_conv(x, w, shape["pad"], **kw)
+    assert got.shape == want.shape
+    np.testing.assert_allclose(got, want, rtol=0, atol=1e-12)
+
+
+def test_cross_correlation_mode_flips_the_kernel(oracle):
+    x = RNG.standard_normal((2, 6, 7, 3))
+    w = RNG.standard_normal((4, 3, 3, 3))
+    got = oracle.conv2d(x, w, mode=oracle.CROSS_CORRELATION)
+    want = torch_conv(x, np.ascontiguousarray(w[:, ::-1, ::-1, :]), (-1, -1))
+    np.testing.assert_allclose(got, want, atol=1e-12)
+
+
+def test_conv_hand_computed(oracle):
+    # 1 image 3x3, 1 channel, values 1..9; 3x3 kernel of taps 1..9; offset -1.
+    x = np.arange(1, 10, dtype=np.float64).reshape(1, 3, 3, 1)
+    w = np.arange(1, 10, dtype=np.float64).reshape(1, 3, 3, 1)
+    y = oracle.conv2d(x, w)
+    # centre: sum i*i = 285; corner (0,0): taps 5,6,8,9 over pixels 1,2,4,5 = 5+12+32+45 = 94
+    assert y[0, 1, 1, 0] == 285.0
+    assert y[0, 0, 0, 0] == 94.0
+    # corner (2,2): taps 1,2,4,5 over pixels 5,6,8,9 = 5+12+32+45 = 94
+    assert y[0, 2, 2, 0] == 94.0
+    # edge (0,1): taps 4..9 over pixels 1..6 = 4+10+18+28+40+54 = 154
+    assert y[0, 0, 1, 0] == 154.0
+    # non-zero padding value 2 at the corner adds 2*(1+2+3+4+7) = 34
+    y2 = oracle.conv2d(x, w, padding_value=2.0)
+    assert y2[0, 0, 0, 0] == 94.0 + 34.0
+
+
+def test_conv_invariants(oracle):
+    x = RNG.standard_normal((2, 5, 6, 3))
+    # delta kernel at tap (0, 2) of channel c -> copy shifted by (pad + 0, pad + 2)
+    w = np.zeros((3, 3, 3, 3))
+    for k in range(3):
+        w[k, 0, 2, k] = 1.0
+    y = oracle.conv2d(x, w)
+    want = np.zeros_like(x)
+    want[:, 1:, :-1, :] = x[:, :-1, 1:, :]
+    np.testing.assert_array_equal(y, want)
+    # all-ones input and kernel: window population count
+    ones = oracle.conv2d(np.ones((1, 4, 4, 1)), np.ones((1, 3, 3, 1)))[0, :, :, 0]
+    np.testing.assert_array_equal(ones, np.array([[4, 6, 6, 4], [6, 9, 9, 6], [6, 9, 9, 6], [4, 6, 6, 4]], dtype=float))
+    # linearity in x and w
+    x2 = RNG.standard_normal(x.shape)
+    w1, w2 = RNG.standard_normal((4, 3, 3, 3)), RNG.standard_normal((4, 3, 3, 3))
+    a = oracle.conv2d(2.0 * x + x2, w1 - 3.0 * w2)
+    b = 2 * oracle.conv2d(x, w1) - 6 * oracle.conv2d(x, w2) + oracle.conv2d(x2, w1) - 3 * oracle.conv2d(x2, w2)
+    np.testing.assert_allclose(a, b, atol=1e-11)
+    # 1x1 == matmul
+    w11 = RNG.standard_normal((5, 1, 1, 3))
+    np.testing.assert_allclose(oracle.conv2d(x, w11, pad=(0, 0)), x @ w11[:, 0, 0, :].T, atol=1e-13)
+
+
+def test_conv_epilogue_order(oracle):
+    x = RNG.standard_normal((2, 4, 5, 3))
+    w = RNG.standard_normal((6, 3, 3, 3))
+    b = RNG.standard_normal(6)
+    z = RNG.standard_normal((2, 4, 5, 6))
+    y0 = RNG.standard_normal((2, 4, 5, 6))
+    conv = torch_conv(x, w, (-1, -1))
+    got = oracle.conv2d(x, w, b, z, y0, alpha1=1.1, alpha2=1.2, beta=0.1, activation=oracle.RELU)
+    want = np.maximum(1.1 * conv + 1.2 * z + b, 0.0) + 0.1 * y0
+    np.testing.assert_allclose(got, want, atol=1e-12)
+    got = oracle.conv2d(x, w, None, None, y0, alpha1=0.5, beta=0.0, activation=oracle.TANH)
+    np.testing.assert_allclose(got, np.tanh(0.5 * conv), atol=1e-12)
+
+
+def test_activations_against_numpy(oracle):
+    v = np.linspace(-4, 4, 41)
+    np.testing.assert_allclose(oracle.activation(oracle.SIGMOID, v), 1 / (1 + np.exp(-v)), atol=1e-15)
+    np.testing.assert_allclose(oracle.activation(oracle.TANH, v), np.tanh(v), atol=1e-15)
+    np.testing.assert_allclose(oracle.activation(oracle.RELU, v), np.maximum(v, 0))
+    np.testing.assert_allclose(oracle.activation(oracle.ELU, v), np.where(v >= 0, v, np.expm1(v)), atol=1e-15)
+    np.testing.assert_allclose(oracle.activation(oracle.SELU, v), 1.05070098 * np.where(v >= 0, v, 1.67326324 * np.expm1(v)), atol=1e-15)
+    np.testing.assert_allclose(oracle.activation(oracle.EXPONENTIAL, v), np.exp(v), rtol=1e-15)
+    np.testing.assert_allclose(oracle.activation(oracle.SOFTPLUS, v), np.log1p(np.exp(v)), atol=1e-15)
+    np.testing.assert_allclose(oracle.activation(oracle.SOFTSIGN, v), v / (1 + np.abs(v)), atol=1e-15)
+
+
+def test_int8_conv_is_exact(oracle):
+    x = RNG.integers(-127, 128, (2, 6, 7, 16), dtype=np.int8)
+    w = RNG.integers(-127, 128, (5, 3, 3, 16), dtype=np.int8)
+    b = RNG.integers(-2 ** 15, 2 ** 15, 5, dtype=np.int32)
+    got = oracle.conv2d_i8(x, w, b)
+    # independent integer route: zero-padded windows through an int64 einsum
+    xp = np.pad(x.astype(np.int64), ((0, 0), (1, 1), (1, 1), (0, 0)))
+    want = np.zeros((2, 6, 7, 5), dtype=np.int64)
+    for i in range(3):
+        for j in range(3):
+            want += np.einsum("nhwc,kc->nhwk", xp[:, i:i + 6, j:j + 7, :], w[:, i, j, :].astype(np.int64))
+    want += b
+    np.testing.assert_array_equal(got, want.astype(np.int32))
+    # and the fp64 routine is exact at these magnitudes
+    f = oracle.conv2d(x.astype(np.float64), w.astype(np.float64), b.astype(np.float64))
+    np.testing.assert_array_equal(f, want.astype(np.float64))
+    relu = oracle.conv2d_i8(x, w, b, activation=oracle.RELU)
+    np.testing.assert_array_equal(relu, np.maximum(want, 0).astype(np.int32))
+    # 1x1 and stride 2
+    w1 = RNG.integers(-127, 128, (5, 1, 1, 16), dtype=np.int8)
+    np.testing.assert_array_equal(oracle.conv2d_i8(x, w1, None, pad=(0, 0)), np.einsum("nhwc,kc->nhwk", x.astype(np.int64), w1[:, 0, 0].astype(np.int64)))
+    s2 = oracle.conv2d_i8(x, w, b, stride=(2, 2))
+    np.testing.assert_array_equal(s2, want[:, ::2, ::2, :].astype(np.int32))
+
+
+def test_requant_definition(oracle):
+    acc = RNG.integers(-2 ** 22, 2 ** 22, (50, 8)).astype(np.int32)
+    acc[0, :] = [0, 1, -1, 2 ** 30, -2 ** 30, 500, 1500, -1500]
+    scale = RNG.uniform(1e-4, 1e-3, 8).astype(np.float32)
+    scale[5:8] = 1e-3  # 500*1e-3 = 0.5 -> 0 (ties to even); 1.5 -> 2; -1.5 -> -2
+    q = oracle.requant_i8(acc, scale)
+    want = np.clip(np.rint(acc.astype(np.float32) * scale), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(q, want)
+    assert q[0, 3] == 127 and q[0, 4] == -128
+    assert q[0, 5] == 0 and q[0, 6] == 2 and q[0, 7] == -2
+
+
+@pytest.mark.parametrize("m,r", [(2, 3), (4, 3), (2, 5)])
+def test_winograd_tables_reproduce_correlation(oracle, m, r):
+    """A^T[(G g G^T) .* (B^T d B)]A equals the direct correlation of a t x t patch with an r x r kernel."""
+    G, BT, AT = (oracle.winograd_table(m, r, i) for i in range(3))
+    t = m + r - 1
+    d = RNG.standard_normal((t, t))
+    g = RNG.standard_normal((r, r))
+    y = AT @ ((G @ g @ G.T) * (BT @ d @ BT.T)) @ AT.T
+    want = np.array([[np.sum(d[a:a + r, b:b + r] * g) for b in range(m)] for a in range(m)])
+    np.testing.assert_allclose(y, want, atol=1e-12)
+
+
+@pytest.mark.parametrize("m,r,pad", [(2, 3, (-1, -1)), (4, 3, (-1, -1)), (2, 5, (-2, -2)), (4, 3, (0, -2))])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_winograd_pipeline_equals_direct(oracle, m, r, pad, mode):
+    """weight transform -> input transform -> batched GEMM -> output transform == direct convolution,
+    on odd sizes (partial tiles), with bias, residual, activation and beta."""
+    N, H, W, Cin, K = 2, 7, 9, 5, 3
+    x = RNG.standard_normal((N, H, W, Cin))
+    w = RNG.standard_normal((K, r, r, Cin))
+    b = RNG.standard_normal(K)
+    U = oracle.winograd_weight_transform(w, m, invert=(mode == 1))
+    V = oracle.winograd_input_transform(x, m, r, pad)
+    Mx = oracle.gemm_batched(V, U, opA=False, opB=True)
+    if pad == (-(r // 2), -(r // 2)):
+        z = RNG.standard_normal((N, H, W, K))
+        y0 = RNG.standard_normal((N, H, W, K))
+        got = oracle.winograd_output_transform(Mx, (N, H, W, K), m, r, b, z, y0, 1.1, 1.2, 0.1, oracle.RELU)
+        want = oracle.conv2d(x, w, b, z, y0, pad=pad, mode=mode, alpha1=1.1, alpha2=1.2, beta=0.1, activation=oracle.RELU)
+        np.testing.assert_allclose(got, want, atol=1e-11)
+    else:
+        # asymmetric offsets: the tile grid of the output transform still covers H x W outputs, the direct
+        # convolution with the same offsets is defined wherever the window start is (out_shape forces H x W)
+        got = oracle.winograd_output_transform(Mx, (N, H, W, K), m, r)
+        want = oracle.conv2d(x, w, pad=pad, mode=mode, out_shape=(H, W))
+        np.testing.assert_allclose(got, want, atol=1e-11)
+
+
+def test_winograd_layouts(oracle):
+    """[t*t, tiles, C] layout, tile index (n*Th + th)*Tw + tw, padding value substitution."""
+    m, r = 2, 3
+    x = RNG.standard_normal((2, 3, 5, 2))
+    V = oracle.winograd_input_transform(x, m, r, (-1, -1), padding_value=0.5)
+    BT = oracle.winograd_table(m, r, 1)
+    Th, Tw = 2, 3
+    assert V.shape == (16, 2 * Th * Tw, 2)
+    n, th, tw, c = 1, 1, 2, 1
+    d = np.full((4, 4), 0.5)
+    for a in range(4):
+        for b in range(4):
+            ih, iw = -1 + th * 2 + a, -1 + tw * 2 + b
+            if 0 <= ih < 3 and 0 <= iw < 5:
+                d[a, b] = x[n, ih, iw, c]
+    want = BT @ d @ BT.T
+    np.testing.assert_allclose(V[:, (n * Th + th) * Tw + tw, c].reshape(4, 4), want, atol=1e-13)
+    w = RNG.standard_normal((3, 3, 3, 2))
+    U = oracle.winograd_weight_transform(w, m)
+    G = oracle.winograd_table(m, r, 0)
+    np.testing.assert_allclose(U[:, 2, 1].reshape(4, 4), G @ w[2, :, :, 1] @ G.T, atol=1e-13)
+    Ui = oracle.winograd_weight_transform(w, m, invert=True)
+    np.testing.assert_allclose(Ui[:, 2, 1].reshape(4, 4), G @ w[2, ::-1, ::-1, 1] @ G.T, atol=1e-13)
+
+
+@pytest.mark.parametrize("opA", [False, True])
+@pytest.mark.parametrize("opB", [False, True])
+def test_gemm_batched_matches_numpy(oracle, opA, opB):
+    b, M, N, K = 3, 23, 45, 67
+    A = RNG.standard_normal((b, K, M) if opA else (b, M, K))
+    B = RNG.standard_normal((b, N, K) if opB else (b, K, N))
+    C0 = RNG.standard_normal((b, M, N))
+    got = oracle.gemm_batched(A, B, C0, opA, opB, 1.1, 0.1)
+    a = A.transpose(0, 2, 1) if opA else A
+    bb = B.transpose(0, 2, 1) if opB else B
+    np.testing.assert_allclose(got, 1.1 * np.matmul(a, bb) + 0.1 * C0, atol=1e-12)
+
+
+def test_add_bias_formula(oracle):
+    x = RNG.standard_normal((23, 45, 67))
+    z = RNG.standard_normal(x.shape)
+    y0 = RNG.standard_normal(x.shape)
+    b = RNG.standard_normal(67)
+    a1, a2, b1, b2, b3 = 1.1, 1.2, 0.1, 0.2, 0.3
+    got = oracle.add_bias(x, b, z, y0, a1, a2, b1, b2, b3, oracle.SIGMOID)
+    want = a1 / (1 + np.exp(-(a2 * x + b + b1 * z))) + b2 * z + b3 * y0
+    np.testing.assert_allclose(got, want, atol=1e-13)
+    got = oracle.add_bias(x, b, None, None, a1, a2, activation=oracle.RELU)
+    np.testing.assert_allclose(got, a1 * np.maximum(a2 * x + b, 0), atol=1e-13)
+
+
+@pytest.mark.parametrize("R,pad,mode", [(3, (-1, -1), 0), (5, (-2, -2), 0), (3, (-1, -1), 1)])
+def test_im2row_times_weights_is_conv(oracle, R, pad, mode):
+    x = RNG.standard_normal((2, 6, 7, 4))
+    w = RNG.standard_normal((3, R, R, 4))
+    rows = oracle.im2row(x, R, R, pad, mode)
+    got = (rows @ w.reshape(3, -1).T).reshape(2, 6, 7, 3)
+    np.testing.assert_allclose(got, oracle.conv2d(x, w, pad=pad, mode=mode), atol=1e-12)
+
+
+def test_bf16_rounding_helpers(oracle):
+    v = np.array([1.0, 1.00390625, 1.01171875, -3.0e38, 1e-40, np.inf], dtype=np.float32)
+    bits = oracle.f32_to_bf16_bits(v)
+    back = oracle.bf16_bits_to_f32(bits)
+    # 1.00390625 = 1 + 2^-8 is a tie between 1.0 and 1.0078125 -> even mantissa (1.0)
+    assert back[0] == 1.0 and back[1] == 1.0
+    # 1.01171875 = 1 + 3*2^-8 is a tie between 1.0078125 (odd) and 1.015625 (even)
+    assert back[2] == np.float32(1.015625)
+    t = torch.tensor(v).to(torch.bfloat16).to(torch.float32).numpy()
+    np.testing.assert_array_equal(back, t)
+    big = RNG.standard_normal(10000).astype(np.float32)
+    np.testing.assert_array_equal(oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(big)), torch.tensor(big).to(torch.bfloat16).to(torch.float32).numpy())
