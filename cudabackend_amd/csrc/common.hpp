@@ -1,0 +1,200 @@
+/*
+ * common.hpp -- device-side building blocks shared by every kernel file: storage types with
+ * round-to-nearest-even conversion, bounds-aware vector access, activations.
+ *
+ * Behaviour carried over from the reference's Number<T> abstraction (the .cuh files under src/numbers): 16-bit tensors are
+ * computed in fp32, loads and stores near the end of the channel dimension touch only the elements that exist.
+ * Deliberate difference: bf16 stores round to nearest even (the reference truncates, src/numbers/bf16_number.cuh:40-43).
+ */
+#ifndef AVHIP_COMMON_HPP_
+#define AVHIP_COMMON_HPP_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/avocado_hip_kernels.h"
+
+namespace avhip
+{
+	enum DType
+	{
+		DT_UNKNOWN = 0, DT_UINT8, DT_INT8, DT_INT16, DT_INT32, DT_INT64, DT_FLOAT16, DT_BFLOAT16, DT_FLOAT32, DT_FLOAT64, DT_COMPLEX32, DT_COMPLEX64
+	};
+	enum Activation
+	{
+		ACT_LINEAR = 0, ACT_SIGMOID, ACT_TANH, ACT_RELU, ACT_SELU, ACT_ELU, ACT_EXPONENTIAL, ACT_SOFTPLUS, ACT_SOFTSIGN
+	};
+
+	struct bf16_t
+	{
+		uint16_t bits;
+	};
+	typedef _Float16 f16_t;
+
+	__host__ __device__ inline float bf16_to_float(bf16_t v)
+	{
+		union
+		{
+			uint32_t u;
+			float f;
+		} c;
+		c.u = static_cast<uint32_t>(v.bits) << 16;
+		return c.f;
+	}
+	__host__ __device__ inline bf16_t float_to_bf16(float f)
+	{
+		union
+		{
+			uint32_t u;
+			float f;
+		} c;
+		c.f = f;
+		bf16_t r;
+		if ((c.u & 0x7FFFFFFFu) > 0x7F800000u) // NaN stays NaN
+			r.bits = static_cast<uint16_t>((c.u >> 16) | 0x0040u);
+		else
+			r.bits = static_cast<uint16_t>((c.u + 0x7FFFu + ((c.u >> 16) & 1u)) >> 16);
+		return r;
+	}
+
+	/* Storage type -> compute type and conversions. */
+	template<typename T> struct Traits;
+	template<> struct Traits<float>
+	{
+		typedef float compute;
+		static constexpr int dtype = DT_FLOAT32;
+		__host__ __device__ static float load(float v) { return v; }
+		__host__ __device__ static float store(float v) { return v; }
+	};
+	template<> struct Traits<double>
+	{
+		typedef double compute;
+		static constexpr int dtype = DT_FLOAT64;
+		__host__ __device__ static double load(double v) { return v; }
+		__host__ __device__ static double store(double v) { return v; }
+	};
+	template<> struct Traits<f16_t>
+	{
+		typedef float compute;
+		static constexpr int dtype = DT_FLOAT16;
+		__host__ __device__ static float load(f16_t v) { return static_cast<float>(v); }
+		__host__ __device__ static f16_t store(float v) { return static_cast<f16_t>(v); }
+	};
+	template<> struct Traits<bf16_t>
+	{
+		typedef float compute;
+		static constexpr int dtype = DT_BFLOAT16;
+		__host__ __device__ static float load(bf16_t v) { return bf16_to_float(v); }
+		__host__ __device__ static bf16_t store(float v) { return float_to_bf16(v); }
+	};
+
+	/* A naturally aligned pack of V elements of T moved with one memory instruction. */
+	template<typename T, int V>
+	struct alignas(sizeof(T) * V) Pack
+	{
+		T v[V];
+	};
+
+	/* Loads V consecutive elements starting at ptr into compute values; elements at or beyond `valid` are not touched
+	 * and read as zero.  With allow_vector the pointer must be aligned to the pack whenever valid >= V. */
+	template<typename T, int V, typename CT>
+	__device__ inline void load_vec(const T *ptr, int valid, CT (&out)[V], bool allow_vector = true)
+	{
+		if (V > 1 && valid >= V && allow_vector)
+		{
+			const Pack<T, V> p = *reinterpret_cast<const Pack<T, V>*>(ptr);
+#pragma unroll
+			for (int i = 0; i < V; i++)
+				out[i] = Traits<T>::load(p.v[i]);
+		}
+		else
+		{
+#pragma unroll
+			for (int i = 0; i < V; i++)
+				out[i] = (i < valid) ? static_cast<CT>(Traits<T>::load(ptr[i])) : static_cast<CT>(0);
+		}
+	}
+	template<typename T, int V, typename CT>
+	__device__ inline void store_vec(T *ptr, int valid, const CT (&in)[V], bool allow_vector = true)
+	{
+		if (V > 1 && valid >= V && allow_vector)
+		{
+			Pack<T, V> p;
+#pragma unroll
+			for (int i = 0; i < V; i++)
+				p.v[i] = Traits<T>::store(in[i]);
+			*reinterpret_cast<Pack<T, V>*>(ptr) = p;
+		}
+		else
+		{
+#pragma unroll
+			for (int i = 0; i < V; i++)
+				if (i < valid)
+					ptr[i] = Traits<T>::store(in[i]);
+		}
+	}
+
+	/* Forward activations, src/activations.cuh:202-425 of the reference. */
+	template<typename CT>
+	__device__ inline CT activation_forward(int act, CT x)
+	{
+		switch (act)
+		{
+			default:
+			case ACT_LINEAR:
+				return x;
+			case ACT_SIGMOID:
+				return static_cast<CT>(1) / (static_cast<CT>(1) + exp(-x));
+			case ACT_TANH:
+				return tanh(x);
+			case ACT_RELU:
+				return x > static_cast<CT>(0) ? x : static_cast<CT>(0);
+			case ACT_SELU:
+				return static_cast<CT>(1.05070098) * (x >= static_cast<CT>(0) ? x : static_cast<CT>(1.67326324) * expm1(x));
+			case ACT_ELU:
+				return x >= static_cast<CT>(0) ? x : expm1(x);
+			case ACT_EXPONENTIAL:
+				return exp(x);
+			case ACT_SOFTPLUS:
+				return log1p(exp(x));
+			case ACT_SOFTSIGN:
+				return x / (fabs(x) + static_cast<CT>(1));
+		}
+	}
+
+	__host__ inline int dtype_size(int dtype)
+	{
+		switch (dtype)
+		{
+			case DT_UINT8:
+			case DT_INT8:
+				return 1;
+			case DT_INT16:
+			case DT_FLOAT16:
+			case DT_BFLOAT16:
+				return 2;
+			case DT_INT32:
+			case DT_FLOAT32:
+				return 4;
+			case DT_INT64:
+			case DT_FLOAT64:
+			case DT_COMPLEX32:
+				return 8;
+			case DT_COMPLEX64:
+				return 16;
+			default:
+				return 0;
+		}
+	}
+
+	__host__ inline unsigned int ceil_div(int64_t a, int64_t b)
+	{
+		return static_cast<unsigned int>((a + b - 1) / b);
+	}
+	__host__ inline bool aligned_to(const void *p, size_t bytes)
+	{
+		return (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
+	}
+}
+
+#endif /* AVHIP_COMMON_HPP_ */

@@ -1,0 +1,307 @@
+/*
+ * elementwise.hip -- the bandwidth-bound helpers around the convolution path: bias + activation, explicit im2row,
+ * element type conversion, pattern fill.
+ *
+ * Replaces kernel_add_bias (src/tensor_op.cu:199-228), kernel_im2row_conv2d (src/im2row.cu:29-66), kernel_convert
+ * (src/conversions.cu:253-258) and kernel_setall (src/descriptors.cu:22-39) of the reference.  One work-item moves one
+ * 16-byte (or 8-byte) vector; grids are sized to the data, not capped, so a launch always fills 256 CUs.
+ */
+#include <cstring>
+
+#include "common.hpp"
+
+namespace
+{
+	using namespace avhip;
+
+	template<typename T, int V>
+	__global__ __launch_bounds__(256) void k_add_bias(const T *__restrict__ x, const typename Traits<T>::compute *__restrict__ b, const T *z, T *y,
+			int64_t first, int last, typename Traits<T>::compute alpha1, typename Traits<T>::compute alpha2, typename Traits<T>::compute beta1,
+			typename Traits<T>::compute beta2, typename Traits<T>::compute beta3, int activation)
+	{
+		typedef typename Traits<T>::compute CT;
+		const int LV = (last + V - 1) / V;
+		const int64_t gid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+		const int64_t row = gid / LV;
+		if (row >= first)
+			return;
+		const int j = static_cast<int>(gid - row * LV) * V;
+		const int valid = last - j;
+		const int64_t idx = row * last + j;
+
+		CT xv[V], t[V];
+		load_vec<T, V, CT>(x + idx, valid, xv);
+#pragma unroll
+		for (int v = 0; v < V; v++)
+			t[v] = alpha2 * xv[v] + ((v < valid) ? b[j + v] : static_cast<CT>(0));
+		if (beta1 != static_cast<CT>(0) || beta2 != static_cast<CT>(0))
+		{
+			CT zv[V];
+			load_vec<T, V, CT>(z + idx, valid, zv);
+#pragma unroll
+			for (int v = 0; v < V; v++)
+				t[v] = alpha1 * activation_forward<CT>(activation, t[v] + beta1 * zv[v]) + beta2 * zv[v];
+		}
+		else
+		{
+#pragma unroll
+			for (int v = 0; v < V; v++)
+				t[v] = alpha1 * activation_forward<CT>(activation, t[v]);
+		}
+		if (beta3 != static_cast<CT>(0))
+		{
+			CT yv[V];
+			load_vec<T, V, CT>(y + idx, valid, yv);
+#pragma unroll
+			for (int v = 0; v < V; v++)
+				t[v] += beta3 * yv[v];
+		}
+		store_vec<T, V, CT>(y + idx, valid, t);
+	}
+
+	template<typename T>
+	int launch_add_bias(hipStream_t s, const void *x, const void *b, const void *z, void *y, int64_t first, int last, double alpha1, double alpha2,
+			double beta1, double beta2, double beta3, int activation)
+	{
+		typedef typename Traits<T>::compute CT;
+		constexpr int V = 16 / sizeof(T) > 4 ? 4 : 16 / sizeof(T);
+		const bool vec = last % V == 0 && aligned_to(x, V * sizeof(T)) && aligned_to(y, V * sizeof(T)) && (z == nullptr || aligned_to(z, V * sizeof(T)));
+		const int v = vec ? V : 1;
+		const int64_t items = first * ((last + v - 1) / v);
+		const dim3 grid(ceil_div(items, 256));
+#define ARGS static_cast<const T*>(x), static_cast<const CT*>(b), static_cast<const T*>(z), static_cast<T*>(y), first, last, static_cast<CT>(alpha1), \
+		static_cast<CT>(alpha2), static_cast<CT>(beta1), static_cast<CT>(beta2), static_cast<CT>(beta3), activation
+		if (vec)
+			hipLaunchKernelGGL((k_add_bias<T, V>), grid, dim3(256), 0, s, ARGS);
+		else
+			hipLaunchKernelGGL((k_add_bias<T, 1>), grid, dim3(256), 0, s, ARGS);
+#undef ARGS
+		return 0;
+	}
+
+	/* rows[pixel, (i*S + j)*C + c] = x[n, pad_h + oh + i', pad_w + ow + j', c]; one work-item per element of `rows`. */
+	template<typename E>
+	__global__ __launch_bounds__(256) void k_im2row(const E *__restrict__ x, E *__restrict__ rows, avhipConvShape s, E padv, int64_t total)
+	{
+		const int64_t gid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+		if (gid >= total)
+			return;
+		int64_t t = gid;
+		const int c = static_cast<int>(t % s.C);
+		t /= s.C;
+		const int j = static_cast<int>(t % s.S);
+		t /= s.S;
+		const int i = static_cast<int>(t % s.R);
+		t /= s.R;
+		const int ow = static_cast<int>(t % s.Wo);
+		t /= s.Wo;
+		const int oh = static_cast<int>(t % s.Ho);
+		const int64_t n = t / s.Ho;
+		const int ii = s.mode ? (s.R - 1 - i) : i;
+		const int jj = s.mode ? (s.S - 1 - j) : j;
+		const int ih = s.pad_h + oh + ii;
+		const int iw = s.pad_w + ow + jj;
+		E v = padv;
+		if (ih >= 0 && ih < s.H && iw >= 0 && iw < s.W)
+			v = x[((n * s.H + ih) * s.W + iw) * s.C + c];
+		rows[gid] = v;
+	}
+	template<typename E>
+	int launch_im2row(hipStream_t st, const avhipConvShape &s, const void *x, void *rows, const void *padding_value)
+	{
+		E padv;
+		if (padding_value != nullptr)
+			std::memcpy(&padv, padding_value, sizeof(E));
+		else
+			std::memset(&padv, 0, sizeof(E));
+		const int64_t total = static_cast<int64_t>(s.N) * s.Ho * s.Wo * s.R * s.S * s.C;
+		hipLaunchKernelGGL((k_im2row<E>), dim3(ceil_div(total, 256)), dim3(256), 0, st, static_cast<const E*>(x), static_cast<E*>(rows), s, padv, total);
+		return 0;
+	}
+
+	/* Conversions go through double (exact for every supported source type); integers round to nearest even and saturate. */
+	template<typename T> __device__ inline double to_double(T v) { return static_cast<double>(v); }
+	template<> __device__ inline double to_double<bf16_t>(bf16_t v) { return static_cast<double>(bf16_to_float(v)); }
+	template<> __device__ inline double to_double<f16_t>(f16_t v) { return static_cast<double>(static_cast<float>(v)); }
+
+	template<typename T> struct FromDouble
+	{
+		__device__ static inline T run(double v, double lo, double hi)
+		{
+			if (!(v == v))
+				return static_cast<T>(0);
+			double r = rint(v);
+			r = r < lo ? lo : r;
+			r = r > hi ? hi : r;
+			return static_cast<T>(r);
+		}
+	};
+	template<> struct FromDouble<float>
+	{
+		__device__ static inline float run(double v, double, double) { return static_cast<float>(v); }
+	};
+	template<> struct FromDouble<double>
+	{
+		__device__ static inline double run(double v, double, double) { return v; }
+	};
+	template<> struct FromDouble<f16_t>
+	{
+		__device__ static inline f16_t run(double v, double, double) { return static_cast<f16_t>(v); }
+	};
+	template<> struct FromDouble<bf16_t>
+	{
+		/* double -> float -> bf16 would round twice; float inputs (the only practical source) are exact in double and the
+		 * first step is then the identity. */
+		__device__ static inline bf16_t run(double v, double, double) { return float_to_bf16(static_cast<float>(v)); }
+	};
+
+	template<typename D, typename S>
+	__global__ __launch_bounds__(256) void k_convert(D *__restrict__ dst, const S *__restrict__ src, int64_t elements, double lo, double hi)
+	{
+		const int64_t gid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+		if (gid < elements)
+			dst[gid] = FromDouble<D>::run(to_double<S>(src[gid]), lo, hi);
+	}
+	template<typename D>
+	int convert_from(hipStream_t s, void *dst, const void *src, int src_dtype, int64_t n, double lo, double hi)
+	{
+		const dim3 grid(ceil_div(n, 256));
+#define CASE(DT, S) case DT: hipLaunchKernelGGL((k_convert<D, S>), grid, dim3(256), 0, s, static_cast<D*>(dst), static_cast<const S*>(src), n, lo, hi); return 0;
+		switch (src_dtype)
+		{
+			CASE(DT_UINT8, uint8_t)
+			CASE(DT_INT8, int8_t)
+			CASE(DT_INT16, int16_t)
+			CASE(DT_INT32, int32_t)
+			CASE(DT_FLOAT16, f16_t)
+			CASE(DT_BFLOAT16, bf16_t)
+			CASE(DT_FLOAT32, float)
+			CASE(DT_FLOAT64, double)
+			default:
+				return AVHIP_UNSUPPORTED_DATATYPE;
+		}
+#undef CASE
+	}
+
+	template<typename E>
+	__global__ __launch_bounds__(256) void k_fill(E *dst, int64_t count, E value)
+	{
+		const int64_t gid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+		if (gid < count)
+			dst[gid] = value;
+	}
+	template<typename E>
+	int launch_fill(hipStream_t s, void *dst, int64_t bytes, const void *pattern)
+	{
+		E v;
+		std::memcpy(&v, pattern, sizeof(E));
+		const int64_t count = bytes / static_cast<int64_t>(sizeof(E));
+		if (count > 0)
+			hipLaunchKernelGGL((k_fill<E>), dim3(ceil_div(count, 256)), dim3(256), 0, s, static_cast<E*>(dst), count, v);
+		return 0;
+	}
+}
+
+extern "C"
+{
+	int avhip_add_bias(void *stream, int dtype, const void *x, const void *b, const void *z, void *y, int64_t first, int last, double alpha1,
+			double alpha2, double beta1, double beta2, double beta3, int activation)
+	{
+		if (x == nullptr || b == nullptr || y == nullptr || first <= 0 || last <= 0)
+			return AVHIP_BAD_PARAM;
+		if ((beta1 != 0.0 || beta2 != 0.0) && z == nullptr)
+			return AVHIP_BAD_PARAM;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+		switch (dtype)
+		{
+			case DT_FLOAT16:
+				return launch_add_bias<f16_t>(s, x, b, z, y, first, last, alpha1, alpha2, beta1, beta2, beta3, activation);
+			case DT_BFLOAT16:
+				return launch_add_bias<bf16_t>(s, x, b, z, y, first, last, alpha1, alpha2, beta1, beta2, beta3, activation);
+			case DT_FLOAT32:
+				return launch_add_bias<float>(s, x, b, z, y, first, last, alpha1, alpha2, beta1, beta2, beta3, activation);
+			case DT_FLOAT64:
+				return launch_add_bias<double>(s, x, b, z, y, first, last, alpha1, alpha2, beta1, beta2, beta3, activation);
+			default:
+				return AVHIP_UNSUPPORTED_DATATYPE;
+		}
+	}
+
+	int avhip_im2row(void *stream, int elem_size, const avhipConvShape *shape, const void *x, void *rows, const void *padding_value)
+	{
+		if (shape == nullptr || x == nullptr || rows == nullptr)
+			return AVHIP_BAD_PARAM;
+		if (shape->stride_h != 1 || shape->stride_w != 1 || shape->dil_h != 1 || shape->dil_w != 1)
+			return AVHIP_NOT_SUPPORTED;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+		switch (elem_size)
+		{
+			case 1:
+				return launch_im2row<uint8_t>(s, *shape, x, rows, padding_value);
+			case 2:
+				return launch_im2row<uint16_t>(s, *shape, x, rows, padding_value);
+			case 4:
+				return launch_im2row<uint32_t>(s, *shape, x, rows, padding_value);
+			case 8:
+				return launch_im2row<uint2>(s, *shape, x, rows, padding_value);
+			case 16:
+				return launch_im2row<uint4>(s, *shape, x, rows, padding_value);
+			default:
+				return AVHIP_UNSUPPORTED_DATATYPE;
+		}
+	}
+
+	int avhip_change_type(void *stream, void *dst, int dst_dtype, const void *src, int src_dtype, int64_t elements)
+	{
+		if (dst == nullptr || src == nullptr || elements < 0)
+			return AVHIP_BAD_PARAM;
+		if (elements == 0)
+			return 0;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+		switch (dst_dtype)
+		{
+			case DT_UINT8:
+				return convert_from<uint8_t>(s, dst, src, src_dtype, elements, 0.0, 255.0);
+			case DT_INT8:
+				return convert_from<int8_t>(s, dst, src, src_dtype, elements, -128.0, 127.0);
+			case DT_INT16:
+				return convert_from<int16_t>(s, dst, src, src_dtype, elements, -32768.0, 32767.0);
+			case DT_INT32:
+				return convert_from<int32_t>(s, dst, src, src_dtype, elements, -2147483648.0, 2147483647.0);
+			case DT_FLOAT16:
+				return convert_from<f16_t>(s, dst, src, src_dtype, elements, 0.0, 0.0);
+			case DT_BFLOAT16:
+				return convert_from<bf16_t>(s, dst, src, src_dtype, elements, 0.0, 0.0);
+			case DT_FLOAT32:
+				return convert_from<float>(s, dst, src, src_dtype, elements, 0.0, 0.0);
+			case DT_FLOAT64:
+				return convert_from<double>(s, dst, src, src_dtype, elements, 0.0, 0.0);
+			default:
+				return AVHIP_UNSUPPORTED_DATATYPE;
+		}
+	}
+
+	int avhip_set_memory(void *stream, void *dst, int64_t bytes, const void *pattern, int pattern_size)
+	{
+		if (dst == nullptr || pattern == nullptr || bytes < 0 || pattern_size <= 0 || bytes % pattern_size != 0)
+			return AVHIP_BAD_PARAM;
+		if (!aligned_to(dst, pattern_size))
+			return AVHIP_BAD_PARAM;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+		switch (pattern_size)
+		{
+			case 1:
+				return launch_fill<uint8_t>(s, dst, bytes, pattern);
+			case 2:
+				return launch_fill<uint16_t>(s, dst, bytes, pattern);
+			case 4:
+				return launch_fill<uint32_t>(s, dst, bytes, pattern);
+			case 8:
+				return launch_fill<uint2>(s, dst, bytes, pattern);
+			case 16:
+				return launch_fill<uint4>(s, dst, bytes, pattern);
+			default:
+				return AVHIP_BAD_PARAM;
+		}
+	}
+}

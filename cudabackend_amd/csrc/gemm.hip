@@ -1,0 +1,222 @@
+/*
+ * gemm.hip -- C[b] = alpha * op(A[b]) op(B[b]) + beta * C[b] for row-major operands.
+ *
+ * Replaces the cuBLAS calls behind cudaGemm / cudaGemmBatched of the reference (src/gemm.cpp:25-209).  The batched
+ * (N, T) form  M[b] = V[b] * U[b]^T  is the matrix-core stage of non-fused Winograd (app/CudaBackend.cu:417-418): both
+ * operands are contiguous along k, so it runs on the shared MFMA engine with fp32 (int32 for int8) accumulation and the
+ * result is rounded once, to nearest even, on store.  Every other operand form, and fp64, goes through a small LDS-tiled
+ * kernel that exists for completeness of the API, not for speed.
+ * Unlike the reference there is a bf16 case, fp16 always accumulates in fp32, and the result of a 16-bit product may be
+ * kept in fp32.
+ */
+#include "mfma_core.hpp"
+
+namespace
+{
+	using namespace avhip;
+
+	template<typename TE>
+	struct RowLoader
+	{
+		const TE *base;
+		int rows, K, ld, row0;
+		bool vec_ok;
+		__device__ inline uint4 operator()(int step, int q, int part) const
+		{
+			constexpr int E = 16 / sizeof(TE);
+			constexpr int KE = STEP_BYTES / sizeof(TE);
+			const int row = row0 + (threadIdx.x >> 2) + 64 * q;
+			const int k = step * KE + part * E;
+			if (row >= rows)
+				return make_uint4(0u, 0u, 0u, 0u);
+			return fetch_chunk<TE>(base + static_cast<size_t>(row) * ld + k, K - k, vec_ok);
+		}
+	};
+
+	/* Writes alpha * acc + beta * C for 4 consecutive columns (fewer at the right edge of the matrix). */
+	template<typename TC>
+	__device__ inline void store_c(TC *p, int valid, bool vec, const float (&acc)[4], float alpha, float beta)
+	{
+		float v[4];
+#pragma unroll
+		for (int q = 0; q < 4; q++)
+			v[q] = alpha * acc[q];
+		if (beta != 0.0f)
+		{
+			float old[4];
+			load_vec<TC, 4, float>(p, valid, old, vec);
+#pragma unroll
+			for (int q = 0; q < 4; q++)
+				v[q] += beta * old[q];
+		}
+		store_vec<TC, 4, float>(p, valid, v, vec);
+	}
+	__device__ inline void store_c(int *p, int valid, bool vec, const int (&acc)[4], int alpha, int beta)
+	{
+		int v[4];
+#pragma unroll
+		for (int q = 0; q < 4; q++)
+		{
+			v[q] = alpha * acc[q];
+			if (beta != 0 && q < valid)
+				v[q] += beta * p[q];
+		}
+		if (vec && valid >= 4)
+			*reinterpret_cast<int4*>(p) = make_int4(v[0], v[1], v[2], v[3]);
+		else
+		{
+#pragma unroll
+			for (int q = 0; q < 4; q++)
+				if (q < valid)
+					p[q] = v[q];
+		}
+	}
+
+	template<typename TE, typename TC>
+	__global__ __launch_bounds__(256) void k_gemm_nt_mfma(const TE *__restrict__ A, const TE *__restrict__ B, TC *C, int M, int N, int K, int lda, int ldb,
+			int ldc, int64_t strideA, int64_t strideB, int64_t strideC, typename Mma<TE>::scalar_t alpha, typename Mma<TE>::scalar_t beta, int vec_ok)
+	{
+		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
+		constexpr int KE = STEP_BYTES / sizeof(TE);
+		const int batch = blockIdx.z;
+		const int m0 = blockIdx.x * BLOCK_M;
+		const int n0 = blockIdx.y * BLOCK_N;
+
+		RowLoader<TE> la { A + batch * strideA, M, K, lda, m0, (vec_ok & 1) != 0 };
+		RowLoader<TE> lb { B + batch * strideB, N, K, ldb, n0, (vec_ok & 1) != 0 };
+		typename Mma<TE>::acc_t acc[2][2];
+		block_mma<TE>(lds, (K + KE - 1) / KE, la, lb, acc);
+
+		TC *c = C + batch * strideC;
+		const bool vec_c = (vec_ok & 2) != 0;
+		drain_tile<TE>(lds, acc, [&](int r, int col, const typename Mma<TE>::scalar_t (&v)[4])
+		{
+			const int row = m0 + r;
+			const int cc = n0 + col;
+			if (row < M && cc < N)
+				store_c(c + static_cast<size_t>(row) * ldc + cc, N - cc, vec_c, v, alpha, beta);
+		});
+	}
+
+	/* Any operand form, any supported type: 16 x 16 outputs per workgroup, k in slices of 16 through LDS. */
+	template<typename TA, typename TC, typename CT>
+	__global__ __launch_bounds__(256) void k_gemm_generic(const TA *__restrict__ A, const TA *__restrict__ B, TC *C, int M, int N, int K, int opA, int opB,
+			int lda, int ldb, int ldc, int64_t strideA, int64_t strideB, int64_t strideC, CT alpha, CT beta)
+	{
+		__shared__ CT sa[16][17];
+		__shared__ CT sb[16][17];
+		const int batch = blockIdx.z;
+		const TA *a = A + batch * strideA;
+		const TA *b = B + batch * strideB;
+		const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+		const int row = blockIdx.y * 16 + ty;
+		const int col = blockIdx.x * 16 + tx;
+		CT acc = 0;
+		for (int k0 = 0; k0 < K; k0 += 16)
+		{
+			{ // sa[ty][tx] = opA(A)[row0 + ty][k0 + tx]
+				const int r = blockIdx.y * 16 + ty, k = k0 + tx;
+				CT v = 0;
+				if (r < M && k < K)
+					v = static_cast<CT>(opA ? a[static_cast<size_t>(k) * lda + r] : a[static_cast<size_t>(r) * lda + k]);
+				sa[ty][tx] = v;
+			}
+			{ // sb[ty][tx] = opB(B)[k0 + ty][col0 + tx]
+				const int k = k0 + ty, cidx = blockIdx.x * 16 + tx;
+				CT v = 0;
+				if (k < K && cidx < N)
+					v = static_cast<CT>(opB ? b[static_cast<size_t>(cidx) * ldb + k] : b[static_cast<size_t>(k) * ldb + cidx]);
+				sb[ty][tx] = v;
+			}
+			__syncthreads();
+#pragma unroll
+			for (int k = 0; k < 16; k++)
+				acc += sa[ty][k] * sb[k][tx];
+			__syncthreads();
+		}
+		if (row < M && col < N)
+		{
+			TC *p = C + batch * strideC + static_cast<size_t>(row) * ldc + col;
+			CT v = alpha * acc;
+			if (beta != static_cast<CT>(0))
+				v += beta * static_cast<CT>(*p);
+			*p = static_cast<TC>(v);
+		}
+	}
+
+	/* Thin value wrappers so that the generic kernel can static_cast 16-bit storage types. */
+	struct bf16_val
+	{
+		bf16_t raw;
+		__device__ operator float() const { return bf16_to_float(raw); }
+		__device__ bf16_val() = default;
+		__device__ bf16_val(float f) : raw(float_to_bf16(f)) {}
+	};
+
+	template<typename TE, typename TC>
+	int launch_mfma(hipStream_t s, const void *A, const void *B, void *C, int batch, int M, int N, int K, int lda, int ldb, int ldc, int64_t sA, int64_t sB,
+			int64_t sC, double alpha, double beta)
+	{
+		typedef typename Mma<TE>::scalar_t S;
+		const bool vec_ok = aligned_to(A, 16) && aligned_to(B, 16) && (lda * sizeof(TE)) % 16 == 0 && (ldb * sizeof(TE)) % 16 == 0
+				&& (sA * sizeof(TE)) % 16 == 0 && (sB * sizeof(TE)) % 16 == 0;
+		const bool vec_c = aligned_to(C, 4 * sizeof(TC)) && ldc % 4 == 0 && sC % 4 == 0;
+		const dim3 grid(ceil_div(M, BLOCK_M), ceil_div(N, BLOCK_N), batch);
+		hipLaunchKernelGGL((k_gemm_nt_mfma<TE, TC>), grid, dim3(256), 0, s, static_cast<const TE*>(A), static_cast<const TE*>(B), static_cast<TC*>(C), M, N, K,
+				lda, ldb, ldc, sA, sB, sC, static_cast<S>(alpha), static_cast<S>(beta), (vec_ok ? 1 : 0) | (vec_c ? 2 : 0));
+		return 0;
+	}
+	template<typename TA, typename TC, typename CT>
+	int launch_generic(hipStream_t s, const void *A, const void *B, void *C, int batch, int M, int N, int K, int opA, int opB, int lda, int ldb, int ldc,
+			int64_t sA, int64_t sB, int64_t sC, double alpha, double beta)
+	{
+		const dim3 grid(ceil_div(N, 16), ceil_div(M, 16), batch);
+		hipLaunchKernelGGL((k_gemm_generic<TA, TC, CT>), grid, dim3(256), 0, s, static_cast<const TA*>(A), static_cast<const TA*>(B), static_cast<TC*>(C), M, N,
+				K, opA, opB, lda, ldb, ldc, sA, sB, sC, static_cast<CT>(alpha), static_cast<CT>(beta));
+		return 0;
+	}
+}
+
+extern "C" int avhip_gemm_batched(void *stream, int ab_dtype, int c_dtype, int opA, int opB, const void *A, const void *B, void *C, int batch, int M,
+		int N, int K, int lda, int ldb, int ldc, int64_t strideA, int64_t strideB, int64_t strideC, double alpha, double beta)
+{
+	if (A == nullptr || B == nullptr || C == nullptr || batch <= 0 || M <= 0 || N <= 0 || K <= 0)
+		return AVHIP_BAD_PARAM;
+	if (batch > 65535)
+		return AVHIP_NOT_SUPPORTED;
+	hipStream_t s = static_cast<hipStream_t>(stream);
+	const bool nt = (opA == 0 && opB != 0);
+#define ARGS_MFMA s, A, B, C, batch, M, N, K, lda, ldb, ldc, strideA, strideB, strideC, alpha, beta
+#define ARGS_GEN s, A, B, C, batch, M, N, K, opA, opB, lda, ldb, ldc, strideA, strideB, strideC, alpha, beta
+	switch (ab_dtype)
+	{
+		case DT_FLOAT32:
+			if (c_dtype != DT_FLOAT32)
+				return AVHIP_UNSUPPORTED_DATATYPE;
+			return nt ? launch_mfma<float, float>(ARGS_MFMA) : launch_generic<float, float, float>(ARGS_GEN);
+		case DT_FLOAT64:
+			if (c_dtype != DT_FLOAT64)
+				return AVHIP_UNSUPPORTED_DATATYPE;
+			return launch_generic<double, double, double>(ARGS_GEN);
+		case DT_FLOAT16:
+			if (c_dtype == DT_FLOAT16)
+				return nt ? launch_mfma<f16_t, f16_t>(ARGS_MFMA) : launch_generic<f16_t, f16_t, float>(ARGS_GEN);
+			if (c_dtype == DT_FLOAT32)
+				return nt ? launch_mfma<f16_t, float>(ARGS_MFMA) : launch_generic<f16_t, float, float>(ARGS_GEN);
+			return AVHIP_UNSUPPORTED_DATATYPE;
+		case DT_BFLOAT16:
+			if (c_dtype == DT_BFLOAT16)
+				return nt ? launch_mfma<bf16_t, bf16_t>(ARGS_MFMA) : launch_generic<bf16_val, bf16_val, float>(ARGS_GEN);
+			if (c_dtype == DT_FLOAT32)
+				return nt ? launch_mfma<bf16_t, float>(ARGS_MFMA) : launch_generic<bf16_val, float, float>(ARGS_GEN);
+			return AVHIP_UNSUPPORTED_DATATYPE;
+		case DT_INT8:
+			if (c_dtype != DT_INT32)
+				return AVHIP_UNSUPPORTED_DATATYPE;
+			return nt ? launch_mfma<int8_t, int>(ARGS_MFMA) : launch_generic<int8_t, int, int>(ARGS_GEN);
+		default:
+			return AVHIP_UNSUPPORTED_DATATYPE;
+	}
+#undef ARGS_MFMA
+#undef ARGS_GEN
+}

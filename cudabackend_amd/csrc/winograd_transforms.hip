@@ -1,0 +1,414 @@
+/*
+ * winograd_transforms.hip -- the three non-fused Winograd transforms for F(2x2,3x3), F(4x4,3x3) and F(2x2,5x5).
+ *
+ * Replaces kernel_winograd_{weight,input,output}_transform and their launchers of the reference
+ * (src/winograd_nonfused.cu:257-423, 609-777).  The mathematics is the same sandwich product M * tile * M^T with the
+ * same coefficient tables (src/winograd_nonfused.cu:534-575); the mapping to the machine is not:
+ *
+ *  - these kernels are HBM-bound, so one work-item owns one tile x one 16-byte (or 8-byte) vector of channels, issues
+ *    all t*t vector loads up front, transforms in registers and writes t*t vectors.  A 64-wide wavefront therefore reads
+ *    and writes whole 512- or 1024-byte channel rows, and consecutive wavefronts walk consecutive tiles of one matrix plane;
+ *  - the coefficient tables are compile-time constants: zero terms disappear and +-1 terms become adds when the loops are
+ *    unrolled, so there is no table upload, no LDS and no data-dependent branch;
+ *  - overlapping tile halos are served by L2 / Infinity Cache, not staged through LDS;
+ *  - the matrix dtype is independent of the tensor dtype (fp16 or fp32 matrices for 16-bit tensors keep F(4x4,3x3) usable);
+ *  - 16-bit values are computed in fp32 and rounded to nearest even on store.
+ */
+#include "common.hpp"
+
+namespace
+{
+	using namespace avhip;
+
+	/* Coefficient tables (row-major).  which: 0 = G [t x r], 1 = B^T [t x t], 2 = A^T [m x t]. */
+	template<int M, int R> struct Tab;
+	template<> struct Tab<2, 3>
+	{
+		__host__ __device__ static constexpr double get(int which, int i, int j)
+		{
+			constexpr double G[4 * 3] = { 1, 0, 0, 1, 1, 1, 1, -1, 1, 0, 0, 1 };
+			constexpr double BT[4 * 4] = { 1, 0, -1, 0, 0, 1, 1, 0, 0, -1, 1, 0, 0, -1, 0, 1 };
+			constexpr double AT[2 * 4] = { 1, 0.5, 0.5, 0, 0, 0.5, -0.5, 1 };
+			return which == 0 ? G[i * 3 + j] : which == 1 ? BT[i * 4 + j] : AT[i * 4 + j];
+		}
+	};
+	template<> struct Tab<4, 3>
+	{
+		__host__ __device__ static constexpr double get(int which, int i, int j)
+		{
+			constexpr double a = 1.0 / 3.0;
+			constexpr double G[6 * 3] = { 1, 0, 0, 2 * a, 2 * a, 2 * a, 2 * a, -2 * a, 2 * a, a, 2 * a, 4 * a, a, -2 * a, 4 * a, 0, 0, 2 };
+			constexpr double BT[6 * 6] = { 1, 0, -1.25, 0, 0.25, 0, 0, 1, 1, -0.25, -0.25, 0, 0, -1, 1, 0.25, -0.25, 0, 0, -1, -0.5, 1, 0.5, 0, 0, 1, -0.5,
+					-1, 0.5, 0, 0, 1, 0, -1.25, 0, 0.25 };
+			constexpr double AT[4 * 6] = { 1, 1, 1, 0.25, 0.25, 0, 0, 1, -1, 0.5, -0.5, 0, 0, 1, 1, 1, 1, 0, 0, 1, -1, 2, -2, 2 };
+			return which == 0 ? G[i * 3 + j] : which == 1 ? BT[i * 6 + j] : AT[i * 6 + j];
+		}
+	};
+	template<> struct Tab<2, 5>
+	{
+		__host__ __device__ static constexpr double get(int which, int i, int j)
+		{
+			constexpr double a = 1.0 / 3.0;
+			constexpr double G[6 * 5] = { 1, 0, 0, 0, 0, 2 * a, 2 * a, 2 * a, 2 * a, 2 * a, 2 * a, -2 * a, 2 * a, -2 * a, 2 * a, a / 2, a, 2 * a, 4 * a, 8 * a,
+					a / 2, -a, 2 * a, -4 * a, 8 * a, 0, 0, 0, 0, 2 };
+			constexpr double BT[6 * 6] = { 1, 0, -1.25, 0, 0.25, 0, 0, 1, 1, -0.25, -0.25, 0, 0, -1, 1, 0.25, -0.25, 0, 0, -1, -0.5, 1, 0.5, 0, 0, 1, -0.5,
+					-1, 0.5, 0, 0, 1, 0, -1.25, 0, 0.25 };
+			constexpr double AT[2 * 6] = { 1, 1, 1, 0.5, 0.5, 0, 0, 1, -1, 1, -1, 2 };
+			return which == 0 ? G[i * 5 + j] : which == 1 ? BT[i * 6 + j] : AT[i * 6 + j];
+		}
+	};
+
+	/* acc (+)= c * d with the coefficient known at compile time once the caller's loops are unrolled. */
+	template<typename CT, int V>
+	__device__ inline void axpy(bool &have, CT (&acc)[V], double c, const CT (&d)[V])
+	{
+		if (c == 0.0)
+			return;
+#pragma unroll
+		for (int v = 0; v < V; v++)
+		{
+			const CT term = (c == 1.0) ? d[v] : (c == -1.0) ? -d[v] : static_cast<CT>(c) * d[v];
+			acc[v] = have ? acc[v] + term : term;
+		}
+		have = true;
+	}
+
+	/* out[ROWS x ROWS] = Mx[ROWS x COLS] * d[COLS x COLS] * Mx^T, Mx = table `WHICH` of Tab<M, R>. */
+	template<int M, int R, int WHICH, int ROWS, int COLS, typename CT, int V>
+	__device__ inline void sandwich(const CT (&d)[COLS * COLS][V], CT (&out)[ROWS * ROWS][V])
+	{
+		CT tmp[ROWS * COLS][V];
+#pragma unroll
+		for (int i = 0; i < ROWS; i++)
+#pragma unroll
+			for (int j = 0; j < COLS; j++)
+			{
+				bool have = false;
+#pragma unroll
+				for (int k = 0; k < COLS; k++)
+					axpy<CT, V>(have, tmp[i * COLS + j], Tab<M, R>::get(WHICH, i, k), d[k * COLS + j]);
+				if (!have)
+				{
+#pragma unroll
+					for (int v = 0; v < V; v++)
+						tmp[i * COLS + j][v] = static_cast<CT>(0);
+				}
+			}
+#pragma unroll
+		for (int i = 0; i < ROWS; i++)
+#pragma unroll
+			for (int j = 0; j < ROWS; j++)
+			{
+				bool have = false;
+#pragma unroll
+				for (int k = 0; k < COLS; k++)
+					axpy<CT, V>(have, out[i * ROWS + j], Tab<M, R>::get(WHICH, j, k), tmp[i * COLS + k]);
+				if (!have)
+				{
+#pragma unroll
+					for (int v = 0; v < V; v++)
+						out[i * ROWS + j][v] = static_cast<CT>(0);
+				}
+			}
+	}
+
+	template<int M, int R, typename T, typename TM, int V>
+	__global__ __launch_bounds__(256) void k_weight_transform(const T *__restrict__ w, TM *__restrict__ U, int K, int C, int invert)
+	{
+		typedef typename Traits<T>::compute CT;
+		constexpr int t = M + R - 1;
+		const int CV = (C + V - 1) / V;
+		const size_t gid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+		const int cv = static_cast<int>(gid % CV);
+		const size_t k = gid / CV;
+		if (k >= static_cast<size_t>(K))
+			return;
+		const int c = cv * V;
+		const int valid = C - c;
+
+		CT g[R * R][V];
+#pragma unroll
+		for (int i = 0; i < R; i++)
+#pragma unroll
+			for (int j = 0; j < R; j++)
+			{
+				const int si = invert ? (R - 1 - i) : i;
+				const int sj = invert ? (R - 1 - j) : j;
+				load_vec<T, V, CT>(w + ((k * R + si) * R + sj) * C + c, valid, g[i * R + j]);
+			}
+		CT out[t * t][V];
+		sandwich<M, R, 0, t, R, CT, V>(g, out);
+#pragma unroll
+		for (int i = 0; i < t * t; i++)
+		{
+			typename Traits<TM>::compute o[V];
+#pragma unroll
+			for (int v = 0; v < V; v++)
+				o[v] = static_cast<typename Traits<TM>::compute>(out[i][v]);
+			store_vec<TM, V>(U + (static_cast<size_t>(i) * K + k) * C + c, valid, o);
+		}
+	}
+
+	template<int M, int R, typename T, typename TM, int V>
+	__global__ __launch_bounds__(256) void k_input_transform(const T *__restrict__ x, TM *__restrict__ Vm, int N, int H, int W, int C, int Th, int Tw,
+			int pad_h, int pad_w, typename Traits<T>::compute padv)
+	{
+		typedef typename Traits<T>::compute CT;
+		constexpr int t = M + R - 1;
+		const int CV = (C + V - 1) / V;
+		const size_t tiles = static_cast<size_t>(N) * Th * Tw;
+		const size_t gid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+		const int cv = static_cast<int>(gid % CV);
+		const size_t tile = gid / CV;
+		if (tile >= tiles)
+			return;
+		const int tw = static_cast<int>(tile % Tw);
+		const int th = static_cast<int>((tile / Tw) % Th);
+		const size_t n = tile / (static_cast<size_t>(Tw) * Th);
+		const int c = cv * V;
+		const int valid = C - c;
+
+		CT d[t * t][V];
+#pragma unroll
+		for (int a = 0; a < t; a++)
+#pragma unroll
+			for (int b = 0; b < t; b++)
+			{
+				const int ih = pad_h + th * M + a;
+				const int iw = pad_w + tw * M + b;
+				if (ih >= 0 && ih < H && iw >= 0 && iw < W)
+					load_vec<T, V, CT>(x + ((n * H + ih) * W + iw) * C + c, valid, d[a * t + b]);
+				else
+				{
+#pragma unroll
+					for (int v = 0; v < V; v++)
+						d[a * t + b][v] = padv;
+				}
+			}
+		CT out[t * t][V];
+		sandwich<M, R, 1, t, t, CT, V>(d, out);
+#pragma unroll
+		for (int i = 0; i < t * t; i++)
+		{
+			typename Traits<TM>::compute o[V];
+#pragma unroll
+			for (int v = 0; v < V; v++)
+				o[v] = static_cast<typename Traits<TM>::compute>(out[i][v]);
+			store_vec<TM, V>(Vm + (static_cast<size_t>(i) * tiles + tile) * C + c, valid, o);
+		}
+	}
+
+	template<int M, int R, typename T, typename TM, int V>
+	__global__ __launch_bounds__(256) void k_output_transform(const TM *__restrict__ Mx, T *y, const typename Traits<T>::compute *__restrict__ bias,
+			const T *z, int N, int H, int W, int K, int Th, int Tw, typename Traits<T>::compute alpha1, typename Traits<T>::compute alpha2,
+			typename Traits<T>::compute beta, int activation)
+	{
+		typedef typename Traits<T>::compute CT;
+		constexpr int t = M + R - 1;
+		const int KV = (K + V - 1) / V;
+		const size_t tiles = static_cast<size_t>(N) * Th * Tw;
+		const size_t gid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+		const int kv = static_cast<int>(gid % KV);
+		const size_t tile = gid / KV;
+		if (tile >= tiles)
+			return;
+		const int tw = static_cast<int>(tile % Tw);
+		const int th = static_cast<int>((tile / Tw) % Th);
+		const size_t n = tile / (static_cast<size_t>(Tw) * Th);
+		const int k = kv * V;
+		const int valid = K - k;
+
+		CT d[t * t][V];
+#pragma unroll
+		for (int i = 0; i < t * t; i++)
+		{
+			typename Traits<TM>::compute tmp[V];
+			load_vec<TM, V>(Mx + (static_cast<size_t>(i) * tiles + tile) * K + k, valid, tmp);
+#pragma unroll
+			for (int v = 0; v < V; v++)
+				d[i][v] = static_cast<CT>(tmp[v]);
+		}
+		CT out[M * M][V];
+		sandwich<M, R, 2, M, t, CT, V>(d, out);
+
+		CT bv[V];
+#pragma unroll
+		for (int v = 0; v < V; v++)
+			bv[v] = (bias != nullptr && v < valid) ? bias[k + v] : static_cast<CT>(0);
+
+#pragma unroll
+		for (int a = 0; a < M; a++)
+#pragma unroll
+			for (int b = 0; b < M; b++)
+			{
+				const int oh = th * M + a;
+				const int ow = tw * M + b;
+				if (oh < H && ow < W)
+				{
+					const size_t idx = ((n * H + oh) * W + ow) * K + k;
+					CT r[V];
+#pragma unroll
+					for (int v = 0; v < V; v++)
+						r[v] = alpha1 * out[a * M + b][v] + bv[v];
+					if (z != nullptr)
+					{
+						CT zv[V];
+						load_vec<T, V, CT>(z + idx, valid, zv);
+#pragma unroll
+						for (int v = 0; v < V; v++)
+							r[v] += alpha2 * zv[v];
+					}
+#pragma unroll
+					for (int v = 0; v < V; v++)
+						r[v] = activation_forward<CT>(activation, r[v]);
+					if (beta != static_cast<CT>(0))
+					{
+						CT yv[V];
+						load_vec<T, V, CT>(y + idx, valid, yv);
+#pragma unroll
+						for (int v = 0; v < V; v++)
+							r[v] += beta * yv[v];
+					}
+					store_vec<T, V>(y + idx, valid, r);
+				}
+			}
+	}
+
+	/* Widest vector (in elements) that keeps every access of a [.., C] tensor of `elem` bytes aligned. */
+	template<typename T, typename TM>
+	int pick_vec(int C, const void *p0, const void *p1, const void *p2 = nullptr)
+	{
+		constexpr int V = 4 * sizeof(float) / ((sizeof(T) > sizeof(TM) ? sizeof(T) : sizeof(TM))); // 16 B of the wider type
+		constexpr int VV = V > 4 ? 4 : V; // at most 4 channels per work-item keeps the t*t tile in registers
+		const size_t need = VV * (sizeof(T) > sizeof(TM) ? sizeof(T) : sizeof(TM));
+		if (VV > 1 && C % VV == 0 && aligned_to(p0, need) && aligned_to(p1, need) && (p2 == nullptr || aligned_to(p2, need)))
+			return VV;
+		return 1;
+	}
+	template<typename T, typename TM> struct VecOf
+	{
+		static constexpr int wide = 4 * sizeof(float) / ((sizeof(T) > sizeof(TM) ? sizeof(T) : sizeof(TM)));
+		static constexpr int value = wide > 4 ? 4 : wide;
+	};
+
+	template<typename T> typename Traits<T>::compute host_scalar(const void *p)
+	{
+		if (p == nullptr)
+			return static_cast<typename Traits<T>::compute>(0);
+		return Traits<T>::load(*reinterpret_cast<const T*>(p));
+	}
+
+	template<int M, int R, typename T, typename TM>
+	int launch_weight(hipStream_t s, const void *w, void *U, int K, int C, int invert)
+	{
+		const int V = pick_vec<T, TM>(C, w, U);
+		const size_t items = static_cast<size_t>(K) * ((C + V - 1) / V);
+		const dim3 grid(ceil_div(items, 256));
+		if (V > 1)
+			hipLaunchKernelGGL((k_weight_transform<M, R, T, TM, VecOf<T, TM>::value>), grid, dim3(256), 0, s, static_cast<const T*>(w), static_cast<TM*>(U), K, C,
+					invert);
+		else
+			hipLaunchKernelGGL((k_weight_transform<M, R, T, TM, 1>), grid, dim3(256), 0, s, static_cast<const T*>(w), static_cast<TM*>(U), K, C, invert);
+		return 0;
+	}
+	template<int M, int R, typename T, typename TM>
+	int launch_input(hipStream_t s, const void *x, void *Vm, int N, int H, int W, int C, int pad_h, int pad_w, const void *padding_value)
+	{
+		const int Th = (H + M - 1) / M, Tw = (W + M - 1) / M;
+		const int V = pick_vec<T, TM>(C, x, Vm);
+		const size_t items = static_cast<size_t>(N) * Th * Tw * ((C + V - 1) / V);
+		const dim3 grid(ceil_div(items, 256));
+		const typename Traits<T>::compute padv = host_scalar<T>(padding_value);
+		if (V > 1)
+			hipLaunchKernelGGL((k_input_transform<M, R, T, TM, VecOf<T, TM>::value>), grid, dim3(256), 0, s, static_cast<const T*>(x), static_cast<TM*>(Vm), N, H, W,
+					C, Th, Tw, pad_h, pad_w, padv);
+		else
+			hipLaunchKernelGGL((k_input_transform<M, R, T, TM, 1>), grid, dim3(256), 0, s, static_cast<const T*>(x), static_cast<TM*>(Vm), N, H, W, C, Th, Tw,
+					pad_h, pad_w, padv);
+		return 0;
+	}
+	template<int M, int R, typename T, typename TM>
+	int launch_output(hipStream_t s, const void *Mx, void *y, const void *bias, const void *z, int N, int H, int W, int K, double alpha1, double alpha2,
+			double beta, int activation)
+	{
+		typedef typename Traits<T>::compute CT;
+		const int Th = (H + M - 1) / M, Tw = (W + M - 1) / M;
+		int V = pick_vec<T, TM>(K, Mx, y, z);
+		const size_t items = static_cast<size_t>(N) * Th * Tw * ((K + V - 1) / V);
+		const dim3 grid(ceil_div(items, 256));
+		if (V > 1)
+			hipLaunchKernelGGL((k_output_transform<M, R, T, TM, VecOf<T, TM>::value>), grid, dim3(256), 0, s, static_cast<const TM*>(Mx), static_cast<T*>(y),
+					static_cast<const CT*>(bias), static_cast<const T*>(z), N, H, W, K, Th, Tw, static_cast<CT>(alpha1), static_cast<CT>(alpha2),
+					static_cast<CT>(beta), activation);
+		else
+			hipLaunchKernelGGL((k_output_transform<M, R, T, TM, 1>), grid, dim3(256), 0, s, static_cast<const TM*>(Mx), static_cast<T*>(y),
+					static_cast<const CT*>(bias), static_cast<const T*>(z), N, H, W, K, Th, Tw, static_cast<CT>(alpha1), static_cast<CT>(alpha2),
+					static_cast<CT>(beta), activation);
+		return 0;
+	}
+
+	/* Supported (tensor dtype, matrix dtype) pairs: equal types (the reference's behaviour), and fp16 or fp32 matrices
+	 * for 16-bit tensors.  CALL is instantiated with <T, TM>. */
+#define AVHIP_DISPATCH_PAIR(dtype, mat_dtype, CALL)                                              \
+	switch (dtype)                                                                                 \
+	{                                                                                              \
+		case DT_FLOAT32:                                                                           \
+			if (mat_dtype == DT_FLOAT32) { CALL(float, float); }                                   \
+			return AVHIP_UNSUPPORTED_DATATYPE;                                                     \
+		case DT_FLOAT64:                                                                           \
+			if (mat_dtype == DT_FLOAT64) { CALL(double, double); }                                 \
+			return AVHIP_UNSUPPORTED_DATATYPE;                                                     \
+		case DT_FLOAT16:                                                                           \
+			if (mat_dtype == DT_FLOAT16) { CALL(f16_t, f16_t); }                                   \
+			if (mat_dtype == DT_FLOAT32) { CALL(f16_t, float); }                                   \
+			return AVHIP_UNSUPPORTED_DATATYPE;                                                     \
+		case DT_BFLOAT16:                                                                          \
+			if (mat_dtype == DT_BFLOAT16) { CALL(bf16_t, bf16_t); }                                \
+			if (mat_dtype == DT_FLOAT16) { CALL(bf16_t, f16_t); }                                  \
+			if (mat_dtype == DT_FLOAT32) { CALL(bf16_t, float); }                                  \
+			return AVHIP_UNSUPPORTED_DATATYPE;                                                     \
+		default:                                                                                   \
+			return AVHIP_UNSUPPORTED_DATATYPE;                                                     \
+	}
+
+#define AVHIP_DISPATCH_MR(m, r, FN, T, TM, ...)                                                  \
+	if (m == 2 && r == 3) return FN<2, 3, T, TM>(__VA_ARGS__);                                    \
+	if (m == 4 && r == 3) return FN<4, 3, T, TM>(__VA_ARGS__);                                    \
+	if (m == 2 && r == 5) return FN<2, 5, T, TM>(__VA_ARGS__);                                    \
+	return AVHIP_NOT_SUPPORTED;
+}
+
+extern "C"
+{
+	int avhip_winograd_weight_transform(void *stream, int dtype, int mat_dtype, int m, int r, int invert, const void *w, void *U, int K, int C)
+	{
+		if (w == nullptr || U == nullptr || K <= 0 || C <= 0)
+			return AVHIP_BAD_PARAM;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+#define CALL(T, TM) AVHIP_DISPATCH_MR(m, r, launch_weight, T, TM, s, w, U, K, C, invert)
+		AVHIP_DISPATCH_PAIR(dtype, mat_dtype, CALL)
+#undef CALL
+	}
+
+	int avhip_winograd_input_transform(void *stream, int dtype, int mat_dtype, int m, int r, const void *x, void *V, int N, int H, int W, int C,
+			int pad_h, int pad_w, const void *padding_value)
+	{
+		if (x == nullptr || V == nullptr || N <= 0 || H <= 0 || W <= 0 || C <= 0)
+			return AVHIP_BAD_PARAM;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+#define CALL(T, TM) AVHIP_DISPATCH_MR(m, r, launch_input, T, TM, s, x, V, N, H, W, C, pad_h, pad_w, padding_value)
+		AVHIP_DISPATCH_PAIR(dtype, mat_dtype, CALL)
+#undef CALL
+	}
+
+	int avhip_winograd_output_transform(void *stream, int dtype, int mat_dtype, int m, int r, const void *M, void *y, const void *bias, const void *z,
+			int N, int H, int W, int K, double alpha1, double alpha2, double beta, int activation)
+	{
+		if (M == nullptr || y == nullptr || N <= 0 || H <= 0 || W <= 0 || K <= 0)
+			return AVHIP_BAD_PARAM;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+#define CALL(T, TM) AVHIP_DISPATCH_MR(m, r, launch_output, T, TM, s, M, y, bias, z, N, H, W, K, alpha1, alpha2, beta, activation)
+		AVHIP_DISPATCH_PAIR(dtype, mat_dtype, CALL)
+#undef CALL
+	}
+}

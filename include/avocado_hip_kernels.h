@@ -1,0 +1,106 @@
+/*
+ * avocado_hip_kernels.h
+ *
+ * The thin C-ABI layer between the host code of the backend (descriptors, validation, dispatch) and the
+ * hand-written HIP kernels for gfx950.  Plain device pointers, sizes and a stream; nothing here knows
+ * about descriptors.  Each launcher enqueues on `stream` and returns without synchronising.
+ *
+ * Return value of every launcher:
+ *    0   launched (launch errors are picked up with hipGetLastError by the caller's status mapping)
+ *   >0   a hipError_t
+ *   AVHIP_NOT_SUPPORTED / AVHIP_UNSUPPORTED_DATATYPE / AVHIP_BAD_PARAM (negative)
+ *
+ * Data types are the integer values of avDataType_t.  Tensors are NHWC, weights [K, R, S, C], Winograd
+ * matrices [t*t, tiles, C] with t = m + r - 1 and tile = (n*ceil(H/m) + th)*ceil(W/m) + tw
+ * (src/activations.cuh:30-121 of the reference).  Scalars are passed as double and narrowed to the compute
+ * type of the kernel (fp32 for fp16/bf16/fp32/int8 tensors, fp64 for fp64 tensors).
+ */
+#ifndef AVOCADO_HIP_KERNELS_H_
+#define AVOCADO_HIP_KERNELS_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C"
+{
+#endif
+
+#ifndef AVHIP_API
+#  define AVHIP_API __attribute__((visibility("default")))
+#endif
+
+#define AVHIP_NOT_SUPPORTED (-1)
+#define AVHIP_UNSUPPORTED_DATATYPE (-2)
+#define AVHIP_BAD_PARAM (-3)
+
+	/* Geometry of one 2-D convolution.  pad_* are Avocado's signed input offsets (3x3 "same" is -1). */
+	typedef struct
+	{
+		int N, H, W, C; /* input  [N, H, W, C]  */
+		int K, R, S; /* weights [K, R, S, C] */
+		int Ho, Wo; /* output [N, Ho, Wo, K] */
+		int pad_h, pad_w;
+		int stride_h, stride_w;
+		int dil_h, dil_w;
+		int mode; /* avConvolutionMode_t */
+	} avhipConvShape;
+
+	/* U = G g G^T.  Replaces launch_weight_transform / kernel_winograd_weight_transform,
+	 * src/winograd_nonfused.cu:609,257.  w dtype `dtype`, U dtype `mat_dtype`. */
+	AVHIP_API int avhip_winograd_weight_transform(void *stream, int dtype, int mat_dtype, int m, int r, int invert, const void *w, void *U, int K, int C);
+
+	/* V = B^T d B with offset padding.  Replaces launch_input_transform / kernel_winograd_input_transform,
+	 * src/winograd_nonfused.cu:654,303.  padding_value points to a host scalar of type `dtype` or is null (0). */
+	AVHIP_API int avhip_winograd_input_transform(void *stream, int dtype, int mat_dtype, int m, int r, const void *x, void *V, int N, int H, int W, int C,
+			int pad_h, int pad_w, const void *padding_value);
+
+	/* y = act(alpha1 * A^T M A + bias + alpha2 * z) + beta * y.  Replaces launch_output_transform /
+	 * kernel_winograd_output_transform, src/winograd_nonfused.cu:704,367.  bias is fp32 (fp64 for fp64 tensors)
+	 * or null, z has the dtype of y or is null. */
+	AVHIP_API int avhip_winograd_output_transform(void *stream, int dtype, int mat_dtype, int m, int r, const void *M, void *y, const void *bias, const void *z,
+			int N, int H, int W, int K, double alpha1, double alpha2, double beta, int activation);
+
+	/* C[b] = alpha * op(A[b]) op(B[b]) + beta * C[b], row-major.  Replaces the cuBLAS calls of cudaGemm and
+	 * cudaGemmBatched, src/gemm.cpp:25-124,126-209.  ab_dtype: FLOAT16 / BFLOAT16 / FLOAT32 / FLOAT64 / INT8;
+	 * c_dtype: same as ab_dtype, FLOAT32 for 16-bit inputs, INT32 for INT8.  Strides are in elements. */
+	AVHIP_API int avhip_gemm_batched(void *stream, int ab_dtype, int c_dtype, int opA, int opB, const void *A, const void *B, void *C, int batch, int M, int N,
+			int K, int lda, int ldb, int ldc, int64_t strideA, int64_t strideB, int64_t strideC, double alpha, double beta);
+
+	/* y = act(alpha1 * conv(x, w) + bias + alpha2 * z) + beta * y by implicit GEMM on MFMA.  Replaces
+	 * cuda_convolution2dImplicitGemm / kernel_conv_implicit_gemm, src/conv2d_implicit_gemm.cu:303,152.
+	 *   x_dtype FLOAT16 / BFLOAT16 / FLOAT32 : y and z have x_dtype, bias is fp32
+	 *   x_dtype INT8, y_dtype INT32, bias_dtype INT32, alpha1 == 1, beta == 0, no z, LINEAR or RELU: exact integers
+	 *   x_dtype INT8 otherwise: fp32 epilogue on the int32 sum, bias fp32, y INT32 / INT8 / FLOAT32
+	 *   requant_scale != null (x INT8, y INT8, bias INT32): y = sat_i8(rne(float(sum + bias) * scale[k]))
+	 * padding_value points to a host scalar of x_dtype or is null (0). */
+	AVHIP_API int avhip_conv2d_implicit_gemm(void *stream, int x_dtype, int y_dtype, int bias_dtype, const avhipConvShape *shape, const void *x, const void *w,
+			const void *bias, const void *z, void *y, const void *padding_value, double alpha1, double alpha2, double beta, int activation,
+			const float *requant_scale);
+
+	/* Same formula by a single fused Winograd F(2x2, 3x3) kernel (3x3, stride 1, dilation 1).  Replaces
+	 * cuda_winogradFusedForward / kernel_winograd_fused, src/winograd_fused.cu:789,590.
+	 * U is the transformed weight set [16, K, C] in FLOAT16 (16-bit tensors) or FLOAT32 (fp32 tensors). */
+	AVHIP_API int avhip_conv2d_winograd_fused(void *stream, int dtype, const avhipConvShape *shape, const void *x, const void *U, const void *bias, const void *z,
+			void *y, double alpha1, double alpha2, double beta, int activation);
+
+	/* y = alpha1 * act(alpha2 * x + b + beta1 * z) + beta2 * z + beta3 * y.  Replaces kernel_add_bias,
+	 * src/tensor_op.cu:199-228.  x, y, z have `dtype`; b is fp32 (fp64 for fp64 tensors). */
+	AVHIP_API int avhip_add_bias(void *stream, int dtype, const void *x, const void *b, const void *z, void *y, int64_t first, int last, double alpha1,
+			double alpha2, double beta1, double beta2, double beta3, int activation);
+
+	/* Explicit im2row, stride 1.  Replaces kernel_im2row_conv2d, src/im2row.cu:29-66.  elem_size in bytes. */
+	AVHIP_API int avhip_im2row(void *stream, int elem_size, const avhipConvShape *shape, const void *x, void *rows, const void *padding_value);
+
+	/* Element type conversion with round-to-nearest-even and saturation.  Replaces cudaChangeType's kernels,
+	 * src/conversions.cu:253-258. */
+	AVHIP_API int avhip_change_type(void *stream, void *dst, int dst_dtype, const void *src, int src_dtype, int64_t elements);
+
+	/* Fills `bytes` bytes at dst with a repeating pattern of 1, 2, 4, 8 or 16 bytes.  Replaces kernel_setall,
+	 * src/descriptors.cu:22-39. */
+	AVHIP_API int avhip_set_memory(void *stream, void *dst, int64_t bytes, const void *pattern, int pattern_size);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* AVOCADO_HIP_KERNELS_H_ */

@@ -1,0 +1,209 @@
+"""GPU parity of the convolution entry points (implicit GEMM, fused Winograd, dispatcher, requantised int8) against the CPU
+oracle on identical seeded inputs, through the C API.  Bars: int8 bit-exact; fp32 implicit GEMM rel-L2 <= 1e-5; fp32 Winograd
+<= 1e-4; fp16 / bf16 <= 2e-3."""
+import numpy as np
+import pytest
+
+import cudabackend_amd as cb
+import helpers as h
+
+pytestmark = pytest.mark.gpu
+
+BAR = {"f32": 1e-5, "f16": 2e-3, "bf16": 2e-3}
+
+
+def he(g, shape, dtype, orc):
+    K, R, S, Cin = shape
+    return h.rounded(orc, g.standard_normal(shape) * np.sqrt(2.0 / (R * S * Cin)), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_implicit_gemm_config1(oracle, dtype):
+    """BASELINE config 1: N=8, 15x15, 64->64, 3x3 offset -1, bias U(-0.1,0.1), ReLU."""
+    g = h.rng(20)
+    x = h.rounded(oracle, g.standard_normal((8, 15, 15, 64)), dtype)
+    w = he(g, (64, 3, 3, 64), dtype, oracle)
+    b = g.uniform(-0.1, 0.1, 64).astype(np.float32).astype(np.float64)
+    got = h.conv_forward("implicit_gemm", x, w, (8, 15, 15, 64), dtype, bias=b, activation=cb.ACTIVATION_RELU)
+    want = oracle.conv2d(x, w, b, activation=oracle.RELU)
+    err = oracle.rel_l2(got, want)
+    print("implicit gemm %s rel-L2 = %.3e" % (dtype, err))
+    assert err < BAR[dtype]
+
+
+CASES = [
+    # x shape, w shape, pad, stride, dilation, mode
+    dict(x=(3, 13, 14, 135), w=(21, 3, 3, 135), pad=(-1, -1)),                                   # odd everything, scalar tails
+    dict(x=(2, 12, 12, 32), w=(40, 5, 5, 32), pad=(-2, -2)),                                     # 5x5 "same"
+    dict(x=(2, 11, 13, 48), w=(24, 1, 1, 48), pad=(0, 0)),                                       # pointwise
+    dict(x=(2, 16, 16, 32), w=(48, 3, 3, 32), pad=(-1, -1), stride=(2, 2)),                       # downsampling
+    dict(x=(2, 15, 15, 16), w=(20, 3, 3, 16), pad=(-2, -2), dilation=(2, 2)),                     # dilated
+    dict(x=(2, 10, 9, 24), w=(36, 3, 3, 24), pad=(-1, -1), mode=1),                               # cross-correlation mode flips the kernel
+    dict(x=(2, 9, 10, 4), w=(32, 3, 3, 4), pad=(-1, -1)),                                         # 4 input planes (tower stem)
+    dict(x=(2, 8, 8, 160), w=(136, 3, 3, 160), pad=(-1, -1)),                                     # more than one filter block
+    dict(x=(1, 9, 11, 20), w=(8, 3, 2, 20), pad=(-1, 0)),                                         # non-square filter, asymmetric offsets
+]
+
+
+def out_shape(orc, c):
+    N, H, W, _ = c["x"]
+    K, R, S, _ = c["w"]
+    Ho, Wo = orc.conv_output_shape(H, W, R, S, c["pad"], c.get("stride", (1, 1)), c.get("dilation", (1, 1)))
+    return (N, Ho, Wo, K)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", CASES, ids=[str(i) for i in range(len(CASES))])
+def test_implicit_gemm_geometry(oracle, dtype, case):
+    g = h.rng(21)
+    x = h.rounded(oracle, g.standard_normal(case["x"]), dtype)
+    w = he(g, case["w"], dtype, oracle)
+    ys = out_shape(oracle, case)
+    kw = dict(pad=case["pad"], stride=case.get("stride", (1, 1)), dilation=case.get("dilation", (1, 1)), mode=case.get("mode", 0))
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, **kw)
+    want = oracle.conv2d(x, w, **kw)
+    assert got.shape == want.shape
+    assert oracle.rel_l2(got, want) < BAR[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_implicit_gemm_full_epilogue(oracle, dtype):
+    """alpha1, alpha2, beta, bias, residual and every activation, in the order of the reference's epilogue
+    (src/winograd_nonfused.cu:407-417)."""
+    g = h.rng(22)
+    x = h.rounded(oracle, g.standard_normal((2, 9, 9, 32)), dtype)
+    w = he(g, (24, 3, 3, 32), dtype, oracle)
+    b = g.uniform(-0.1, 0.1, 24).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal((2, 9, 9, 24)), dtype)
+    y0 = h.rounded(oracle, g.standard_normal((2, 9, 9, 24)), dtype)
+    a1, a2, be = float(np.float32(1.1)), float(np.float32(1.2)), float(np.float32(0.1))
+    for act in range(9):
+        got = h.conv_forward("implicit_gemm", x, w, y0.shape, dtype, bias=b, z=z, y0=y0, alpha1=a1, alpha2=a2, beta=be, activation=act)
+        want = oracle.conv2d(x, w, b, z, y0, alpha1=a1, alpha2=a2, beta=be, activation=act)
+        assert oracle.rel_l2(got, want) < BAR[dtype] * (3 if dtype == "f32" else 1), act
+
+
+def test_implicit_gemm_padding_value(oracle):
+    g = h.rng(23)
+    x = h.rounded(oracle, g.standard_normal((2, 7, 8, 32)), "f32")
+    w = he(g, (16, 3, 3, 32), "f32", oracle)
+    got = h.conv_forward("implicit_gemm", x, w, (2, 7, 8, 16), "f32", padding_value=0.5)
+    want = oracle.conv2d(x, w, padding_value=0.5)
+    assert oracle.rel_l2(got, want) < 1e-5
+
+
+# ---- int8 ------------------------------------------------------------------------------------------------------------
+INT8_CASES = [
+    dict(x=(4, 20, 20, 128), w=(128, 3, 3, 128), pad=(-1, -1)),      # config 4 at a reduced batch
+    dict(x=(4, 20, 20, 128), w=(128, 1, 1, 128), pad=(0, 0)),
+    dict(x=(2, 9, 11, 36), w=(20, 3, 3, 36), pad=(-1, -1)),          # channels not a multiple of the 64-byte step
+    dict(x=(2, 12, 12, 64), w=(72, 3, 3, 64), pad=(-1, -1), stride=(2, 2)),
+    dict(x=(2, 10, 10, 16), w=(8, 5, 5, 16), pad=(-2, -2), mode=1),
+    dict(x=(1, 6, 6, 7), w=(5, 3, 3, 7), pad=(-1, -1)),              # unaligned rows: element-wise loads
+]
+
+
+@pytest.mark.parametrize("case", INT8_CASES, ids=[str(i) for i in range(len(INT8_CASES))])
+def test_int8_int32_bit_exact(oracle, case):
+    g = h.rng(24)
+    x = g.integers(-127, 128, case["x"], dtype=np.int8)
+    w = g.integers(-127, 128, case["w"], dtype=np.int8)
+    b = g.integers(-2 ** 15, 2 ** 15, case["w"][0]).astype(np.int32)
+    kw = dict(pad=case["pad"], stride=case.get("stride", (1, 1)), mode=case.get("mode", 0))
+    ys = out_shape(oracle, case)
+    for act in (cb.ACTIVATION_LINEAR, cb.ACTIVATION_RELU):
+        got = h.conv_forward("implicit_gemm", x, w, ys, "i8", y_dtype="i32", bias=b, bias_dtype="i32", activation=act, **kw)
+        want = oracle.conv2d_i8(x, w, b, activation=act, **kw)
+        np.testing.assert_array_equal(got, want)
+    got = h.conv_forward("implicit_gemm", x, w, ys, "i8", y_dtype="i32", **kw)
+    np.testing.assert_array_equal(got, oracle.conv2d_i8(x, w, None, **kw))
+
+
+def test_int8_padding_value_bit_exact(oracle):
+    g = h.rng(25)
+    x = g.integers(-127, 128, (2, 8, 8, 32), dtype=np.int8)
+    w = g.integers(-127, 128, (16, 3, 3, 32), dtype=np.int8)
+    got = h.conv_forward("implicit_gemm", x, w, (2, 8, 8, 16), "i8", y_dtype="i32", padding_value=-3)
+    np.testing.assert_array_equal(got, oracle.conv2d_i8(x, w, None, padding_value=-3))
+
+
+@pytest.mark.parametrize("case", INT8_CASES[:3], ids=["3x3", "1x1", "ragged"])
+def test_int8_requantised_bit_exact(oracle, case):
+    """q = sat_i8(rne(float(sum + bias) * scale[k])), scale ~ U(1e-4, 1e-3) per output channel."""
+    g = h.rng(26)
+    x = g.integers(-127, 128, case["x"], dtype=np.int8)
+    w = g.integers(-127, 128, case["w"], dtype=np.int8)
+    K = case["w"][0]
+    b = g.integers(-2 ** 15, 2 ** 15, K).astype(np.int32)
+    scale = g.uniform(1e-4, 1e-3, K).astype(np.float32)
+    ys = out_shape(oracle, case)
+    for act in (cb.ACTIVATION_LINEAR, cb.ACTIVATION_RELU):
+        got = h.conv_forward("requant", x, w, ys, "i8", y_dtype="i8", bias=b, bias_dtype="i32", scale=scale, activation=act, pad=case["pad"])
+        want = oracle.requant_i8(oracle.conv2d_i8(x, w, b, pad=case["pad"], activation=act), scale)
+        np.testing.assert_array_equal(got, want)
+    assert np.abs(want).max() > 20  # the scale range really exercises the int8 range
+
+
+@pytest.mark.parametrize("y_dtype", ["i32", "i8", "f32"])
+def test_int8_float_epilogue(oracle, y_dtype):
+    """The header's convention for integer tensors: cast the int32 sum to fp32, scale and add in fp32, round to nearest even
+    and saturate on store (include/Avocado/cuda_backend.h:43-49).  Parity unpinned in the reference; the oracle restates the
+    same sequence of single roundings, so the comparison is exact for LINEAR / RELU."""
+    g = h.rng(27)
+    x = g.integers(-127, 128, (2, 6, 6, 64), dtype=np.int8)
+    w = g.integers(-127, 128, (16, 3, 3, 64), dtype=np.int8)
+    acc = oracle.conv2d_i8(x, w, None)
+    bias = g.uniform(-100, 100, 16).astype(np.float32)
+    np_dt = {"i32": np.int32, "i8": np.int8, "f32": np.float32}[y_dtype]
+    z = g.integers(-100, 100, acc.shape).astype(np_dt)
+    y0 = g.integers(-100, 100, acc.shape).astype(np_dt)
+    a1 = float(np.float32(1e-4 if y_dtype == "i8" else 0.37))
+    a2, be = float(np.float32(1.2)), float(np.float32(0.1))
+    got = h.conv_forward("implicit_gemm", x, w, acc.shape, "i8", y_dtype=y_dtype, bias=bias, bias_dtype="f32", z=z, y0=y0, alpha1=a1, alpha2=a2,
+                         beta=be, activation=cb.ACTIVATION_RELU)
+    want = oracle.conv2d_i8_float_epilogue(acc, bias, z, y0.copy(), a1, a2, be, oracle.RELU)
+    if y_dtype == "f32":
+        np.testing.assert_array_equal(np.asarray(got, dtype=np.float32), want)
+    else:
+        np.testing.assert_array_equal(got, want)
+
+
+# ---- dispatcher and argument checking -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,tol", [("f32", 1e-4), ("f16", 2e-3), ("bf16", 2e-3)])
+def test_dispatcher_config1(oracle, dtype, tol):
+    g = h.rng(28)
+    x = h.rounded(oracle, g.standard_normal((8, 15, 15, 64)), dtype)
+    w = he(g, (64, 3, 3, 64), dtype, oracle)
+    b = g.uniform(-0.1, 0.1, 64).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal((8, 15, 15, 64)), dtype)
+    got = h.conv_forward("dispatch", x, w, (8, 15, 15, 64), dtype, bias=b, z=z, activation=cb.ACTIVATION_RELU)
+    want = oracle.conv2d(x, w, b, z, activation=oracle.RELU)
+    err = oracle.rel_l2(got, want)
+    print("dispatcher %s rel-L2 = %.3e" % (dtype, err))
+    assert err < tol
+
+
+def test_dispatcher_without_workspace_falls_back(oracle):
+    g = h.rng(29)
+    x = h.rounded(oracle, g.standard_normal((2, 15, 15, 64)), "f32")
+    w = he(g, (64, 3, 3, 64), "f32", oracle)
+    got = h.conv_forward("dispatch", x, w, (2, 15, 15, 64), "f32", workspace_bytes=0)
+    assert oracle.rel_l2(got, oracle.conv2d(x, w)) < 1e-4
+    # stride 2 and int8 never use Winograd
+    got = h.conv_forward("dispatch", x, w, (2, 8, 8, 64), "f32", stride=(2, 2))
+    assert oracle.rel_l2(got, oracle.conv2d(x, w, stride=(2, 2))) < 1e-5
+    xi = g.integers(-127, 128, (2, 6, 6, 64), dtype=np.int8)
+    wi = g.integers(-127, 128, (8, 3, 3, 64), dtype=np.int8)
+    got = h.conv_forward("dispatch", xi, wi, (2, 6, 6, 8), "i8", y_dtype="i32")
+    np.testing.assert_array_equal(got, oracle.conv2d_i8(xi, wi, None))
+
+
+def test_convolution_argument_errors(oracle):
+    x = np.zeros((2, 6, 6, 8))
+    w = np.zeros((4, 3, 3, 8))
+    h.conv_forward("implicit_gemm", x, w, (2, 6, 6, 5), "f32", expect=cb.STATUS_BAD_PARAM)              # K mismatch
+    h.conv_forward("implicit_gemm", x, np.zeros((4, 3, 3, 7)), (2, 6, 6, 4), "f32", expect=cb.STATUS_BAD_PARAM)   # C mismatch
+    h.conv_forward("implicit_gemm", x, w, (2, 6, 6, 4), "f32", groups=2, expect=cb.STATUS_NOT_SUPPORTED)
+    h.conv_forward("implicit_gemm", x, w, (2, 6, 6, 4), "f64", expect=cb.STATUS_UNSUPPORTED_DATATYPE)
+    h.conv_forward("implicit_gemm", x, w, (2, 20, 20, 4), "f32", expect=cb.STATUS_BAD_PARAM)            # output larger than any window grid
+    h.conv_forward("winograd_fused", x, np.zeros((4, 5, 5, 8)), (2, 6, 6, 4), "f32", pad=(-2, -2), expect=cb.STATUS_NOT_SUPPORTED)

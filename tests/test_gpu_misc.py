@@ -1,0 +1,132 @@
+"""GPU tests of the helpers around the convolution path: add-bias, im2row, type conversion, memory and context entries."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import cudabackend_amd as cb
+import helpers as h
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype,tol", [("f16", 1e-3), ("bf16", 1e-2), ("f32", 1e-4), ("f64", 1e-4)])
+def test_add_bias_reference_case(oracle, dtype, tol):
+    """test/test_tensor_op.cpp:151-198: {23,45,67}, alpha1 1.1, alpha2 1.2, beta1 0.1, beta2 0.2, beta3 0.3, same tolerances."""
+    g = h.rng(30)
+    x = h.rounded(oracle, g.standard_normal((23, 45, 67)), dtype)
+    z = h.rounded(oracle, g.standard_normal((23, 45, 67)), dtype)
+    y0 = h.rounded(oracle, g.standard_normal((23, 45, 67)), dtype)
+    b = g.standard_normal(67)
+    b = b if dtype == "f64" else b.astype(np.float32).astype(np.float64)
+    s = (lambda v: v) if dtype == "f64" else (lambda v: float(np.float32(v)))
+    args = [s(1.1), s(1.2), s(0.1), s(0.2), s(0.3)]
+    for act in (cb.ACTIVATION_LINEAR, cb.ACTIVATION_RELU, cb.ACTIVATION_SIGMOID, cb.ACTIVATION_TANH):
+        got = h.add_bias(x, b, dtype, z, y0, *args, activation=act)
+        want = oracle.add_bias(x, b, z, y0, *args, activation=act)
+        assert oracle.rel_l2(got, want) < tol
+    # vectorised path (last dimension a multiple of 4), no z, no y
+    x4 = h.rounded(oracle, g.standard_normal((50, 128)), dtype)
+    b4 = g.standard_normal(128).astype(np.float32).astype(np.float64)
+    got = h.add_bias(x4, b4, dtype, activation=cb.ACTIVATION_RELU)
+    assert oracle.rel_l2(got, oracle.add_bias(x4, b4, activation=oracle.RELU)) < tol
+
+
+@pytest.mark.parametrize("R,pad,dtype", [(3, (-1, -1), "f32"), (5, (-2, -2), "f32"), (3, (-1, -1), "bf16"), (3, (-1, -1), "i8")])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_im2row(oracle, R, pad, dtype, mode):
+    """test/test_im2row.cpp:16-29: x {12,23,34,45}, 11 filters, 3x3 offset -1 and 5x5 offset -2 (batch reduced to 3)."""
+    g = h.rng(31)
+    shape = (3, 23, 34, 45)
+    if dtype == "i8":
+        x = g.integers(-127, 128, shape, dtype=np.int8)
+    else:
+        x = h.rounded(oracle, g.standard_normal(shape), dtype)
+    with h.Call() as c:
+        conv = cb.ConvolutionDescriptor(mode=mode, padding=pad)
+        xt = c.tensor(x, dtype)
+        wt = c.empty((11, R, R, 45), dtype)
+        rows = c.empty((3 * 23 * 34, R * R * 45), dtype)
+        cb.check(c.lib.cudaIm2Row(c.ctx.handle, conv.handle, wt.desc, xt.desc, xt.mem, rows.desc, rows.mem), "cudaIm2Row")
+        c.finish()
+        got = rows.download()
+    want = oracle.im2row(np.asarray(x, dtype=np.float64), R, R, pad, mode)
+    np.testing.assert_array_equal(np.asarray(got, dtype=np.float64), want)
+
+
+def test_change_type(oracle):
+    g = h.rng(32)
+    v = np.concatenate([g.standard_normal(1000) * 50, [0.5, 1.5, 2.5, -0.5, -1.5, 127.5, 300.0, -300.0, 1e10, -1e10]]).astype(np.float32)
+    import torch
+    with h.Call() as c:
+        src = c.tensor(v, "f32")
+        n = v.size
+        for dst_dtype, want in [
+            (cb.DTYPE_FLOAT16, v.astype(np.float16).astype(np.float64)),
+            (cb.DTYPE_BFLOAT16, torch.tensor(v).to(torch.bfloat16).to(torch.float64).numpy()),
+            (cb.DTYPE_INT8, np.clip(np.rint(v.astype(np.float64)), -128, 127)),
+            (cb.DTYPE_INT32, np.clip(np.rint(v.astype(np.float64)), -2 ** 31, 2 ** 31 - 1)),
+            (cb.DTYPE_FLOAT64, v.astype(np.float64)),
+        ]:
+            dst = c.empty((n,), dst_dtype)
+            cb.check(c.lib.cudaChangeType(c.ctx.handle, dst.mem, dst_dtype, src.mem, cb.DTYPE_FLOAT32, n), "cudaChangeType")
+            c.finish()
+            np.testing.assert_array_equal(np.asarray(dst.download(), dtype=np.float64), want)
+        # and back up: bf16 / int8 -> fp32 are exact
+        i8 = c.tensor(g.integers(-128, 128, 777, dtype=np.int8), "i8")
+        f = c.empty((777,), "f32")
+        cb.check(c.lib.cudaChangeType(c.ctx.handle, f.mem, cb.DTYPE_FLOAT32, i8.mem, cb.DTYPE_INT8, 777), "cudaChangeType")
+        c.finish()
+        np.testing.assert_array_equal(f.download(), i8.download().astype(np.float64))
+
+
+def test_memory_entries():
+    lib = cb.load_library()
+    assert lib.cudaGetNumberOfDevices() >= 1
+    name = C.create_string_buffer(256)
+    cb.check(lib.cudaGetDeviceProperty(0, cb.DEVICE_NAME, name), "name")
+    cus = C.c_int32(0)
+    cb.check(lib.cudaGetDeviceProperty(0, cb.DEVICE_PROCESSOR_COUNT, C.byref(cus)), "cus")
+    mem = C.c_int64(0)
+    cb.check(lib.cudaGetDeviceProperty(0, cb.DEVICE_MEMORY, C.byref(mem)), "memory")
+    print("device:", name.value.decode(), cus.value, "CUs", mem.value >> 30, "GiB")
+    assert cus.value > 0 and mem.value > 0
+    ctx = cb.Context(0)
+    dflt = lib.cudaGetDefaultContext(0)
+    m = C.c_int64(0)
+    cb.check(lib.cudaCreateMemoryDescriptor(C.byref(m), 0, 4096), "alloc")
+    # pattern fills of every width, checked on the host
+    for width in (1, 2, 4, 8, 16):
+        pattern = bytes(range(1, width + 1))
+        cb.check(lib.cudaSetMemory(ctx.handle, m.value, 0, 4096, pattern, width), "set")
+        ctx.synchronize()
+        host = np.empty(4096, dtype=np.uint8)
+        cb.check(lib.cudaCopyMemoryToHost(dflt, host.ctypes.data_as(C.c_void_p), m.value, 0, 4096), "d2h")
+        np.testing.assert_array_equal(host, np.tile(np.frombuffer(pattern, dtype=np.uint8), 4096 // width))
+    assert lib.cudaSetMemory(ctx.handle, m.value, 0, 4095, b"\1\2", 2) == cb.STATUS_BAD_PARAM          # size not a multiple of the pattern
+    assert lib.cudaSetMemory(ctx.handle, m.value, 0, 8192, None, 0) == cb.STATUS_BAD_PARAM             # beyond the block
+    cb.check(lib.cudaSetMemory(dflt, m.value, 100, 1000, None, 0), "zero")
+    host = np.empty(4096, dtype=np.uint8)
+    cb.check(lib.cudaCopyMemoryToHost(dflt, host.ctypes.data_as(C.c_void_p), m.value, 0, 4096), "d2h")
+    assert host[100:1100].sum() == 0 and host[99] != 0 and host[1100] != 0
+    # view + device-to-device copy
+    v = C.c_int64(0)
+    cb.check(lib.cudaCreateMemoryView(C.byref(v), m.value, 1024, 2048), "view")
+    assert lib.cudaCreateMemoryView(C.byref(C.c_int64(0)), v.value, 16, 0) == cb.STATUS_BAD_PARAM        # views of views are refused
+    assert lib.cudaCreateMemoryView(C.byref(C.c_int64(0)), m.value, 4096, 1) == cb.STATUS_BAD_PARAM
+    src = np.arange(1024, dtype=np.uint8)
+    cb.check(lib.cudaCopyMemoryFromHost(dflt, v.value, 0, src.ctypes.data_as(C.c_void_p), 1024), "h2d")
+    cb.check(lib.cudaCopyMemory(ctx.handle, m.value, 0, v.value, 0, 1024), "d2d")
+    ctx.synchronize()
+    cb.check(lib.cudaCopyMemoryToHost(dflt, host.ctypes.data_as(C.c_void_p), m.value, 0, 4096), "d2h")
+    np.testing.assert_array_equal(host[:1024], src)
+    np.testing.assert_array_equal(host[2048:3072], src)
+    ready = C.c_bool(False)
+    cb.check(lib.cudaIsContextReady(ctx.handle, C.byref(ready)), "ready")
+    assert ready.value
+    assert lib.cudaCopyMemoryToHost(dflt, None, m.value, 0, 4) == cb.STATUS_BAD_PARAM
+    cb.check(lib.cudaDestroyMemoryDescriptor(v.value), "free view")
+    cb.check(lib.cudaDestroyMemoryDescriptor(m.value), "free")
+    assert lib.cudaDestroyMemoryDescriptor(m.value) == cb.STATUS_BAD_PARAM
+    assert lib.cudaDestroyContextDescriptor(dflt) == cb.STATUS_BAD_PARAM                                # the default context cannot be destroyed
+    ctx.close()

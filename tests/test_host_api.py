@@ -1,0 +1,118 @@
+"""CPU-only checks of the boundary: the shared library loads without a GPU, exports every symbol the headers declare, and its
+host-side descriptor logic and argument validation behave as the reference's C API documents."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+import cudabackend_amd as cb
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"\b((?:cuda|avhip)[A-Za-z_0-9]+)\s*\(", text))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = cb.load_library()
+    api = declared_symbols("avocado_hip_backend.h")
+    kernels = declared_symbols("avocado_hip_kernels.h")
+    assert len(api) >= 40 and len(kernels) == 10
+    for name in sorted(api | kernels):
+        assert hasattr(lib, name), name
+    # the Python binding covers the whole API header
+    assert api == set(cb.api.PROTOTYPES)
+    assert kernels == set(cb.api.KERNEL_LAYER_SYMBOLS)
+
+
+def test_missing_library_is_an_error(tmp_path):
+    with pytest.raises(FileNotFoundError):
+        cb.load_library(str(tmp_path / "libavocado_hip.so"))
+
+
+def test_tensor_descriptor_roundtrip():
+    lib = cb.load_library()
+    d = C.c_int64(0)
+    cb.check(lib.cudaCreateTensorDescriptor(C.byref(d)))
+    dims = (C.c_int * 4)(12, 13, 14, 135)
+    cb.check(lib.cudaSetTensorDescriptor(d.value, cb.DTYPE_BFLOAT16, 4, dims))
+    dtype, nb, out = C.c_int(0), C.c_int(0), (C.c_int * 8)()
+    cb.check(lib.cudaGetTensorDescriptor(d.value, C.byref(dtype), C.byref(nb), out))
+    assert dtype.value == cb.DTYPE_BFLOAT16 and nb.value == 4 and list(out)[:4] == [12, 13, 14, 135]
+    assert lib.cudaSetTensorDescriptor(d.value, cb.DTYPE_FLOAT32, 9, dims) == cb.STATUS_BAD_PARAM      # more than 8 dimensions
+    assert lib.cudaSetTensorDescriptor(d.value, cb.DTYPE_FLOAT32, 2, None) == cb.STATUS_BAD_PARAM
+    cb.check(lib.cudaSetTensorDescriptor(d.value, cb.DTYPE_FLOAT32, 0, None))
+    cb.check(lib.cudaDestroyTensorDescriptor(d.value))
+    assert lib.cudaDestroyTensorDescriptor(d.value) == cb.STATUS_BAD_PARAM
+    assert lib.cudaGetTensorDescriptor(d.value, None, None, None) == cb.STATUS_BAD_PARAM
+    assert lib.cudaCreateTensorDescriptor(None) == cb.STATUS_BAD_PARAM
+
+
+def test_convolution_descriptor_defaults_and_roundtrip():
+    lib = cb.load_library()
+    d = C.c_int64(0)
+    cb.check(lib.cudaCreateConvolutionDescriptor(C.byref(d)))
+    # null arrays mean padding 0, stride 1, dilation 1 (reference header :758-762)
+    cb.check(lib.cudaSetConvolutionDescriptor(d.value, cb.CROSS_CORRELATION_MODE, 2, None, None, None, 1, None))
+    mode, nb, groups = C.c_int(0), C.c_int(0), C.c_int(0)
+    pad, st, dil = (C.c_int * 3)(9, 9, 9), (C.c_int * 3)(9, 9, 9), (C.c_int * 3)(9, 9, 9)
+    pv = C.create_string_buffer(16)
+    cb.check(lib.cudaGetConvolutionDescriptor(d.value, C.byref(mode), C.byref(nb), pad, st, dil, C.byref(groups), pv))
+    assert (mode.value, nb.value, groups.value) == (cb.CROSS_CORRELATION_MODE, 2, 1)
+    assert list(pad)[:2] == [0, 0] and list(st)[:2] == [1, 1] and list(dil)[:2] == [1, 1] and pv.raw == b"\0" * 16
+    value = C.create_string_buffer(bytes(range(16)), 16)
+    cb.check(lib.cudaSetConvolutionDescriptor(d.value, cb.CONVOLUTION_MODE, 2, (C.c_int * 2)(-1, -2), (C.c_int * 2)(2, 3), (C.c_int * 2)(1, 2), 1, value))
+    cb.check(lib.cudaGetConvolutionDescriptor(d.value, C.byref(mode), C.byref(nb), pad, st, dil, C.byref(groups), pv))
+    assert list(pad)[:2] == [-1, -2] and list(st)[:2] == [2, 3] and list(dil)[:2] == [1, 2] and pv.raw == bytes(range(16))
+    assert lib.cudaSetConvolutionDescriptor(d.value, cb.CONVOLUTION_MODE, 4, None, None, None, 1, None) == cb.STATUS_BAD_PARAM
+    assert lib.cudaSetConvolutionDescriptor(d.value, cb.CONVOLUTION_MODE, 2, None, None, None, 0, None) == cb.STATUS_BAD_PARAM
+    cb.check(lib.cudaDestroyConvolutionDescriptor(d.value))
+    assert lib.cudaDestroyConvolutionDescriptor(d.value) == cb.STATUS_BAD_PARAM
+
+
+def test_handles_are_typed():
+    lib = cb.load_library()
+    t = C.c_int64(0)
+    cb.check(lib.cudaCreateTensorDescriptor(C.byref(t)))
+    assert lib.cudaDestroyConvolutionDescriptor(t.value) == cb.STATUS_BAD_PARAM
+    assert lib.cudaDestroyMemoryDescriptor(t.value) == cb.STATUS_BAD_PARAM
+    assert lib.cudaDestroyContextDescriptor(t.value) == cb.STATUS_BAD_PARAM
+    assert lib.cudaSynchronizeWithContext(t.value) == cb.STATUS_BAD_PARAM
+    cb.check(lib.cudaDestroyTensorDescriptor(t.value))
+
+
+@pytest.mark.skipif(cb.load_library().cudaGetNumberOfDevices() > 0, reason="checks the no-GPU behaviour")
+def test_no_device_paths_fail_with_status_codes():
+    lib = cb.load_library()
+    assert lib.cudaGetNumberOfDevices() == 0
+    assert lib.cudaGetDefaultContext(0) == -1
+    h = C.c_int64(0)
+    assert lib.cudaCreateContextDescriptor(C.byref(h), 0) == cb.STATUS_BAD_PARAM
+    assert lib.cudaCreateMemoryDescriptor(C.byref(h), 0, 16) == cb.STATUS_BAD_PARAM
+    # a compute entry with an invalid context is refused before anything is launched
+    assert lib.cudaGemm(-1, 0, 0, None, 0, 0, 0, 0, None, 0, 0) == cb.STATUS_BAD_PARAM
+    assert lib.cudaConvolutionImplicitGemmForward(-1, 0, None, 0, 0, 0, 0, 0, 0, None, 0, 0, None, 0, 0, 0) == cb.STATUS_BAD_PARAM
+    buf = C.create_string_buffer(256)
+    assert lib.cudaGetDeviceProperty(0, cb.DEVICE_NAME, buf) == cb.STATUS_BAD_PARAM
+
+
+def test_page_lock_is_reported_as_not_supported():
+    lib = cb.load_library()
+    buf = C.create_string_buffer(64)
+    assert lib.cudaPageLock(None, 64) == cb.STATUS_BAD_PARAM
+    assert lib.cudaPageLock(buf, 64) == cb.STATUS_NOT_SUPPORTED
+    assert lib.cudaPageUnlock(buf) == cb.STATUS_NOT_SUPPORTED
+
+
+def test_copy_possible_only_within_one_device():
+    lib = cb.load_library()
+    r = C.c_bool(False)
+    cb.check(lib.cudaIsCopyPossible(0, 0, C.byref(r)))
+    assert r.value
+    cb.check(lib.cudaIsCopyPossible(0, 1, C.byref(r)))
+    assert not r.value
+    assert lib.cudaIsCopyPossible(0, 0, None) == cb.STATUS_BAD_PARAM
