@@ -1,0 +1,314 @@
+#!/usr/bin/env python3
+"""Benchmark of the convolution hot path on one MI355X.
+
+Workload (BASELINE config 2): residual tower, NHWC, N=256, 15x15, 128 channels: stem 3x3 conv 4->128, then 10 blocks of
+[3x3 conv + bias + ReLU, 3x3 conv + bias + residual + ReLU] = 21 convolutions per step, every one a call of
+cudaConvolutionBiasActivationForward.  Synthetic seeded data: inputs are 4 planes of Bernoulli(0.15) ones, weights He-normal,
+biases U(-0.1, 0.1).  All tensors are resident in HBM before the timed region; the timed region is bracketed by HIP events on
+the context's stream and by device synchronisation.
+
+Prints ONE JSON line.  `value` is direct-convolution-equivalent TFLOP/s (2*N*Ho*Wo*K*C*R*S per convolution) of the whole tower
+in the headline dtype (bf16).  `roofline` is for the dominant kernel (the 128->128 body convolution), its duration measured
+with HIP events around each of its launches inside the timed region.  `cpu_baseline` is the restated CPU direct convolution
+(oracle/cpu_baseline.c, "port") timed on the host cores on a batch slice of the same body convolution.  `detail` carries the
+other dtypes and the per-stage figures of the non-fused Winograd path.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import cudabackend_amd as cb  # noqa: E402
+
+PEAK = {"hbm_GBs": 8000.0, "bf16": 2500.0, "f16": 2500.0, "i8": 5000.0, "f32": 157.3}
+DT = {"bf16": cb.DTYPE_BFLOAT16, "f16": cb.DTYPE_FLOAT16, "f32": cb.DTYPE_FLOAT32, "i8": cb.DTYPE_INT8}
+SEED = 0xA70CAD0
+
+
+class Hip:
+    """The few HIP runtime calls the harness needs itself: events on a given stream."""
+
+    def __init__(self):
+        self.rt = C.CDLL("libamdhip64.so")
+        self.rt.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.rt.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.rt.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.rt.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.rt.hipEventDestroy.argtypes = [C.c_void_p]
+
+    def event(self):
+        e = C.c_void_p()
+        assert self.rt.hipEventCreate(C.byref(e)) == 0
+        return e
+
+    def record(self, e, stream):
+        assert self.rt.hipEventRecord(e, stream) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.rt.hipEventSynchronize(b) == 0
+        ms = C.c_float(0)
+        assert self.rt.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return float(ms.value)
+
+    def sync(self):
+        assert self.rt.hipDeviceSynchronize() == 0
+
+
+def conv_flops(N, Ho, Wo, K, Cin, R, S):
+    return 2.0 * N * Ho * Wo * K * Cin * R * S
+
+
+class Tower:
+    """Config 2.  Holds every tensor on the device; step() enqueues the 21 convolutions of one forward pass."""
+
+    def __init__(self, ctx, dtype, N=256, HW=15, ch=128, blocks=10, planes=4):
+        self.ctx, self.lib, self.dtype = ctx, cb.load_library(), dtype
+        self.N, self.HW, self.ch, self.blocks, self.planes = N, HW, ch, blocks, planes
+        g = np.random.default_rng(SEED + 2)
+        d = DT[dtype]
+        x0 = (g.random((N, HW, HW, planes)) < 0.15).astype(np.float32)
+        self.x0 = cb.DeviceTensor.from_numpy(x0, d)
+        self.conv = cb.ConvolutionDescriptor(padding=(-1, -1), dtype=d)
+        self.layers = []
+        cin = planes
+        for _ in range(1 + 2 * blocks):
+            w = g.standard_normal((ch, 3, 3, cin)).astype(np.float32) * np.float32(np.sqrt(2.0 / (9 * cin)))
+            b = g.uniform(-0.1, 0.1, ch).astype(np.float32)
+            self.layers.append((cb.DeviceTensor.from_numpy(w, d), cb.DeviceTensor.from_numpy(b, cb.DTYPE_FLOAT32)))
+            cin = ch
+        self.act = [cb.DeviceTensor((N, HW, HW, ch), d) for _ in range(3)]
+        need = C.c_int64(0)
+        cb.check(self.lib.cudaGetConvolutionWorkspaceSize(ctx.handle, self.conv.handle, self.act[0].desc, self.layers[1][0].desc, self.layers[1][1].desc,
+                                                          C.byref(need)), "cudaGetConvolutionWorkspaceSize")
+        self.workspace = cb.DeviceTensor((max(int(need.value), 256),), cb.DTYPE_UINT8)
+        self.workspace_bytes = int(need.value)
+        self.flops_body = conv_flops(N, HW, HW, ch, ch, 3, 3)
+        self.flops_step = conv_flops(N, HW, HW, ch, planes, 3, 3) + 2 * blocks * self.flops_body
+
+    def _conv(self, x, layer, z, y):
+        w, b = self.layers[layer]
+        st = self.lib.cudaConvolutionBiasActivationForward(self.ctx.handle, self.conv.handle, None, x.desc, x.mem, w.desc, w.mem, b.desc, b.mem, None,
+                                                           z.desc if z is not None else 0, z.mem if z is not None else 0, None, y.desc, y.mem,
+                                                           cb.ACTIVATION_RELU, self.workspace.mem)
+        cb.check(st, "cudaConvolutionBiasActivationForward")
+
+    def step(self, hip=None, stream=None, marks=None):
+        a, t, b = self.act
+        self._conv(self.x0, 0, None, a)
+        layer = 1
+        for _ in range(self.blocks):
+            for (src, z, dst) in ((a, None, t), (t, a, b)):
+                if marks is not None:
+                    e0, e1 = hip.event(), hip.event()
+                    hip.record(e0, stream)
+                self._conv(src, layer, z, dst)
+                if marks is not None:
+                    hip.record(e1, stream)
+                    marks.append((e0, e1))
+                layer += 1
+            a, b = b, a
+        return a
+
+    def close(self):
+        for t in [self.x0, self.workspace] + self.act + [t for pair in self.layers for t in pair]:
+            t.close()
+
+
+def time_tower(hip, ctx, dtype, steps, warmup):
+    tower = Tower(ctx, dtype)
+    stream = ctx.stream()
+    for _ in range(warmup):
+        tower.step()
+    ctx.synchronize()
+    hip.sync()
+    marks = []
+    e0, e1 = hip.event(), hip.event()
+    hip.record(e0, stream)
+    for _ in range(steps):
+        tower.step(hip, stream, marks)
+    hip.record(e1, stream)
+    ctx.synchronize()
+    hip.sync()
+    total_ms = hip.elapsed_ms(e0, e1)
+    body_ms = [hip.elapsed_ms(a, b) for a, b in marks]
+    out = {"ms_per_step": total_ms / steps, "tflops": tower.flops_step * steps / (total_ms * 1e-3) / 1e12,
+           "body_conv_us": 1e3 * float(np.mean(body_ms)), "body_conv_tflops": tower.flops_body / (np.mean(body_ms) * 1e-3) / 1e12,
+           "workspace_bytes": tower.workspace_bytes}
+    tower.close()
+    return out
+
+
+def time_calls(hip, ctx, fn, iters, warmup=3):
+    stream = ctx.stream()
+    for _ in range(warmup):
+        fn()
+    ctx.synchronize()
+    e0, e1 = hip.event(), hip.event()
+    hip.record(e0, stream)
+    for _ in range(iters):
+        fn()
+    hip.record(e1, stream)
+    ctx.synchronize()
+    return hip.elapsed_ms(e0, e1) / iters
+
+
+def int8_leg(hip, ctx, iters):
+    """Config 4: int8 x int8 -> int32, N=128, 20x20, 128->128, 3x3 offset -1 and 1x1."""
+    lib = cb.load_library()
+    g = np.random.default_rng(SEED + 4)
+    out = {}
+    x = cb.DeviceTensor.from_numpy(g.integers(-127, 128, (128, 20, 20, 128), dtype=np.int8), cb.DTYPE_INT8)
+    b = cb.DeviceTensor.from_numpy(g.integers(-2 ** 15, 2 ** 15, 128).astype(np.int32), cb.DTYPE_INT32)
+    y = cb.DeviceTensor((128, 20, 20, 128), cb.DTYPE_INT32)
+    for r, pad in ((3, -1), (1, 0)):
+        w = cb.DeviceTensor.from_numpy(g.integers(-127, 128, (128, r, r, 128), dtype=np.int8), cb.DTYPE_INT8)
+        conv = cb.ConvolutionDescriptor(padding=(pad, pad), dtype=cb.DTYPE_INT8)
+
+        def call():
+            cb.check(lib.cudaConvolutionImplicitGemmForward(ctx.handle, conv.handle, None, x.desc, x.mem, w.desc, w.mem, b.desc, b.mem, None, 0, 0, None,
+                                                            y.desc, y.mem, cb.ACTIVATION_LINEAR), "int8 conv")
+        ms = time_calls(hip, ctx, call, iters)
+        out["%dx%d" % (r, r)] = {"us": ms * 1e3, "tops": conv_flops(128, 20, 20, 128, 128, r, r) / (ms * 1e-3) / 1e12}
+        w.close()
+    for t in (x, b, y):
+        t.close()
+    return out
+
+
+def nonfused_stages(hip, ctx, dtype, mat_dtype, m, iters):
+    """The four-call non-fused Winograd sequence on the body convolution of config 2, one timing per stage."""
+    lib = cb.load_library()
+    g = np.random.default_rng(SEED + 5)
+    N, HW, ch = 256, 15, 128
+    d, md = DT[dtype], DT[mat_dtype]
+    t = m + 2
+    tiles = N * ((HW + m - 1) // m) ** 2
+    esz, msz = cb.DTYPE_SIZE[d], cb.DTYPE_SIZE[md]
+    x = cb.DeviceTensor.from_numpy(g.standard_normal((N, HW, HW, ch)).astype(np.float32), d)
+    w = cb.DeviceTensor.from_numpy((g.standard_normal((ch, 3, 3, ch)) * np.sqrt(2.0 / (9 * ch))).astype(np.float32), d)
+    b = cb.DeviceTensor.from_numpy(g.uniform(-0.1, 0.1, ch).astype(np.float32), cb.DTYPE_FLOAT32)
+    U = cb.DeviceTensor((t * t, ch, ch), md)
+    V = cb.DeviceTensor((t * t, tiles, ch), md)
+    acc_dtype = cb.DTYPE_FLOAT32
+    Mx = cb.DeviceTensor((t * t, tiles, ch), acc_dtype)
+    y = cb.DeviceTensor((N, HW, HW, ch), d)
+    conv = cb.ConvolutionDescriptor(padding=(-1, -1), dtype=d)
+    h = ctx.handle
+    calls = {
+        "weight_transform": lambda: cb.check(lib.cudaWinogradWeightTransform(h, conv.handle, m, w.desc, w.mem, U.desc, U.mem), "weight"),
+        "input_transform": lambda: cb.check(lib.cudaWinogradInputTransform(h, conv.handle, m, w.desc, x.desc, x.mem, V.desc, V.mem), "input"),
+        "gemm": lambda: cb.check(lib.cudaGemmBatched(h, 0, 1, None, V.desc, V.mem, U.desc, U.mem, None, Mx.desc, Mx.mem), "gemm"),
+        "output_transform": lambda: cb.check(lib.cudaWinogradOutputTransform(h, conv.handle, m, w.desc, None, Mx.desc, Mx.mem, y.desc, y.mem, b.desc, b.mem,
+                                                                          None, 0, 0, None, cb.ACTIVATION_RELU), "output"),
+    }
+    xbytes = N * HW * HW * ch * esz
+    alg_bytes = {"weight_transform": ch * 9 * ch * esz + t * t * ch * ch * msz, "input_transform": xbytes + t * t * tiles * ch * msz,
+                 "gemm": t * t * tiles * ch * msz + t * t * ch * ch * msz + t * t * tiles * ch * 4, "output_transform": t * t * tiles * ch * 4 + xbytes + 4 * ch}
+    gemm_flops = 2.0 * t * t * tiles * ch * ch
+    out = {}
+    total = 0.0
+    for name, fn in calls.items():
+        ms = time_calls(hip, ctx, fn, iters)
+        rec = {"us": ms * 1e3, "GBs": alg_bytes[name] / (ms * 1e-3) / 1e9, "hbm_frac": alg_bytes[name] / (ms * 1e-3) / 1e9 / PEAK["hbm_GBs"]}
+        if name == "gemm":
+            rec["tflops"] = gemm_flops / (ms * 1e-3) / 1e12
+            rec["mfma_frac"] = rec["tflops"] / PEAK[mat_dtype]
+        out[name] = rec
+        if name != "weight_transform":
+            total += ms
+    out["conv_tflops_direct_equivalent"] = conv_flops(N, HW, HW, ch, ch, 3, 3) / (total * 1e-3) / 1e12
+    for tns in (x, w, b, U, V, Mx, y):
+        tns.close()
+    return out
+
+
+def copy_bandwidth(hip, ctx, iters=10):
+    lib = cb.load_library()
+    nbytes = 1 << 30
+    a, b = cb.DeviceTensor((nbytes,), cb.DTYPE_UINT8), cb.DeviceTensor((nbytes,), cb.DTYPE_UINT8)
+    ms = time_calls(hip, ctx, lambda: cb.check(lib.cudaCopyMemory(ctx.handle, b.mem, 0, a.mem, 0, nbytes), "copy"), iters)
+    a.close()
+    b.close()
+    return 2.0 * nbytes / (ms * 1e-3) / 1e9
+
+
+def cpu_baseline(seconds=12.0):
+    """fp32 direct convolution of the body layer (128->128, 15x15, 3x3) on a batch slice, all host cores."""
+    from oracle import oracle as orc
+    g = np.random.default_rng(SEED + 6)
+    n = 32
+    x = g.standard_normal((n, 15, 15, 128)).astype(np.float32)
+    w = (g.standard_normal((128, 3, 3, 128)) * np.sqrt(2.0 / (9 * 128))).astype(np.float32)
+    b = g.uniform(-0.1, 0.1, 128).astype(np.float32)
+    orc.baseline_conv2d_f32(x, w, b)  # warm the threads and the caches
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < seconds:
+        orc.baseline_conv2d_f32(x, w, b)
+        reps += 1
+    dt = time.perf_counter() - t0
+    flops = conv_flops(n, 15, 15, 128, 128, 3, 3) * reps
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": orc.baseline_threads(), "kind": "port",
+            "sample": "fp32 3x3 conv 128->128 15x15, batch slice N=%d of 256, %d repetitions in %.1f s (restated CPU reference, not AvocadoML/CpuBackend)"
+                      % (n, reps, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
+    ap.add_argument("--quick", action="store_true", help="headline tower only (no side legs, no CPU baseline)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards over the batch with no collectives)." % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    lib = cb.load_library()
+    if lib.cudaGetNumberOfDevices() < 1:
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    hip = Hip()
+    ctx = cb.Context(0)
+    head = time_tower(hip, ctx, args.dtype, args.steps, args.warmup)
+    detail = {"headline": head}
+    cpu = None
+    if not args.quick:
+        it = max(5, args.steps)
+        for other in ("f32", "bf16", "f16"):
+            if other != args.dtype:
+                detail["tower_" + other] = time_tower(hip, ctx, other, max(3, args.steps // 2), 2)
+        detail["int8_config4"] = int8_leg(hip, ctx, it)
+        detail["nonfused_winograd_f32_F4"] = nonfused_stages(hip, ctx, "f32", "f32", 4, it)
+        detail["nonfused_winograd_bf16_F2_fp16mat"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it)
+        detail["copy_GBs_measured"] = copy_bandwidth(hip, ctx)
+        if "tower_bf16" in detail or args.dtype == "bf16":
+            bf = head if args.dtype == "bf16" else detail["tower_bf16"]
+            detail["int8_over_bf16_throughput"] = detail["int8_config4"]["3x3"]["tops"] / bf["body_conv_tflops"]
+        cpu = cpu_baseline()
+    ctx.close()
+    peak = PEAK[args.dtype]
+    line = {
+        "metric": "3x3 conv TFLOP/s + % MFMA/HBM roofline at N=256,15x15,128ch; int8 TOPS",
+        "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "BASELINE config 2: residual tower N=256 15x15 128ch, stem 4->128 + 10 blocks (21 3x3 convs), NHWC, bias+ReLU+residual fused",
+                   "global_batch": 256, "entry": "cudaConvolutionBiasActivationForward"},
+        "roofline": {"bound": "mfma", "achieved": head["body_conv_tflops"], "peak": peak, "unit": "TFLOP/s", "frac": head["body_conv_tflops"] / peak,
+                     "traffic": None, "kernel": "body 3x3 conv 128->128 (direct-equivalent flops / HIP-event duration per launch)"},
+        "cpu_baseline": cpu,
+        "detail": detail,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1397,9 +1397,16 @@ namespace avocado
 			const Tensor *x = get_tensor(xDesc), *w = get_tensor(wDesc);
 			if (conv == nullptr || x == nullptr || w == nullptr || x->nb_dims != 4 || w->nb_dims != 4)
 				return AVOCADO_STATUS_BAD_PARAM;
-			/* the output of the only algorithm that needs a workspace has the spatial size of the input */
+			/* output extent of a convolution whose offset padding is mirrored at the far edge */
 			Tensor y = *x;
 			y.dim[3] = w->dim[0];
+			for (int i = 0; i < 2; i++)
+			{
+				const int extent = (w->dim[1 + i] - 1) * conv->dilation[i] + 1;
+				if (conv->strides[i] <= 0 || conv->dilation[i] <= 0)
+					return AVOCADO_STATUS_BAD_PARAM;
+				y.dim[1 + i] = (x->dim[1 + i] - 2 * conv->padding[i] - extent) / conv->strides[i] + 1;
+			}
 			ConvProblem p;
 			const avStatus_t st = make_problem(conv, x, w, &y, p);
 			if (st != AVOCADO_STATUS_SUCCESS)

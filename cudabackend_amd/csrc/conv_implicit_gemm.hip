@@ -172,6 +172,11 @@ namespace
 		I8_FLOAT_F32 /* float epilogue, y fp32                                           */
 	};
 
+	/* From here on every fp32 operation must round exactly once: the float epilogue on integer sums is specified step by
+	 * step (multiply, add, multiply, add), so a*b + c must not be contracted into a fused multiply-add.  The pragma only
+	 * governs expressions written below it, which is why the epilogue uses plain operators and no header intrinsics. */
+#pragma clang fp contract(off)
+
 	template<int MODE>
 	__global__ __launch_bounds__(256) void k_conv_igemm_int8(const int8_t *__restrict__ x, const int8_t *__restrict__ w, const void *__restrict__ bias,
 			const void *z, void *y, const float *__restrict__ scale, ConvGeom g, int8_t padv, int vec_ok, float alpha1, float alpha2, float beta, int activation)
@@ -221,7 +226,7 @@ namespace
 					int8_t o[4];
 #pragma unroll
 					for (int q = 0; q < 4; q++)
-						o[q] = static_cast<int8_t>(round_saturate(__fmul_rn(static_cast<float>(t[q]), q < valid ? scale[k + q] : 0.0f), -128.0f, 127.0f));
+						o[q] = static_cast<int8_t>(round_saturate(static_cast<float>(t[q]) * (q < valid ? scale[k + q] : 0.0f), -128.0f, 127.0f));
 					int8_t *dst = static_cast<int8_t*>(y) + idx;
 					if (vec_y && valid >= 4)
 						*reinterpret_cast<char4*>(dst) = make_char4(o[0], o[1], o[2], o[3]);
@@ -241,21 +246,21 @@ namespace
 				{
 					if (q >= valid)
 						continue;
-					float t = __fmul_rn(alpha1, static_cast<float>(v[q]));
+					float t = alpha1 * static_cast<float>(v[q]);
 					if (bias != nullptr)
-						t = __fadd_rn(t, static_cast<const float*>(bias)[k + q]);
+						t = t + static_cast<const float*>(bias)[k + q];
 					if (z != nullptr)
 					{
 						const float zv = MODE == I8_FLOAT_I32 ? static_cast<float>(static_cast<const int*>(z)[idx + q]) :
 											MODE == I8_FLOAT_I8 ? static_cast<float>(static_cast<const int8_t*>(z)[idx + q]) : static_cast<const float*>(z)[idx + q];
-						t = __fadd_rn(t, __fmul_rn(alpha2, zv));
+						t = t + alpha2 * zv;
 					}
 					t = activation_forward<float>(activation, t);
 					if (beta != 0.0f)
 					{
 						const float yv = MODE == I8_FLOAT_I32 ? static_cast<float>(static_cast<int*>(y)[idx + q]) :
 											MODE == I8_FLOAT_I8 ? static_cast<float>(static_cast<int8_t*>(y)[idx + q]) : static_cast<float*>(y)[idx + q];
-						t = __fadd_rn(t, __fmul_rn(beta, yv));
+						t = t + beta * yv;
 					}
 					if (MODE == I8_FLOAT_I32)
 						static_cast<int*>(y)[idx + q] = round_saturate(t, -2147483648.0f, 2147483520.0f);
