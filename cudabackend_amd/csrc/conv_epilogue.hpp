@@ -1,0 +1,223 @@
+/*
+ * conv_epilogue.hpp -- what happens to a convolution accumulator on its way to y, shared by the implicit-GEMM kernels.
+ *
+ *   y = activation(alpha1 * conv + bias[k] + alpha2 * z) + beta * y
+ * in the operation order of the reference's epilogue (src/winograd_nonfused.cu:407-417 of the reference): scale, add bias,
+ * add the scaled residual, activate, add the scaled old output, store.  The MFMA engine hands every work-item four
+ * consecutive output filters of one output pixel at a time; the per-filter constants of those four columns (bias, requant
+ * scale) never change for a work-item, so they are loaded once, before the k loop, and not in the store loop.
+ */
+#ifndef AVHIP_CONV_EPILOGUE_HPP_
+#define AVHIP_CONV_EPILOGUE_HPP_
+
+#include "common.hpp"
+
+namespace avhip
+{
+	/* How a kernel instance treats the activation.  ACT_SIMPLE instances are launched only for LINEAR and RELU and pay one
+	 * compare and one select per element; ACT_ANY instances switch over all nine functions.  The split is made on the host,
+	 * per launch: a per-element switch in one kernel would make the compiler evaluate every transcendental and select. */
+	constexpr int ACT_SIMPLE = -2;
+	constexpr int ACT_ANY = -1;
+	__host__ inline bool is_simple_activation(int activation)
+	{
+		return activation == ACT_LINEAR || activation == ACT_RELU;
+	}
+	template<int ACT, typename CT>
+	__device__ __forceinline__ CT activate(int activation, CT x)
+	{
+		if (ACT == ACT_SIMPLE)
+			return (activation == ACT_RELU && x < static_cast<CT>(0)) ? static_cast<CT>(0) : x;
+		return activation_forward<CT>(activation, x);
+	}
+
+	__device__ inline int round_saturate(float v, float lo, float hi)
+	{
+		if (!(v == v))
+			return 0;
+		float r = rintf(v);
+		r = r < lo ? lo : r;
+		r = r > hi ? hi : r;
+		return static_cast<int>(r);
+	}
+
+	/* Floating tensors: TE in, TE out, fp32 bias, fp32 arithmetic, one round-to-nearest-even on store. */
+	template<typename TE>
+	struct FloatEpilogue
+	{
+		typedef float scalar_t;
+		struct Columns
+		{
+			float bias[4];
+		};
+		const float *bias;
+		const TE *z;
+		TE *y;
+		float alpha1, alpha2, beta;
+		int activation, K;
+		bool vec; /* y / z rows may be accessed as 4-element vectors */
+
+		__device__ __forceinline__ void load_columns(int k, Columns &c) const
+		{
+#pragma unroll
+			for (int q = 0; q < 4; q++)
+				c.bias[q] = (bias != nullptr && k + q < K) ? bias[k + q] : 0.0f;
+		}
+		/* p: index of the output pixel (row of y), k: first of the four filters */
+		template<int ACT>
+		__device__ __forceinline__ void store(int64_t p, int k, const float (&v)[4], const Columns &c) const
+		{
+			const int valid = K - k;
+			const int64_t idx = p * K + k;
+			float t[4];
+#pragma unroll
+			for (int q = 0; q < 4; q++)
+				t[q] = alpha1 * v[q] + c.bias[q];
+			if (z != nullptr)
+			{
+				float zv[4];
+				load_vec<TE, 4, float>(z + idx, valid, zv, vec);
+#pragma unroll
+				for (int q = 0; q < 4; q++)
+					t[q] += alpha2 * zv[q];
+			}
+#pragma unroll
+			for (int q = 0; q < 4; q++)
+				t[q] = activate<ACT, float>(activation, t[q]);
+			if (beta != 0.0f)
+			{
+				float yv[4];
+				load_vec<TE, 4, float>(y + idx, valid, yv, vec);
+#pragma unroll
+				for (int q = 0; q < 4; q++)
+					t[q] += beta * yv[q];
+			}
+			store_vec<TE, 4, float>(y + idx, valid, t, vec);
+		}
+	};
+
+	enum Int8Mode
+	{
+		I8_EXACT = 0, /* y int32 = act(sum + bias_i32)                                   */
+		I8_REQUANT, /* y int8  = sat(rne(float(act(sum + bias_i32)) * scale[k]))        */
+		I8_FLOAT_I32, /* float epilogue, y int32                                         */
+		I8_FLOAT_I8, /* float epilogue, y int8                                           */
+		I8_FLOAT_F32 /* float epilogue, y fp32                                           */
+	};
+
+	/* int8 x int8 -> int32 sums.  EXACT and REQUANT add an int32 bias in integer arithmetic; the FLOAT modes follow the
+	 * header's convention for integer tensors: cast to fp32, scale and add in fp32 (every step rounded once, no fused
+	 * multiply-add), cast back with round-to-nearest-even and saturation. */
+	template<int MODE>
+	struct Int8Epilogue
+	{
+		typedef int scalar_t;
+		struct Columns
+		{
+			int ibias[4];
+			float fbias[4];
+			float scale[4];
+		};
+		const void *bias, *z;
+		void *y;
+		const float *scale;
+		float alpha1, alpha2, beta;
+		int activation, K;
+		bool vec;
+
+		__device__ __forceinline__ void load_columns(int k, Columns &c) const
+		{
+#pragma unroll
+			for (int q = 0; q < 4; q++)
+			{
+				const bool in = k + q < K;
+				c.ibias[q] = (MODE <= I8_REQUANT && bias != nullptr && in) ? static_cast<const int*>(bias)[k + q] : 0;
+				c.fbias[q] = (MODE > I8_REQUANT && bias != nullptr && in) ? static_cast<const float*>(bias)[k + q] : 0.0f;
+				c.scale[q] = (MODE == I8_REQUANT && in) ? scale[k + q] : 0.0f;
+			}
+		}
+		template<int ACT>
+		__device__ __forceinline__ void store(int64_t p, int k, const int (&v)[4], const Columns &c) const
+		{
+			/* every fp32 operation below rounds exactly once: a * b + c must not become a fused multiply-add.  The pragma
+			 * governs the expressions written in this block, which is why they use plain operators and no intrinsics. */
+#pragma clang fp contract(off)
+			const int valid = K - k;
+			const int64_t idx = p * K + k;
+			if (MODE == I8_EXACT || MODE == I8_REQUANT)
+			{
+				int t[4];
+#pragma unroll
+				for (int q = 0; q < 4; q++)
+				{
+					t[q] = v[q] + c.ibias[q];
+					if (activation == ACT_RELU && t[q] < 0)
+						t[q] = 0;
+				}
+				if (MODE == I8_EXACT)
+				{
+					int *dst = static_cast<int*>(y) + idx;
+					if (vec && valid >= 4)
+						*reinterpret_cast<int4*>(dst) = make_int4(t[0], t[1], t[2], t[3]);
+					else
+					{
+#pragma unroll
+						for (int q = 0; q < 4; q++)
+							if (q < valid)
+								dst[q] = t[q];
+					}
+				}
+				else
+				{
+					int8_t o[4];
+#pragma unroll
+					for (int q = 0; q < 4; q++)
+						o[q] = static_cast<int8_t>(round_saturate(static_cast<float>(t[q]) * c.scale[q], -128.0f, 127.0f));
+					int8_t *dst = static_cast<int8_t*>(y) + idx;
+					if (vec && valid >= 4)
+						*reinterpret_cast<char4*>(dst) = make_char4(o[0], o[1], o[2], o[3]);
+					else
+					{
+#pragma unroll
+						for (int q = 0; q < 4; q++)
+							if (q < valid)
+								dst[q] = o[q];
+					}
+				}
+			}
+			else
+			{
+#pragma unroll
+				for (int q = 0; q < 4; q++)
+				{
+					if (q >= valid)
+						continue;
+					float t = alpha1 * static_cast<float>(v[q]);
+					if (bias != nullptr)
+						t = t + c.fbias[q];
+					if (z != nullptr)
+					{
+						const float zv = MODE == I8_FLOAT_I32 ? static_cast<float>(static_cast<const int*>(z)[idx + q]) :
+											MODE == I8_FLOAT_I8 ? static_cast<float>(static_cast<const int8_t*>(z)[idx + q]) : static_cast<const float*>(z)[idx + q];
+						t = t + alpha2 * zv;
+					}
+					t = activate<ACT, float>(activation, t);
+					if (beta != 0.0f)
+					{
+						const float yv = MODE == I8_FLOAT_I32 ? static_cast<float>(static_cast<int*>(y)[idx + q]) :
+											MODE == I8_FLOAT_I8 ? static_cast<float>(static_cast<int8_t*>(y)[idx + q]) : static_cast<float*>(y)[idx + q];
+						t = t + beta * yv;
+					}
+					if (MODE == I8_FLOAT_I32)
+						static_cast<int*>(y)[idx + q] = round_saturate(t, -2147483648.0f, 2147483520.0f);
+					else if (MODE == I8_FLOAT_I8)
+						static_cast<int8_t*>(y)[idx + q] = static_cast<int8_t>(round_saturate(t, -128.0f, 127.0f));
+					else
+						static_cast<float*>(y)[idx + q] = t;
+				}
+			}
+		}
+	};
+}
+
+#endif /* AVHIP_CONV_EPILOGUE_HPP_ */

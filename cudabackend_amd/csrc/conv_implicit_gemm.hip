@@ -6,7 +6,7 @@
  * Here the convolution descriptor is honoured: any R x S, signed offsets, stride, dilation, both modes, any padding value.
  *
  * GEMM view: rows = output pixels (n, oh, ow) in NHWC order, columns = output filters, k = (tap, input channel).
- * Both operands are contiguous along the channel part of k, so a 64-byte k-step is a run of channels of one tap:
+ * Both operands are contiguous along the channel part of k, so a 128-byte k-step is a run of channels of one tap:
  *   A chunk = 16 bytes of x[n, ih, iw, c..]   (or the padding value outside the image),
  *   B chunk = 16 bytes of w[k, i, j, c..],
  * fetched straight from global memory (L2 serves the 9-fold tap reuse) into the shared MFMA engine.  Channel counts that
@@ -17,6 +17,10 @@
  *   int8 requantised : y = sat_i8(rne(float(sum + bias) * scale[k])), each step a single fp32 rounding;
  *   int8 with float scalars: the header's convention (cast to fp32, scale, cast back with rounding and saturation).
  */
+#include <cstring>
+
+#include "conv_epilogue.hpp"
+#include "conv_tile.hpp"
 #include "mfma_core.hpp"
 
 namespace
@@ -30,26 +34,49 @@ namespace
 		int flip; /* cross-correlation mode: tap (i, j) reads the input at (R-1-i, S-1-j) */
 		int steps_per_tap;
 		int64_t pixels; /* N * Ho * Wo */
+		int64_t images; /* N */
 	};
 
-	template<typename TE>
+	/* Walks k = (tap, channel slice) in order; shared by both operand loaders. */
+	struct TapCursor
+	{
+		int i = 0, j = 0, slice = 0, tap = 0;
+		__device__ inline void advance(const ConvGeom &g)
+		{
+			if (++slice == g.steps_per_tap)
+			{
+				slice = 0;
+				tap++;
+				if (++j == g.S)
+				{
+					j = 0;
+					i++;
+				}
+			}
+		}
+	};
+
+	/* Rows of A are output pixels; a chunk is 16 bytes of channels of the input pixel that tap (i, j) reads.
+	 * General form: any alignment, any channel count, any padding value. */
+	template<typename TE, bool FAST>
 	struct PixelLoader
 	{
 		const TE *x;
 		const ConvGeom &g;
 		TE padv;
 		bool vec_ok;
-		int ih0[2], iw0[2];
-		int64_t img[2]; /* pixel index of (n, 0, 0) */
-		bool ok[2];
+		TapCursor cur;
+		int ih0[FETCH_PASSES], iw0[FETCH_PASSES];
+		int64_t img[FETCH_PASSES]; /* pixel index of (n, 0, 0) */
+		bool ok[FETCH_PASSES];
 
-		__device__ inline PixelLoader(const TE *x_, const ConvGeom &g_, TE padv_, bool vec_ok_, int64_t p0, int frow) :
+		__device__ inline PixelLoader(const TE *x_, const ConvGeom &g_, TE padv_, bool vec_ok_, int64_t p0) :
 				x(x_), g(g_), padv(padv_), vec_ok(vec_ok_)
 		{
 #pragma unroll
-			for (int q = 0; q < 2; q++)
+			for (int q = 0; q < FETCH_PASSES; q++)
 			{
-				const int64_t p = p0 + frow + 64 * q;
+				const int64_t p = p0 + threadIdx.x / STEP_CHUNKS + FETCH_ROWS * q;
 				ok[q] = p < g.pixels;
 				const int64_t pp = ok[q] ? p : 0;
 				const int ow = static_cast<int>(pp % g.Wo);
@@ -60,21 +87,15 @@ namespace
 				img[q] = n * g.H * g.W;
 			}
 		}
-		__device__ inline uint4 operator()(int step, int q, int part) const
+		__device__ inline uint4 load(int q, int part) const
 		{
 			constexpr int E = 16 / sizeof(TE);
 			constexpr int KE = STEP_BYTES / sizeof(TE);
-			if (!ok[q])
+			if (!ok[q] || cur.i >= g.R)
 				return make_uint4(0u, 0u, 0u, 0u);
-			const int tap = step / g.steps_per_tap;
-			const int c = (step - tap * g.steps_per_tap) * KE + part * E;
-			int i = tap / g.S;
-			int j = tap - i * g.S;
-			if (g.flip)
-			{
-				i = g.R - 1 - i;
-				j = g.S - 1 - j;
-			}
+			const int c = cur.slice * KE + part * E;
+			const int i = g.flip ? g.R - 1 - cur.i : cur.i;
+			const int j = g.flip ? g.S - 1 - cur.j : cur.j;
 			const int ih = ih0[q] + i * g.dil_h;
 			const int iw = iw0[q] + j * g.dil_w;
 			const int valid = g.C - c;
@@ -82,194 +103,174 @@ namespace
 				return fetch_chunk<TE>(x + (img[q] + static_cast<int64_t>(ih) * g.W + iw) * g.C + c, valid, vec_ok);
 			return splat_chunk<TE>(padv, valid);
 		}
+		__device__ inline void next()
+		{
+			cur.advance(g);
+		}
 	};
-
+	/*
+	 * Fast form: x 16-byte aligned and below 2 GiB, C a multiple of the chunk, zero padding value, at most 32 taps.
+	 * Everything that depends on the output pixel is computed once per work-item: the byte offset of the window origin
+	 * (with this work-item's chunk already added) and a bit mask of the taps that fall inside the image.  Everything that
+	 * depends on the k-slice is uniform and lives in scalar registers.  A chunk then costs one add, one bit test and one
+	 * select before its branch-free buffer load, whose offset is OUT_OF_RANGE (hardware returns zeros) when it does not exist.
+	 */
 	template<typename TE>
-	struct FilterLoader
+	struct PixelLoader<TE, true>
 	{
-		const TE *w;
+		__amdgpu_buffer_rsrc_t rsrc;
 		const ConvGeom &g;
-		bool vec_ok;
-		int k0;
-		__device__ inline uint4 operator()(int step, int q, int part) const
+		TapCursor cur;
+		unsigned int origin[FETCH_PASSES]; /* byte offset of (n, ih0, iw0, chunk channel); may wrap below zero, never used then */
+		unsigned int inside[FETCH_PASSES]; /* bit t: tap t reads a pixel inside the image */
+		int chunk_channel; /* first channel of this work-item's chunk within a k-slice */
+		unsigned int tap_bytes; /* uniform: offset of the current tap and slice relative to the window origin */
+
+		__device__ inline PixelLoader(const TE *x, const ConvGeom &g_, TE, bool, int64_t p0) :
+				g(g_)
 		{
 			constexpr int E = 16 / sizeof(TE);
+			rsrc = make_buffer(x, static_cast<unsigned int>(g.images * g.H * g.W * g.C * sizeof(TE)));
+			chunk_channel = (threadIdx.x % STEP_CHUNKS) * E;
+#pragma unroll
+			for (int q = 0; q < FETCH_PASSES; q++)
+			{
+				/* the tensor is below 2 GiB, so pixel indices fit 32 bits and the divisions stay cheap */
+				const unsigned int p = static_cast<unsigned int>(p0) + threadIdx.x / STEP_CHUNKS + FETCH_ROWS * q;
+				const bool ok = p < static_cast<unsigned int>(g.pixels);
+				const unsigned int pp = ok ? p : 0u;
+				const unsigned int row = pp / static_cast<unsigned int>(g.Wo);
+				const int ow = static_cast<int>(pp - row * g.Wo);
+				const unsigned int n = row / static_cast<unsigned int>(g.Ho);
+				const int oh = static_cast<int>(row - n * g.Ho);
+				const int ih0 = oh * g.stride_h + g.pad_h;
+				const int iw0 = ow * g.stride_w + g.pad_w;
+				origin[q] = static_cast<unsigned int>((static_cast<int>(n * g.H + ih0) * g.W + iw0) * g.C + chunk_channel) * static_cast<unsigned int>(sizeof(TE));
+				unsigned int m = 0;
+				for (int t = 0; t < g.R * g.S; t++)
+				{
+					int i = t / g.S, j = t - (t / g.S) * g.S;
+					if (g.flip)
+					{
+						i = g.R - 1 - i;
+						j = g.S - 1 - j;
+					}
+					const int ih = ih0 + i * g.dil_h, iw = iw0 + j * g.dil_w;
+					if (ok && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
+						m |= 1u << t;
+				}
+				inside[q] = m;
+			}
+			set_tap();
+		}
+		__device__ inline void set_tap()
+		{
+			const int i = g.flip ? g.R - 1 - cur.i : cur.i;
+			const int j = g.flip ? g.S - 1 - cur.j : cur.j;
+			tap_bytes = static_cast<unsigned int>(((i * g.dil_h) * g.W + j * g.dil_w) * g.C) * static_cast<unsigned int>(sizeof(TE))
+					+ static_cast<unsigned int>(cur.slice) * STEP_BYTES;
+		}
+		__device__ inline uint4 load(int q, int) const
+		{
 			constexpr int KE = STEP_BYTES / sizeof(TE);
-			const int k = k0 + (threadIdx.x >> 2) + 64 * q;
-			if (k >= g.K)
-				return make_uint4(0u, 0u, 0u, 0u);
-			const int tap = step / g.steps_per_tap;
-			const int c = (step - tap * g.steps_per_tap) * KE + part * E;
-			return fetch_chunk<TE>(w + (static_cast<int64_t>(k) * g.R * g.S + tap) * g.C + c, g.C - c, vec_ok);
+			const bool exists = (((inside[q] >> cur.tap) & 1u) != 0u) & (cur.slice * KE + chunk_channel < g.C) & (cur.tap < 32);
+			return buffer_fetch(rsrc, exists ? origin[q] + tap_bytes : OUT_OF_RANGE);
+		}
+		__device__ inline void next()
+		{
+			cur.advance(g);
+			set_tap();
 		}
 	};
 
-	__device__ inline int round_saturate(float v, float lo, float hi)
+	/* Rows of B are output filters; a chunk is 16 bytes of channels of w[k, i, j, :]. */
+	template<typename TE, bool FAST>
+	struct FilterLoader
 	{
-		if (!(v == v))
-			return 0;
-		float r = rintf(v);
-		r = r < lo ? lo : r;
-		r = r > hi ? hi : r;
-		return static_cast<int>(r);
-	}
-
-	/* Floating tensors: TE in, TE out, fp32 bias. */
+		const ConvGeom &g;
+		bool vec_ok;
+		TapCursor cur;
+		const TE *rows[FETCH_PASSES];
+		__device__ inline FilterLoader(const TE *w, const ConvGeom &g_, bool vec_ok_, int k0) :
+				g(g_), vec_ok(vec_ok_)
+		{
+#pragma unroll
+			for (int q = 0; q < FETCH_PASSES; q++)
+			{
+				const int k = k0 + threadIdx.x / STEP_CHUNKS + FETCH_ROWS * q;
+				rows[q] = k < g.K ? w + static_cast<int64_t>(k) * g.R * g.S * g.C : nullptr;
+			}
+		}
+		__device__ inline uint4 load(int q, int part) const
+		{
+			constexpr int E = 16 / sizeof(TE);
+			constexpr int KE = STEP_BYTES / sizeof(TE);
+			if (rows[q] == nullptr || cur.i >= g.R)
+				return make_uint4(0u, 0u, 0u, 0u);
+			const int c = cur.slice * KE + part * E;
+			return fetch_chunk<TE>(rows[q] + static_cast<int64_t>(cur.tap) * g.C + c, g.C - c, vec_ok);
+		}
+		__device__ inline void next()
+		{
+			cur.advance(g);
+		}
+	};
 	template<typename TE>
-	__global__ __launch_bounds__(256) void k_conv_igemm_float(const TE *__restrict__ x, const TE *__restrict__ w, const float *__restrict__ bias, const TE *z,
-			TE *y, ConvGeom g, TE padv, int vec_ok, float alpha1, float alpha2, float beta, int activation)
+	struct FilterLoader<TE, true>
+	{
+		__amdgpu_buffer_rsrc_t rsrc;
+		const ConvGeom &g;
+		TapCursor cur;
+		unsigned int origin[FETCH_PASSES]; /* byte offset of w[k, 0, 0, chunk channel]; OUT_OF_RANGE for k >= K stays out of range */
+		int chunk_channel;
+		__device__ inline FilterLoader(const TE *w, const ConvGeom &g_, bool, int k0) :
+				g(g_)
+		{
+			constexpr int E = 16 / sizeof(TE);
+			rsrc = make_buffer(w, static_cast<unsigned int>(static_cast<int64_t>(g.K) * g.R * g.S * g.C * sizeof(TE)));
+			chunk_channel = (threadIdx.x % STEP_CHUNKS) * E;
+#pragma unroll
+			for (int q = 0; q < FETCH_PASSES; q++)
+			{
+				const int k = k0 + threadIdx.x / STEP_CHUNKS + FETCH_ROWS * q;
+				origin[q] = k < g.K ? static_cast<unsigned int>((k * g.R * g.S * g.C + chunk_channel) * sizeof(TE)) : OUT_OF_RANGE;
+			}
+		}
+		__device__ inline uint4 load(int q, int) const
+		{
+			constexpr int KE = STEP_BYTES / sizeof(TE);
+			const unsigned int tap_bytes = static_cast<unsigned int>(cur.tap * g.C) * static_cast<unsigned int>(sizeof(TE))
+					+ static_cast<unsigned int>(cur.slice) * STEP_BYTES;
+			const bool exists = (cur.slice * KE + chunk_channel < g.C) & (cur.i < g.R);
+			return buffer_fetch(rsrc, exists ? origin[q] + tap_bytes : OUT_OF_RANGE);
+		}
+		__device__ inline void next()
+		{
+			cur.advance(g);
+		}
+	};
+
+	/* One kernel for every epilogue: Epi is FloatEpilogue<TE> or Int8Epilogue<mode>.  FAST instances use the branch-free
+	 * loaders and are launched for LINEAR / RELU only; everything else runs the general instance. */
+	template<typename TE, bool FAST, typename Epi>
+	__global__ __launch_bounds__(256, 2) void k_conv_igemm(const TE *__restrict__ x, const TE *__restrict__ w, ConvGeom g, TE padv, int vec_ok, Epi epi)
 	{
 		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
 		const int64_t p0 = static_cast<int64_t>(blockIdx.x) * BLOCK_M;
-		const int k0 = blockIdx.y * BLOCK_N;
-		PixelLoader<TE> la(x, g, padv, (vec_ok & 1) != 0, p0, threadIdx.x >> 2);
-		FilterLoader<TE> lb { w, g, (vec_ok & 1) != 0, k0 };
+		const int k = blockIdx.y * BLOCK_N + drain_column<2>();
+		typename Epi::Columns columns;
+		epi.load_columns(k, columns); /* issued before the k loop: its latency is hidden behind the whole convolution */
+
+		PixelLoader<TE, FAST> la(x, g, padv, (vec_ok & 1) != 0, p0);
+		FilterLoader<TE, FAST> lb(w, g, (vec_ok & 1) != 0, blockIdx.y * BLOCK_N);
 		typename Mma<TE>::acc_t acc[2][2];
 		block_mma<TE>(lds, g.R * g.S * g.steps_per_tap, la, lb, acc);
 
-		const bool vec_y = (vec_ok & 2) != 0;
-		drain_tile<TE>(lds, acc, [&](int r, int col, const float (&v)[4])
+		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const typename Epi::scalar_t (&v)[4]) __attribute__((always_inline))
 		{
 			const int64_t p = p0 + r;
-			const int k = k0 + col;
-			if (p >= g.pixels || k >= g.K)
-				return;
-			const int valid = g.K - k;
-			const int64_t idx = p * g.K + k;
-			float t[4];
-#pragma unroll
-			for (int q = 0; q < 4; q++)
-				t[q] = alpha1 * v[q] + ((bias != nullptr && q < valid) ? bias[k + q] : 0.0f);
-			if (z != nullptr)
-			{
-				float zv[4];
-				load_vec<TE, 4, float>(z + idx, valid, zv, vec_y);
-#pragma unroll
-				for (int q = 0; q < 4; q++)
-					t[q] += alpha2 * zv[q];
-			}
-#pragma unroll
-			for (int q = 0; q < 4; q++)
-				t[q] = activation_forward<float>(activation, t[q]);
-			if (beta != 0.0f)
-			{
-				float yv[4];
-				load_vec<TE, 4, float>(y + idx, valid, yv, vec_y);
-#pragma unroll
-				for (int q = 0; q < 4; q++)
-					t[q] += beta * yv[q];
-			}
-			store_vec<TE, 4, float>(y + idx, valid, t, vec_y);
-		});
-	}
-
-	enum Int8Epilogue
-	{
-		I8_EXACT = 0, /* y int32 = act(sum + bias_i32)                                   */
-		I8_REQUANT, /* y int8  = sat(rne(float(sum + bias_i32) * scale[k]))             */
-		I8_FLOAT_I32, /* float epilogue, y int32                                         */
-		I8_FLOAT_I8, /* float epilogue, y int8                                           */
-		I8_FLOAT_F32 /* float epilogue, y fp32                                           */
-	};
-
-	/* From here on every fp32 operation must round exactly once: the float epilogue on integer sums is specified step by
-	 * step (multiply, add, multiply, add), so a*b + c must not be contracted into a fused multiply-add.  The pragma only
-	 * governs expressions written below it, which is why the epilogue uses plain operators and no header intrinsics. */
-#pragma clang fp contract(off)
-
-	template<int MODE>
-	__global__ __launch_bounds__(256) void k_conv_igemm_int8(const int8_t *__restrict__ x, const int8_t *__restrict__ w, const void *__restrict__ bias,
-			const void *z, void *y, const float *__restrict__ scale, ConvGeom g, int8_t padv, int vec_ok, float alpha1, float alpha2, float beta, int activation)
-	{
-		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
-		const int64_t p0 = static_cast<int64_t>(blockIdx.x) * BLOCK_M;
-		const int k0 = blockIdx.y * BLOCK_N;
-		PixelLoader<int8_t> la(x, g, padv, (vec_ok & 1) != 0, p0, threadIdx.x >> 2);
-		FilterLoader<int8_t> lb { w, g, (vec_ok & 1) != 0, k0 };
-		Mma<int8_t>::acc_t acc[2][2];
-		block_mma<int8_t>(lds, g.R * g.S * g.steps_per_tap, la, lb, acc);
-
-		const bool vec_y = (vec_ok & 2) != 0;
-		drain_tile<int8_t>(lds, acc, [&](int r, int col, const int (&v)[4])
-		{
-			const int64_t p = p0 + r;
-			const int k = k0 + col;
-			if (p >= g.pixels || k >= g.K)
-				return;
-			const int valid = g.K - k;
-			const int64_t idx = p * g.K + k;
-			if (MODE == I8_EXACT || MODE == I8_REQUANT)
-			{
-				int t[4];
-#pragma unroll
-				for (int q = 0; q < 4; q++)
-				{
-					t[q] = v[q] + ((bias != nullptr && q < valid) ? static_cast<const int*>(bias)[k + q] : 0);
-					if (activation == ACT_RELU && t[q] < 0)
-						t[q] = 0;
-				}
-				if (MODE == I8_EXACT)
-				{
-					int *dst = static_cast<int*>(y) + idx;
-					if (vec_y && valid >= 4)
-						*reinterpret_cast<int4*>(dst) = make_int4(t[0], t[1], t[2], t[3]);
-					else
-					{
-#pragma unroll
-						for (int q = 0; q < 4; q++)
-							if (q < valid)
-								dst[q] = t[q];
-					}
-				}
-				else
-				{
-					int8_t o[4];
-#pragma unroll
-					for (int q = 0; q < 4; q++)
-						o[q] = static_cast<int8_t>(round_saturate(static_cast<float>(t[q]) * (q < valid ? scale[k + q] : 0.0f), -128.0f, 127.0f));
-					int8_t *dst = static_cast<int8_t*>(y) + idx;
-					if (vec_y && valid >= 4)
-						*reinterpret_cast<char4*>(dst) = make_char4(o[0], o[1], o[2], o[3]);
-					else
-					{
-#pragma unroll
-						for (int q = 0; q < 4; q++)
-							if (q < valid)
-								dst[q] = o[q];
-					}
-				}
-			}
-			else
-			{
-#pragma unroll
-				for (int q = 0; q < 4; q++)
-				{
-					if (q >= valid)
-						continue;
-					float t = alpha1 * static_cast<float>(v[q]);
-					if (bias != nullptr)
-						t = t + static_cast<const float*>(bias)[k + q];
-					if (z != nullptr)
-					{
-						const float zv = MODE == I8_FLOAT_I32 ? static_cast<float>(static_cast<const int*>(z)[idx + q]) :
-											MODE == I8_FLOAT_I8 ? static_cast<float>(static_cast<const int8_t*>(z)[idx + q]) : static_cast<const float*>(z)[idx + q];
-						t = t + alpha2 * zv;
-					}
-					t = activation_forward<float>(activation, t);
-					if (beta != 0.0f)
-					{
-						const float yv = MODE == I8_FLOAT_I32 ? static_cast<float>(static_cast<int*>(y)[idx + q]) :
-											MODE == I8_FLOAT_I8 ? static_cast<float>(static_cast<int8_t*>(y)[idx + q]) : static_cast<float*>(y)[idx + q];
-						t = t + beta * yv;
-					}
-					if (MODE == I8_FLOAT_I32)
-						static_cast<int*>(y)[idx + q] = round_saturate(t, -2147483648.0f, 2147483520.0f);
-					else if (MODE == I8_FLOAT_I8)
-						static_cast<int8_t*>(y)[idx + q] = static_cast<int8_t>(round_saturate(t, -128.0f, 127.0f));
-					else
-						static_cast<float*>(y)[idx + q] = t;
-				}
-			}
+			if (p < g.pixels && k < g.K)
+				epi.template store<FAST ? ACT_SIMPLE : ACT_ANY>(p, k, v, columns);
 		});
 	}
 
@@ -295,6 +296,7 @@ namespace
 		constexpr int KE = STEP_BYTES / sizeof(TE);
 		g.steps_per_tap = (s.C + KE - 1) / KE;
 		g.pixels = static_cast<int64_t>(s.N) * s.Ho * s.Wo;
+		g.images = s.N;
 		return g;
 	}
 	/* bit 0: operand chunks may use 16-byte loads; bit 1: y / z rows may use 4-element vectors of `out_elem` bytes. */
@@ -306,32 +308,57 @@ namespace
 		return (in_ok ? 1 : 0) | (out_ok ? 2 : 0);
 	}
 
+	/* The branch-free loaders need aligned, complete chunks (bit 0 of flags), a zero padding value and 32-bit byte offsets. */
 	template<typename TE>
-	int launch_float(hipStream_t st, const avhipConvShape &s, const void *x, const void *w, const void *bias, const void *z, void *y, const void *padding_value,
-			double alpha1, double alpha2, double beta, int activation)
+	bool fast_path_ok(const avhipConvShape &s, int flags, const void *padding_value)
+	{
+		bool zero_padding = true;
+		if (padding_value != nullptr)
+			for (size_t i = 0; i < sizeof(TE); i++)
+				zero_padding = zero_padding && static_cast<const unsigned char*>(padding_value)[i] == 0;
+		const int64_t x_bytes = static_cast<int64_t>(s.N) * s.H * s.W * s.C * sizeof(TE);
+		const int64_t w_bytes = static_cast<int64_t>(s.K) * s.R * s.S * s.C * sizeof(TE);
+		const int64_t pixels = static_cast<int64_t>(s.N) * s.Ho * s.Wo;
+		return (flags & 1) != 0 && zero_padding && x_bytes < (1ll << 31) && w_bytes < (1ll << 31) && pixels < (1ll << 31) - BLOCK_M && s.R * s.S <= 32;
+	}
+
+	template<typename TE, typename Epi>
+	int launch(hipStream_t st, const avhipConvShape &s, const void *x, const void *w, const void *padding_value, int flags, const Epi &epi)
 	{
 		const ConvGeom g = make_geom<TE>(s);
 		TE padv;
 		if (padding_value != nullptr)
 			padv = *static_cast<const TE*>(padding_value);
 		else
-			padv = Traits<TE>::store(0.0f);
+			std::memset(&padv, 0, sizeof(TE));
 		const dim3 grid(ceil_div(g.pixels, BLOCK_M), ceil_div(s.K, BLOCK_N));
-		hipLaunchKernelGGL((k_conv_igemm_float<TE>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w),
-				static_cast<const float*>(bias), static_cast<const TE*>(z), static_cast<TE*>(y), g, padv, vector_flags<TE>(s, x, w, y, z, sizeof(TE)),
-				static_cast<float>(alpha1), static_cast<float>(alpha2), static_cast<float>(beta), activation);
+		const bool fast = fast_path_ok<TE>(s, flags, padding_value) && is_simple_activation(epi.activation);
+		/* stride-1 filters with more than one tap first try the kernel that keeps an image tile resident in LDS */
+		if (fast && s.R * s.S > 1 && conv_tile_launch<TE, Epi>(st, s, x, w, epi))
+			return 0;
+		if (fast)
+			hipLaunchKernelGGL((k_conv_igemm<TE, true, Epi>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags, epi);
+		else
+			hipLaunchKernelGGL((k_conv_igemm<TE, false, Epi>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags, epi);
 		return 0;
+	}
+	template<typename TE>
+	int launch_float(hipStream_t st, const avhipConvShape &s, const void *x, const void *w, const void *bias, const void *z, void *y, const void *padding_value,
+			double alpha1, double alpha2, double beta, int activation)
+	{
+		const int flags = vector_flags<TE>(s, x, w, y, z, sizeof(TE));
+		const FloatEpilogue<TE> epi { static_cast<const float*>(bias), static_cast<const TE*>(z), static_cast<TE*>(y), static_cast<float>(alpha1),
+				static_cast<float>(alpha2), static_cast<float>(beta), activation, s.K, (flags & 2) != 0 };
+		return launch<TE>(st, s, x, w, padding_value, flags, epi);
 	}
 	template<int MODE>
 	int launch_int8(hipStream_t st, const avhipConvShape &s, const void *x, const void *w, const void *bias, const void *z, void *y, const float *scale,
 			const void *padding_value, double alpha1, double alpha2, double beta, int activation)
 	{
-		const ConvGeom g = make_geom<int8_t>(s);
-		const int8_t padv = padding_value != nullptr ? *static_cast<const int8_t*>(padding_value) : static_cast<int8_t>(0);
-		const dim3 grid(ceil_div(g.pixels, BLOCK_M), ceil_div(s.K, BLOCK_N));
-		hipLaunchKernelGGL((k_conv_igemm_int8<MODE>), grid, dim3(256), 0, st, static_cast<const int8_t*>(x), static_cast<const int8_t*>(w), bias, z, y, scale, g,
-				padv, vector_flags<int8_t>(s, x, w, y, z, MODE == I8_REQUANT || MODE == I8_FLOAT_I8 ? 1 : 4), static_cast<float>(alpha1), static_cast<float>(alpha2), static_cast<float>(beta), activation);
-		return 0;
+		const int flags = vector_flags<int8_t>(s, x, w, y, z, MODE == I8_REQUANT || MODE == I8_FLOAT_I8 ? 1 : 4);
+		const Int8Epilogue<MODE> epi { bias, z, y, scale, static_cast<float>(alpha1), static_cast<float>(alpha2), static_cast<float>(beta), activation, s.K,
+				(flags & 2) != 0 };
+		return launch<int8_t>(st, s, x, w, padding_value, flags, epi);
 	}
 }
 

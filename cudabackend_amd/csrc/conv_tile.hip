@@ -1,0 +1,312 @@
+/*
+ * conv_tile.hip -- implicit-GEMM convolution for stride-1 filters that keeps an image tile resident in LDS.
+ *
+ * The general implicit-GEMM kernel (conv_implicit_gemm.hip) re-fetches every input pixel once per filter tap from L2: for
+ * a 3x3 filter that is 9x the input volume plus the weights once per 128 output pixels, and on MI355X this L2 -> CU traffic,
+ * not the matrix cores, bounds it.  This kernel removes most of that traffic:
+ *
+ *   - a workgroup owns TH x TW <= 256 output pixels of ONE image (the whole image when it is 15 x 15) and 64 filters;
+ *   - for each 128-byte slice of input channels it loads the (TH+R-1) x (TW+S-1) input halo ONCE into LDS (pixels outside
+ *     the image come back as zeros from the buffer load) and then walks the R*S taps, reading the A operand of tap (i, j)
+ *     straight from the halo at a per-tap uniform offset: the input is read from L2 about once per slice, not R*S times;
+ *   - only the weights stream: 64 filters x 128 bytes per step, fetched two steps ahead into registers and double buffered
+ *     in LDS exactly as in the general engine;
+ *   - the halo of the next channel slice is fetched during the last tap of the current one.
+ * Four wavefronts stack in M (64 pixels x 64 filters each, 2 x 2 MFMA tiles of 32 x 32); 60 KB of LDS and <= 256 registers
+ * let two workgroups share a CU.  k order is (channel slice, tap), which sums the same products as (tap, channel).
+ */
+#include "conv_tile.hpp"
+#include "mfma_core.hpp"
+
+namespace
+{
+	using namespace avhip;
+
+	constexpr int TILE_M = 256; /* output pixels per workgroup */
+	constexpr int TILE_N = 64; /* output filters per workgroup */
+	constexpr int PIXEL_PITCH = STEP_BYTES + 16; /* LDS bytes per halo pixel: 128 of channels + 16 of bank stagger */
+	constexpr int HALO_MAX = 300; /* halo pixels that fit */
+	constexpr int HALO_BYTES = HALO_MAX * PIXEL_PITCH;
+	constexpr int FILTER_TILE = TILE_N * LDS_ROW;
+	constexpr int TILE_LDS = HALO_BYTES + 2 * FILTER_TILE;
+	constexpr int HALO_FETCHES = (HALO_MAX * STEP_CHUNKS + 255) / 256; /* 16-byte chunks of the halo per work-item */
+	constexpr int FILTER_FETCHES = TILE_N * STEP_CHUNKS / 256;
+	static_assert(DrainShape<1>::bytes <= TILE_LDS, "the drain buffer reuses the operand buffers");
+
+	struct TileGeom
+	{
+		int H, W, C, K, R, S, Ho, Wo, pad_h, pad_w, flip;
+		int TH, TW; /* output tile */
+		int HH, HW; /* halo = (TH + R - 1) x (TW + S - 1) */
+		int tiles_h, tiles_w;
+		int slices; /* 128-byte channel slices */
+		int images;
+	};
+
+	template<typename TE, typename Epi>
+	__global__ __launch_bounds__(256, 2) void k_conv_tile(const TE *__restrict__ x, const TE *__restrict__ w, TileGeom g, Epi epi)
+	{
+		__shared__ __attribute__((aligned(16))) char lds[TILE_LDS];
+		char *halo = lds;
+		char *filt = lds + HALO_BYTES;
+		constexpr int E = 16 / sizeof(TE);
+		constexpr int KE = STEP_BYTES / sizeof(TE);
+		constexpr unsigned int SZ = sizeof(TE);
+		const int tid = threadIdx.x;
+		const int lane = tid & 63;
+		const int wave = tid >> 6;
+		const int part = tid % STEP_CHUNKS;
+		const int chunk_channel = part * E;
+
+		int b = blockIdx.x;
+		const int tw = b % g.tiles_w;
+		b /= g.tiles_w;
+		const int th = b % g.tiles_h;
+		const int n = b / g.tiles_h;
+		const int oh0 = th * g.TH, ow0 = tw * g.TW;
+		const int k0 = blockIdx.y * TILE_N;
+		const int kcol = k0 + drain_column<1>();
+		typename Epi::Columns columns;
+		epi.load_columns(kcol, columns);
+
+		const __amdgpu_buffer_rsrc_t rx = make_buffer(x, static_cast<unsigned int>(g.images) * g.H * g.W * g.C * SZ);
+		const __amdgpu_buffer_rsrc_t rw = make_buffer(w, static_cast<unsigned int>(g.K) * g.R * g.S * g.C * SZ);
+
+		/* where this work-item's halo chunks come from (slice 0) and go to */
+		unsigned int halo_src[HALO_FETCHES];
+		const int halo_pixels = g.HH * g.HW;
+#pragma unroll
+		for (int f = 0; f < HALO_FETCHES; f++)
+		{
+			const int h = tid / STEP_CHUNKS + f * (256 / STEP_CHUNKS);
+			const int hy = h / g.HW, hx = h - hy * g.HW;
+			const int ih = oh0 + g.pad_h + hy, iw = ow0 + g.pad_w + hx;
+			const bool inside = (h < halo_pixels) & (ih >= 0) & (ih < g.H) & (iw >= 0) & (iw < g.W);
+			halo_src[f] = inside ? static_cast<unsigned int>(((n * g.H + ih) * g.W + iw) * g.C + chunk_channel) * SZ : OUT_OF_RANGE;
+		}
+		const int halo_dst = (tid / STEP_CHUNKS) * PIXEL_PITCH + part * 16;
+		unsigned int filt_src[FILTER_FETCHES];
+#pragma unroll
+		for (int f = 0; f < FILTER_FETCHES; f++)
+		{
+			const int k = k0 + tid / STEP_CHUNKS + f * (256 / STEP_CHUNKS);
+			filt_src[f] = k < g.K ? static_cast<unsigned int>(k * g.R * g.S * g.C + chunk_channel) * SZ : OUT_OF_RANGE;
+		}
+		const int filt_dst = (tid / STEP_CHUNKS) * LDS_ROW + part * 16;
+
+		/* MFMA operand addresses: lane l supplies row (l % 32) of a 32-row tile and k-chunk (l / 32) */
+		int a_off[2];
+#pragma unroll
+		for (int tm = 0; tm < 2; tm++)
+		{
+			const int row = wave * 64 + tm * 32 + (lane & 31);
+			const int py = row / g.TW, px = row - py * g.TW;
+			const int pix = row < g.TH * g.TW ? py * g.HW + px : 0; /* rows past the tile read pixel 0 and are never stored */
+			a_off[tm] = pix * PIXEL_PITCH + (lane >> 5) * 16;
+		}
+		const int b_off = (lane & 31) * LDS_ROW + (lane >> 5) * 16;
+
+		const int taps = g.R * g.S;
+		const int total = g.slices * taps;
+		typename Mma<TE>::acc_t acc[2][2];
+#pragma unroll
+		for (int i = 0; i < 2; i++)
+#pragma unroll
+			for (int j = 0; j < 2; j++)
+#pragma unroll
+				for (int v = 0; v < 16; v++)
+					acc[i][j][v] = 0;
+
+		/* fetch side: runs two steps ahead of the MFMAs */
+		int f_slice = 0, f_tap = 0;
+		auto fetch_filters = [&](uint4 (&r)[FILTER_FETCHES]) __attribute__((always_inline))
+		{
+			const unsigned int k_bytes = static_cast<unsigned int>(f_tap * g.C) * SZ + static_cast<unsigned int>(f_slice) * STEP_BYTES;
+			const bool exists = (f_slice * KE + chunk_channel < g.C) & (f_slice < g.slices);
+#pragma unroll
+			for (int f = 0; f < FILTER_FETCHES; f++)
+				r[f] = buffer_fetch(rw, exists ? filt_src[f] + k_bytes : OUT_OF_RANGE);
+			if (++f_tap == taps)
+			{
+				f_tap = 0;
+				f_slice++;
+			}
+		};
+		auto stash_filters = [&](int buffer, const uint4 (&r)[FILTER_FETCHES]) __attribute__((always_inline))
+		{
+#pragma unroll
+			for (int f = 0; f < FILTER_FETCHES; f++)
+				*reinterpret_cast<uint4*>(filt + buffer * FILTER_TILE + filt_dst + f * (256 / STEP_CHUNKS) * LDS_ROW) = r[f];
+		};
+		auto fetch_halo = [&](int slice, uint4 (&r)[HALO_FETCHES]) __attribute__((always_inline))
+		{
+			const bool exists = slice * KE + chunk_channel < g.C;
+#pragma unroll
+			for (int f = 0; f < HALO_FETCHES; f++)
+				r[f] = buffer_fetch(rx, exists ? halo_src[f] + static_cast<unsigned int>(slice) * STEP_BYTES : OUT_OF_RANGE);
+		};
+		auto stash_halo = [&](const uint4 (&r)[HALO_FETCHES]) __attribute__((always_inline))
+		{
+#pragma unroll
+			for (int f = 0; f < HALO_FETCHES; f++)
+				if (tid / STEP_CHUNKS + f * (256 / STEP_CHUNKS) < HALO_MAX)
+					*reinterpret_cast<uint4*>(halo + halo_dst + f * (256 / STEP_CHUNKS) * PIXEL_PITCH) = r[f];
+		};
+		/* compute side */
+		int c_slice = 0, c_i = 0, c_j = 0;
+		auto multiply = [&](int buffer) __attribute__((always_inline))
+		{
+			const int i = g.flip ? g.R - 1 - c_i : c_i;
+			const int j = g.flip ? g.S - 1 - c_j : c_j;
+			const char *sa = halo + (i * g.HW + j) * PIXEL_PITCH;
+			const char *sb = filt + buffer * FILTER_TILE + b_off;
+			constexpr int SLABS = STEP_BYTES / 32;
+			Chunk a[2][2], bq[2][2];
+			auto read = [&](int slab, Chunk (&ra_)[2], Chunk (&rb_)[2]) __attribute__((always_inline))
+			{
+#pragma unroll
+				for (int t = 0; t < 2; t++)
+				{
+					ra_[t].u = *reinterpret_cast<const uint4*>(sa + a_off[t] + slab * 32);
+					rb_[t].u = *reinterpret_cast<const uint4*>(sb + t * 32 * LDS_ROW + slab * 32);
+				}
+			};
+			read(0, a[0], bq[0]);
+#pragma unroll
+			for (int slab = 0; slab < SLABS; slab++)
+			{
+				if (slab + 1 < SLABS)
+					read(slab + 1, a[(slab + 1) & 1], bq[(slab + 1) & 1]);
+#pragma unroll
+				for (int tm = 0; tm < 2; tm++)
+#pragma unroll
+					for (int tn = 0; tn < 2; tn++)
+						Mma<TE>::run(a[slab & 1][tm], bq[slab & 1][tn], acc[tm][tn]);
+			}
+		};
+
+		uint4 hr[HALO_FETCHES];
+		uint4 fr[2][FILTER_FETCHES];
+		fetch_halo(0, hr);
+		fetch_filters(fr[0]);
+		fetch_filters(fr[1]);
+		stash_halo(hr);
+		stash_filters(0, fr[0]);
+
+		/* One step = one tap of one channel slice.  Steps run in pairs so that the two register sets and the two LDS
+		 * buffers alternate with compile-time indices; fetches past the last step return zeros and are never multiplied. */
+		auto step = [&](int s, int buffer, uint4 (&mine)[FILTER_FETCHES], uint4 (&other)[FILTER_FETCHES]) __attribute__((always_inline))
+		{
+			__syncthreads(); /* filters of step s and the current halo are visible; everyone is done with step s - 1 */
+			fetch_filters(mine); /* step s + 2 */
+			const bool last_tap = (c_i == g.R - 1) & (c_j == g.S - 1);
+			const bool more_slices = c_slice + 1 < g.slices;
+			if (last_tap & more_slices)
+				fetch_halo(c_slice + 1, hr);
+			if (s < total)
+				multiply(buffer);
+			stash_filters(buffer ^ 1, other); /* step s + 1 */
+			if (++c_j == g.S)
+			{
+				c_j = 0;
+				if (++c_i == g.R)
+				{
+					c_i = 0;
+					c_slice++;
+					if (c_slice < g.slices)
+					{
+						__syncthreads(); /* nobody reads the old halo any more */
+						stash_halo(hr);
+					}
+				}
+			}
+		};
+		for (int s = 0; s < total; s += 2)
+		{
+			step(s, 0, fr[0], fr[1]);
+			step(s + 1, 1, fr[1], fr[0]);
+		}
+
+		drain_tile<TE, 2, 1>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[4]) __attribute__((always_inline))
+		{
+			const int py = row / g.TW, px = row - py * g.TW;
+			const int oh = oh0 + py, ow = ow0 + px;
+			if (row < g.TH * g.TW && oh < g.Ho && ow < g.Wo && kcol < g.K)
+				epi.template store<ACT_SIMPLE>((static_cast<int64_t>(n) * g.Ho + oh) * g.Wo + ow, kcol, v, columns);
+		});
+	}
+
+	/* Picks the output tile: as few tiles per image as possible with TH * TW <= 256 and the halo within HALO_MAX. */
+	bool choose_tile(const avhipConvShape &s, TileGeom &g)
+	{
+		int best_tiles = 0, best_halo = 0;
+		for (int tw = 1; tw <= s.Wo && tw <= TILE_M; tw++)
+			for (int th = 1; th <= s.Ho && th * tw <= TILE_M; th++)
+			{
+				const int halo = (th + s.R - 1) * (tw + s.S - 1);
+				if (halo > HALO_MAX)
+					continue;
+				const int tiles = ((s.Ho + th - 1) / th) * ((s.Wo + tw - 1) / tw);
+				if (best_tiles == 0 || tiles < best_tiles || (tiles == best_tiles && halo < best_halo))
+				{
+					best_tiles = tiles;
+					best_halo = halo;
+					g.TH = th;
+					g.TW = tw;
+				}
+			}
+		return best_tiles > 0;
+	}
+}
+
+namespace avhip
+{
+	template<typename TE, typename Epi>
+	bool conv_tile_launch(hipStream_t stream, const avhipConvShape &s, const void *x, const void *w, const Epi &epi)
+	{
+		if (s.stride_h != 1 || s.stride_w != 1 || s.dil_h != 1 || s.dil_w != 1)
+			return false;
+		TileGeom g;
+		if (!choose_tile(s, g))
+			return false;
+		g.H = s.H;
+		g.W = s.W;
+		g.C = s.C;
+		g.K = s.K;
+		g.R = s.R;
+		g.S = s.S;
+		g.Ho = s.Ho;
+		g.Wo = s.Wo;
+		g.pad_h = s.pad_h;
+		g.pad_w = s.pad_w;
+		g.flip = s.mode != 0 ? 1 : 0;
+		g.HH = g.TH + s.R - 1;
+		g.HW = g.TW + s.S - 1;
+		g.tiles_h = (s.Ho + g.TH - 1) / g.TH;
+		g.tiles_w = (s.Wo + g.TW - 1) / g.TW;
+		g.slices = (s.C * static_cast<int>(sizeof(TE)) + STEP_BYTES - 1) / STEP_BYTES;
+		g.images = s.N;
+		/* the gather kernel wastes nothing on partially filled tiles: keep it when tiles would be mostly padding */
+		const double fill = static_cast<double>(s.Ho) * s.Wo / (static_cast<double>(g.tiles_h) * g.tiles_w * TILE_M);
+		if (fill < 0.5)
+			return false;
+		const int64_t blocks = static_cast<int64_t>(s.N) * g.tiles_h * g.tiles_w;
+		const int64_t filter_blocks = (static_cast<int64_t>(s.K) + TILE_N - 1) / TILE_N;
+		if (blocks > 0x7FFFFFFFll || filter_blocks > 65535)
+			return false;
+		hipLaunchKernelGGL((k_conv_tile<TE, Epi>), dim3(static_cast<unsigned int>(blocks), static_cast<unsigned int>(filter_blocks)), dim3(256), 0, stream,
+				static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
+		return true;
+	}
+
+#define AVHIP_INSTANTIATE(TE, EPI) template bool conv_tile_launch<TE, EPI>(hipStream_t, const avhipConvShape&, const void*, const void*, const EPI&);
+	AVHIP_INSTANTIATE(float, FloatEpilogue<float>)
+	AVHIP_INSTANTIATE(f16_t, FloatEpilogue<f16_t>)
+	AVHIP_INSTANTIATE(bf16_t, FloatEpilogue<bf16_t>)
+	AVHIP_INSTANTIATE(int8_t, Int8Epilogue<I8_EXACT>)
+	AVHIP_INSTANTIATE(int8_t, Int8Epilogue<I8_REQUANT>)
+	AVHIP_INSTANTIATE(int8_t, Int8Epilogue<I8_FLOAT_I32>)
+	AVHIP_INSTANTIATE(int8_t, Int8Epilogue<I8_FLOAT_I8>)
+	AVHIP_INSTANTIATE(int8_t, Int8Epilogue<I8_FLOAT_F32>)
+#undef AVHIP_INSTANTIATE
+}

@@ -15,21 +15,63 @@ namespace
 {
 	using namespace avhip;
 
-	template<typename TE>
+	/* Operand rows of a plain row-major matrix: row r starts at base + r * ld, k runs along the row.
+	 * General form: any alignment, any K; partial chunks are assembled element by element. */
+	template<typename TE, bool FAST>
 	struct RowLoader
 	{
-		const TE *base;
-		int rows, K, ld, row0;
+		const TE *rows[FETCH_PASSES]; /* start of this work-item's rows, nullptr outside the matrix */
+		int K, k;
 		bool vec_ok;
-		__device__ inline uint4 operator()(int step, int q, int part) const
+		__device__ inline RowLoader(const TE *base, int nrows, int K_, int ld, int row0, bool vec_ok_) :
+				K(K_), k(0), vec_ok(vec_ok_)
+		{
+#pragma unroll
+			for (int q = 0; q < FETCH_PASSES; q++)
+			{
+				const int row = row0 + threadIdx.x / STEP_CHUNKS + FETCH_ROWS * q;
+				rows[q] = row < nrows ? base + static_cast<size_t>(row) * ld : nullptr;
+			}
+		}
+		__device__ inline uint4 load(int q, int part) const
 		{
 			constexpr int E = 16 / sizeof(TE);
-			constexpr int KE = STEP_BYTES / sizeof(TE);
-			const int row = row0 + (threadIdx.x >> 2) + 64 * q;
-			const int k = step * KE + part * E;
-			if (row >= rows)
+			if (rows[q] == nullptr)
 				return make_uint4(0u, 0u, 0u, 0u);
-			return fetch_chunk<TE>(base + static_cast<size_t>(row) * ld + k, K - k, vec_ok);
+			const int kk = k + part * E;
+			return fetch_chunk<TE>(rows[q] + kk, K - kk, vec_ok);
+		}
+		__device__ inline void next()
+		{
+			k += STEP_BYTES / sizeof(TE);
+		}
+	};
+	/* Fast form: rows 16-byte aligned, K a multiple of the chunk, matrix below 2 GiB: branch-free buffer loads. */
+	template<typename TE>
+	struct RowLoader<TE, true>
+	{
+		__amdgpu_buffer_rsrc_t rsrc;
+		unsigned int origin[FETCH_PASSES]; /* byte offset of this work-item's chunk in its rows; OUT_OF_RANGE stays out of range */
+		unsigned int chunk_bytes, k_bytes, K_bytes;
+		__device__ inline RowLoader(const TE *base, int nrows, int K, int ld, int row0, bool) :
+				k_bytes(0), K_bytes(K * sizeof(TE))
+		{
+			rsrc = make_buffer(base, (static_cast<unsigned int>(nrows - 1) * ld + K) * sizeof(TE));
+			chunk_bytes = (threadIdx.x % STEP_CHUNKS) * 16;
+#pragma unroll
+			for (int q = 0; q < FETCH_PASSES; q++)
+			{
+				const int row = row0 + threadIdx.x / STEP_CHUNKS + FETCH_ROWS * q;
+				origin[q] = row < nrows ? static_cast<unsigned int>(row) * ld * sizeof(TE) + chunk_bytes : OUT_OF_RANGE;
+			}
+		}
+		__device__ inline uint4 load(int q, int) const
+		{
+			return buffer_fetch(rsrc, (k_bytes + chunk_bytes < K_bytes) ? origin[q] + k_bytes : OUT_OF_RANGE);
+		}
+		__device__ inline void next()
+		{
+			k_bytes += STEP_BYTES;
 		}
 	};
 
@@ -72,8 +114,8 @@ namespace
 		}
 	}
 
-	template<typename TE, typename TC>
-	__global__ __launch_bounds__(256) void k_gemm_nt_mfma(const TE *__restrict__ A, const TE *__restrict__ B, TC *C, int M, int N, int K, int lda, int ldb,
+	template<typename TE, typename TC, bool FAST>
+	__global__ __launch_bounds__(256, 2) void k_gemm_nt_mfma(const TE *__restrict__ A, const TE *__restrict__ B, TC *C, int M, int N, int K, int lda, int ldb,
 			int ldc, int64_t strideA, int64_t strideB, int64_t strideC, typename Mma<TE>::scalar_t alpha, typename Mma<TE>::scalar_t beta, int vec_ok)
 	{
 		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
@@ -82,17 +124,17 @@ namespace
 		const int m0 = blockIdx.x * BLOCK_M;
 		const int n0 = blockIdx.y * BLOCK_N;
 
-		RowLoader<TE> la { A + batch * strideA, M, K, lda, m0, (vec_ok & 1) != 0 };
-		RowLoader<TE> lb { B + batch * strideB, N, K, ldb, n0, (vec_ok & 1) != 0 };
+		RowLoader<TE, FAST> la(A + batch * strideA, M, K, lda, m0, (vec_ok & 1) != 0);
+		RowLoader<TE, FAST> lb(B + batch * strideB, N, K, ldb, n0, (vec_ok & 1) != 0);
 		typename Mma<TE>::acc_t acc[2][2];
 		block_mma<TE>(lds, (K + KE - 1) / KE, la, lb, acc);
 
 		TC *c = C + batch * strideC;
 		const bool vec_c = (vec_ok & 2) != 0;
-		drain_tile<TE>(lds, acc, [&](int r, int col, const typename Mma<TE>::scalar_t (&v)[4])
+		const int cc = n0 + drain_column<2>();
+		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const typename Mma<TE>::scalar_t (&v)[4]) __attribute__((always_inline))
 		{
 			const int row = m0 + r;
-			const int cc = n0 + col;
 			if (row < M && cc < N)
 				store_c(c + static_cast<size_t>(row) * ldc + cc, N - cc, vec_c, v, alpha, beta);
 		});
@@ -162,8 +204,17 @@ namespace
 				&& (sA * sizeof(TE)) % 16 == 0 && (sB * sizeof(TE)) % 16 == 0;
 		const bool vec_c = aligned_to(C, 4 * sizeof(TC)) && ldc % 4 == 0 && sC % 4 == 0;
 		const dim3 grid(ceil_div(M, BLOCK_M), ceil_div(N, BLOCK_N), batch);
-		hipLaunchKernelGGL((k_gemm_nt_mfma<TE, TC>), grid, dim3(256), 0, s, static_cast<const TE*>(A), static_cast<const TE*>(B), static_cast<TC*>(C), M, N, K,
-				lda, ldb, ldc, sA, sB, sC, static_cast<S>(alpha), static_cast<S>(beta), (vec_ok ? 1 : 0) | (vec_c ? 2 : 0));
+		const int flags = (vec_ok ? 1 : 0) | (vec_c ? 2 : 0);
+		const bool small = (static_cast<int64_t>(M) * lda + K) * static_cast<int64_t>(sizeof(TE)) < (1ll << 31)
+				&& (static_cast<int64_t>(N) * ldb + K) * static_cast<int64_t>(sizeof(TE)) < (1ll << 31);
+		const bool fast = vec_ok && small && K % (16 / static_cast<int>(sizeof(TE))) == 0;
+#define AVHIP_GEMM_ARGS static_cast<const TE*>(A), static_cast<const TE*>(B), static_cast<TC*>(C), M, N, K, lda, ldb, ldc, sA, sB, sC, static_cast<S>(alpha), \
+		static_cast<S>(beta), flags
+		if (fast)
+			hipLaunchKernelGGL((k_gemm_nt_mfma<TE, TC, true>), grid, dim3(256), 0, s, AVHIP_GEMM_ARGS);
+		else
+			hipLaunchKernelGGL((k_gemm_nt_mfma<TE, TC, false>), grid, dim3(256), 0, s, AVHIP_GEMM_ARGS);
+#undef AVHIP_GEMM_ARGS
 		return 0;
 	}
 	template<typename TA, typename TC, typename CT>

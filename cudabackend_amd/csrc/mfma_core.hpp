@@ -9,11 +9,11 @@
  *
  * Geometry (one workgroup = 256 work-items = 4 wavefronts of 64):
  *   workgroup tile 128 x 128, wavefront tile 64 x 64 = 2 x 2 MFMA tiles of 32 x 32;
- *   one k-step consumes 64 bytes of every operand row (32 fp16/bf16, 64 int8, 16 fp32 values);
- *   per step each work-item moves two 16-byte chunks of A and two of B: global -> registers -> LDS, the global loads of
- *   step s+1 are issued before the MFMAs of step s (register prefetch) and LDS is double buffered, so there is one
- *   barrier per step;
- *   LDS rows are padded from 64 to 80 bytes so that the 32 rows a wavefront reads with one ds_read_b128 spread over banks.
+ *   one k-step consumes 128 bytes of every operand row (64 fp16/bf16, 128 int8, 32 fp32 values);
+ *   per step each work-item moves four 16-byte chunks of A and four of B: global -> registers -> LDS; global loads run two
+ *   steps ahead of the MFMAs (two register sets) and LDS is double buffered, so there is one barrier per step;
+ *   LDS rows are padded from 128 to 144 bytes so that the 32 rows a wavefront reads with one ds_read_b128 spread over banks;
+ *   two workgroups fit the 160 KB of LDS of a CU.
  * MFMA shapes: v_mfma_f32_32x32x16_{f16,bf16}, v_mfma_i32_32x32x32_i8, v_mfma_f32_32x32x2_f32 (four per 16-byte chunk).
  * Lane l of a wavefront supplies row (l % 32) of the operand tile and the k-chunk (l / 32); it receives, for output column
  * (l % 32), the 16 rows 8*i + 4*(l / 32) + j (i, j < 4).
@@ -104,6 +104,23 @@ namespace avhip
 		}
 		return t.u;
 	}
+	/*
+	 * Fast-path operand fetch: a raw buffer load of 16 bytes at a 32-bit byte offset into a tensor.  The hardware returns
+	 * zeros for offsets beyond the buffer, so "this chunk does not exist" (outside the image, past the last row, past the
+	 * last channel) is expressed by the offset OUT_OF_RANGE: no branch, no select and nothing that would have to wait for
+	 * the data before the next load is issued.  Tensors on this path are smaller than 2 GiB.
+	 */
+	typedef __attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int u32x4_t;
+	constexpr unsigned int OUT_OF_RANGE = 0x80000000u;
+	__device__ inline __amdgpu_buffer_rsrc_t make_buffer(const void *base, unsigned int bytes)
+	{
+		return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+	}
+	__device__ inline uint4 buffer_fetch(__amdgpu_buffer_rsrc_t rsrc, unsigned int byte_offset)
+	{
+		const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(byte_offset), 0, 0);
+		return make_uint4(v[0], v[1], v[2], v[3]);
+	}
 	template<typename TE>
 	__device__ inline uint4 splat_chunk(TE value, int valid)
 	{
@@ -123,26 +140,41 @@ namespace avhip
 
 	constexpr int BLOCK_M = 128;
 	constexpr int BLOCK_N = 128;
-	constexpr int STEP_BYTES = 64; /* bytes of k consumed per row and step */
-	constexpr int LDS_ROW = 80; /* padded row pitch in LDS */
+	constexpr int STEP_BYTES = 128; /* bytes of k consumed per operand row and step */
+	constexpr int STEP_CHUNKS = STEP_BYTES / 16; /* 16-byte chunks per row and step */
+	constexpr int FETCH_ROWS = 256 / STEP_CHUNKS; /* rows covered by one pass of the 256 work-items */
+	constexpr int FETCH_PASSES = BLOCK_M / FETCH_ROWS; /* chunks of each operand a work-item fetches per step */
+	constexpr int LDS_ROW = STEP_BYTES + 16; /* padded row pitch in LDS */
 	constexpr int LDS_TILE = BLOCK_M * LDS_ROW; /* bytes of one operand tile */
 	constexpr int LDS_BYTES = 4 * LDS_TILE; /* A and B, double buffered */
 
 	/*
 	 * Runs the k loop for one 128 x 128 output tile.
-	 *   LoadA(step, q, part) / LoadB(step, q, part) return the 16-byte chunk `part` (0..3) of the 64-byte k-slice `step` of
-	 *   tile row / tile column (t / 4 + 64 * q), q = 0 or 1, where t is the calling work-item; zeros outside the matrix.
-	 * Work-item t thus fetches chunk (t % 4) of rows (t / 4) and (t / 4 + 64) of both operands.
+	 *
+	 * A loader hands out the operand in k order: load(q, part) returns the 16-byte chunk `part` (0..7) of the current
+	 * 128-byte k-slice of tile row (t / 8 + 32 * q), q = 0..3, where t is the calling work-item (zeros outside the matrix
+	 * and for any k-slice at or past `steps`: the pipeline reads up to three slices beyond the end), and next() moves to the
+	 * following k-slice.  Work-item t therefore fetches chunk (t % 8) of four rows of each operand.
+	 *
+	 * Software pipeline, iteration s (register sets R0 / R1 alternate, LDS buffers L0 / L1 alternate):
+	 *     barrier
+	 *     R[s % 2]   <- global(s + 2)             two k-slices ahead of the MFMAs
+	 *     MFMAs of slice s from L[s % 2]
+	 *     L[(s+1) % 2] <- R[(s+1) % 2]            slice s + 1, fetched during iteration s - 1
+	 * so a global load has the MFMAs of two iterations (2 x 16 x 32 cycles per wavefront) to land before it is needed.
 	 * acc[tm][tn] is the (tm, tn) 32 x 32 tile of this wavefront's 64 x 64 quadrant.
 	 */
 	template<typename TE, typename LoadA, typename LoadB>
-	__device__ inline void block_mma(char *lds, int steps, const LoadA &load_a, const LoadB &load_b, typename Mma<TE>::acc_t (&acc)[2][2])
+	__device__ __forceinline__ void block_mma(char *lds, int steps, LoadA &load_a, LoadB &load_b, typename Mma<TE>::acc_t (&acc)[2][2])
 	{
 		const int tid = threadIdx.x;
 		const int lane = tid & 63;
 		const int wave = tid >> 6;
 		const int wm = wave >> 1, wn = wave & 1;
-		const int frow = tid >> 2, fpart = tid & 3;
+		const int fpart = tid & (STEP_CHUNKS - 1);
+		const int st_off = (tid / STEP_CHUNKS) * LDS_ROW + fpart * 16;
+		const int rd_a = (wm * 64 + (lane & 31)) * LDS_ROW + (lane >> 5) * 16;
+		const int rd_b = (wn * 64 + (lane & 31)) * LDS_ROW + (lane >> 5) * 16;
 
 #pragma unroll
 		for (int i = 0; i < 2; i++)
@@ -151,74 +183,118 @@ namespace avhip
 #pragma unroll
 				for (int v = 0; v < 16; v++)
 					acc[i][j][v] = 0;
+		if (steps <= 0)
+			return;
 
-		uint4 ra[2], rb[2];
-		if (steps > 0)
+		uint4 ra[2][FETCH_PASSES], rb[2][FETCH_PASSES];
+		auto fetch = [&](uint4 (&a)[FETCH_PASSES], uint4 (&b)[FETCH_PASSES])
 		{
-			ra[0] = load_a(0, 0, fpart);
-			ra[1] = load_a(0, 1, fpart);
-			rb[0] = load_b(0, 0, fpart);
-			rb[1] = load_b(0, 1, fpart);
-		}
-		const int st_off = frow * LDS_ROW + fpart * 16;
-		const int rd_a = (wm * 64 + (lane & 31)) * LDS_ROW + (lane >> 5) * 16;
-		const int rd_b = (wn * 64 + (lane & 31)) * LDS_ROW + (lane >> 5) * 16;
-
-		for (int step = 0; step < steps; step++)
-		{
-			char *sa = lds + (step & 1) * 2 * LDS_TILE;
-			char *sb = sa + LDS_TILE;
-			*reinterpret_cast<uint4*>(sa + st_off) = ra[0];
-			*reinterpret_cast<uint4*>(sa + st_off + 64 * LDS_ROW) = ra[1];
-			*reinterpret_cast<uint4*>(sb + st_off) = rb[0];
-			*reinterpret_cast<uint4*>(sb + st_off + 64 * LDS_ROW) = rb[1];
-			__syncthreads();
-			if (step + 1 < steps)
-			{
-				ra[0] = load_a(step + 1, 0, fpart);
-				ra[1] = load_a(step + 1, 1, fpart);
-				rb[0] = load_b(step + 1, 0, fpart);
-				rb[1] = load_b(step + 1, 1, fpart);
-			}
 #pragma unroll
-			for (int slab = 0; slab < 2; slab++)
+			for (int q = 0; q < FETCH_PASSES; q++)
 			{
-				Chunk a[2], b[2];
+				a[q] = load_a.load(q, fpart);
+				b[q] = load_b.load(q, fpart);
+			}
+			load_a.next();
+			load_b.next();
+		};
+		auto stash = [&](int buffer, const uint4 (&a)[FETCH_PASSES], const uint4 (&b)[FETCH_PASSES])
+		{
+			char *sa = lds + buffer * 2 * LDS_TILE;
+			char *sb = sa + LDS_TILE;
+#pragma unroll
+			for (int q = 0; q < FETCH_PASSES; q++)
+			{
+				*reinterpret_cast<uint4*>(sa + st_off + q * FETCH_ROWS * LDS_ROW) = a[q];
+				*reinterpret_cast<uint4*>(sb + st_off + q * FETCH_ROWS * LDS_ROW) = b[q];
+			}
+		};
+		auto multiply = [&](int buffer)
+		{
+			const char *sa = lds + buffer * 2 * LDS_TILE;
+			const char *sb = sa + LDS_TILE;
+			constexpr int SLABS = STEP_BYTES / 32;
+			Chunk a[2][2], b[2][2]; /* operands of two consecutive 32-byte slabs: LDS reads run one slab ahead of the MFMAs */
+			auto read = [&](int slab, Chunk (&ra_)[2], Chunk (&rb_)[2])
+			{
 #pragma unroll
 				for (int i = 0; i < 2; i++)
 				{
-					a[i].u = *reinterpret_cast<const uint4*>(sa + rd_a + i * 32 * LDS_ROW + slab * 32);
-					b[i].u = *reinterpret_cast<const uint4*>(sb + rd_b + i * 32 * LDS_ROW + slab * 32);
+					ra_[i].u = *reinterpret_cast<const uint4*>(sa + rd_a + i * 32 * LDS_ROW + slab * 32);
+					rb_[i].u = *reinterpret_cast<const uint4*>(sb + rd_b + i * 32 * LDS_ROW + slab * 32);
 				}
+			};
+			read(0, a[0], b[0]);
+#pragma unroll
+			for (int slab = 0; slab < SLABS; slab++)
+			{
+				if (slab + 1 < SLABS)
+					read(slab + 1, a[(slab + 1) & 1], b[(slab + 1) & 1]);
 #pragma unroll
 				for (int i = 0; i < 2; i++)
 #pragma unroll
 					for (int j = 0; j < 2; j++)
-						Mma<TE>::run(a[i], b[j], acc[i][j]);
+						Mma<TE>::run(a[slab & 1][i], b[slab & 1][j], acc[i][j]);
 			}
+		};
+
+		/* The loop body is branch-free on purpose: the step count is rounded up to even and the loaders return zeros past
+		 * the last k-slice, so the register sets and wait counts are the same in every iteration and a load issued in one
+		 * half-iteration is only waited for one and a half iterations later. */
+		fetch(ra[0], rb[0]);
+		fetch(ra[1], rb[1]);
+		stash(0, ra[0], rb[0]);
+		for (int s = 0; s < steps; s += 2)
+		{
+			__syncthreads();
+			fetch(ra[0], rb[0]);
+			multiply(0);
+			stash(1, ra[1], rb[1]);
+			__syncthreads();
+			fetch(ra[1], rb[1]);
+			multiply(1);
+			stash(0, ra[0], rb[0]);
 		}
 	}
 
 	/*
-	 * Hands the 128 x 128 accumulator tile to the epilogue in row-major order: the accumulators go through LDS (reusing the
-	 * operand buffers, in two halves of 64 rows) so that afterwards each work-item owns 4 consecutive columns of a row and
-	 * 32 neighbouring work-items cover one 128-column row, i.e. global stores are whole contiguous rows.
-	 * f(row, col, v) is called with tile-relative row (0..127), col (multiple of 4) and the four accumulators v[0..3].
-	 * Must be called by all 256 work-items after block_mma.
+	 * Hands an accumulator tile to the epilogue in row-major order.  The workgroup's tile is (2 * TM * 32) rows by 128
+	 * columns when its four wavefronts form a 2 x 2 grid (WAVES_N = 2, wavefront tile TM*32 x 64), or (4 * TM * 32) rows by
+	 * 64 columns when they are stacked (WAVES_N = 1).  The accumulators go through LDS in TM passes so that afterwards each
+	 * work-item owns 4 consecutive columns of a row and neighbouring work-items cover a whole row: global stores are
+	 * contiguous rows.  A work-item always gets the same 4 columns (drain_column()), so per-column constants can be loaded
+	 * once, up front.  f(row, v) is called with the tile-relative row and the four accumulators v[0..3].
+	 * Must be called by all 256 work-items, after the last LDS read of the k loop; `lds` needs drain_bytes<WAVES_N>().
 	 */
-	constexpr int DRAIN_PITCH = 132; /* words per LDS row: 128 + 4 keeps rows 16-byte aligned and staggers banks */
-	template<typename TE, typename F>
-	__device__ inline void drain_tile(char *lds, const typename Mma<TE>::acc_t (&acc)[2][2], const F &f)
+	template<int WAVES_N> struct DrainShape
+	{
+		static constexpr int cols = 64 * WAVES_N; /* columns of the workgroup tile */
+		static constexpr int pitch = cols + 4; /* words per LDS row: keeps rows 16-byte aligned and staggers banks */
+		static constexpr int rows_per_pass = 32 * (4 / WAVES_N); /* one 32-row MFMA tile of every wavefront row */
+		static constexpr int threads_per_row = cols / 4;
+		static constexpr int bytes = rows_per_pass * pitch * 4;
+	};
+	template<int WAVES_N>
+	__device__ inline int drain_column()
+	{
+		return (threadIdx.x % DrainShape<WAVES_N>::threads_per_row) * 4;
+	}
+	template<typename TE, int TM, int WAVES_N, typename F>
+	__device__ __forceinline__ void drain_tile(char *lds, const typename Mma<TE>::acc_t (&acc)[TM][2], const F &f)
 	{
 		typedef typename Mma<TE>::scalar_t S;
-		static_assert(sizeof(S) == 4 && 64 * DRAIN_PITCH * 4 <= LDS_BYTES, "drain buffer must fit the operand buffers");
+		typedef DrainShape<WAVES_N> D;
+		static_assert(sizeof(S) == 4, "accumulators are 32-bit");
 		S *sm = reinterpret_cast<S*>(lds);
 		const int tid = threadIdx.x;
 		const int lane = tid & 63;
 		const int wave = tid >> 6;
-		const int wm = wave >> 1, wn = wave & 1;
+		const int wm = WAVES_N == 2 ? (wave >> 1) : wave;
+		const int wn = WAVES_N == 2 ? (wave & 1) : 0;
+		const int col = drain_column<WAVES_N>();
+		constexpr int ROW_STEP = 256 / D::threads_per_row; /* rows covered by one sweep of the workgroup */
 #pragma unroll
-		for (int tm = 0; tm < 2; tm++)
+		for (int tm = 0; tm < TM; tm++)
 		{
 			__syncthreads();
 #pragma unroll
@@ -227,15 +303,15 @@ namespace avhip
 				for (int i = 0; i < 4; i++)
 #pragma unroll
 					for (int j = 0; j < 4; j++)
-						sm[(wm * 32 + 8 * i + 4 * (lane >> 5) + j) * DRAIN_PITCH + wn * 64 + tn * 32 + (lane & 31)] = acc[tm][tn][4 * i + j];
+						sm[(wm * 32 + 8 * i + 4 * (lane >> 5) + j) * D::pitch + wn * 64 + tn * 32 + (lane & 31)] = acc[tm][tn][4 * i + j];
 			__syncthreads();
-			for (int e = tid; e < 64 * 32; e += 256)
+#pragma unroll
+			for (int it = 0; it < D::rows_per_pass / ROW_STEP; it++)
 			{
-				const int rl = e >> 5;
-				const int col = (e & 31) * 4;
-				const int row = (rl >> 5) * 64 + tm * 32 + (rl & 31);
-				const Pack<S, 4> p = *reinterpret_cast<const Pack<S, 4>*>(sm + rl * DRAIN_PITCH + col);
-				f(row, col, p.v);
+				const int rl = tid / D::threads_per_row + it * ROW_STEP; /* row within this pass */
+				const int row = (rl >> 5) * (TM * 32) + tm * 32 + (rl & 31);
+				const Pack<S, 4> p = *reinterpret_cast<const Pack<S, 4>*>(sm + rl * D::pitch + col);
+				f(row, p.v);
 			}
 		}
 	}
