@@ -41,19 +41,24 @@ namespace avhip
 		c.u = static_cast<uint32_t>(v.bits) << 16;
 		return c.f;
 	}
+	/* Round to nearest even.  On the device this is the single v_cvt_pk_bf16_f32 instruction of gfx950. */
 	__host__ __device__ inline bf16_t float_to_bf16(float f)
 	{
+		bf16_t r;
+#if defined(__HIP_DEVICE_COMPILE__)
+		r.bits = __builtin_bit_cast(unsigned short, static_cast<__bf16>(f));
+#else
 		union
 		{
 			uint32_t u;
 			float f;
 		} c;
 		c.f = f;
-		bf16_t r;
 		if ((c.u & 0x7FFFFFFFu) > 0x7F800000u) // NaN stays NaN
 			r.bits = static_cast<uint16_t>((c.u >> 16) | 0x0040u);
 		else
 			r.bits = static_cast<uint16_t>((c.u + 0x7FFFu + ((c.u >> 16) & 1u)) >> 16);
+#endif
 		return r;
 	}
 
@@ -132,6 +137,16 @@ namespace avhip
 				if (i < valid)
 					ptr[i] = Traits<T>::store(in[i]);
 		}
+	}
+
+	/* Makes a wavefront-uniform 32-bit value live in a scalar register from here on.  Kernel arguments sit in memory and the
+	 * compiler is free to re-load them wherever they are used; in fully unrolled epilogues that puts a scalar load and a
+	 * wait in front of every store.  Passing the value through an empty asm statement makes it opaque, so it is loaded once.
+	 * Not for pointers: a pointer that went through asm loses its address space and every access becomes a slow flat access. */
+	template<typename T>
+	__device__ __forceinline__ void keep_in_sgpr(T &v)
+	{
+		asm volatile("" : "+s"(v));
 	}
 
 	/* Forward activations, src/activations.cuh:202-425 of the reference. */

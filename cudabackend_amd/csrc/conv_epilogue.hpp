@@ -57,17 +57,27 @@ namespace avhip
 		int activation, K;
 		bool vec; /* y / z rows may be accessed as 4-element vectors */
 
+		/* call once on the kernel's copy before the k loop: the members are then read from scalar registers */
+		__device__ __forceinline__ void pin()
+		{
+			keep_in_sgpr(alpha1);
+			keep_in_sgpr(alpha2);
+			keep_in_sgpr(beta);
+			keep_in_sgpr(activation);
+			keep_in_sgpr(K);
+		}
 		__device__ __forceinline__ void load_columns(int k, Columns &c) const
 		{
 #pragma unroll
 			for (int q = 0; q < 4; q++)
 				c.bias[q] = (bias != nullptr && k + q < K) ? bias[k + q] : 0.0f;
 		}
-		/* p: index of the output pixel (row of y), k: first of the four filters */
-		template<int ACT>
+		/* p: index of the output pixel (row of y), k: first of the four filters.  VEC instances require `vec`. */
+		template<int ACT, bool VEC = false>
 		__device__ __forceinline__ void store(int64_t p, int k, const float (&v)[4], const Columns &c) const
 		{
-			const int valid = K - k;
+			const bool vec = VEC || this->vec;
+			const int valid = VEC ? 4 : K - k;
 			const int64_t idx = p * K + k;
 			float t[4];
 #pragma unroll
@@ -125,6 +135,14 @@ namespace avhip
 		int activation, K;
 		bool vec;
 
+		__device__ __forceinline__ void pin()
+		{
+			keep_in_sgpr(alpha1);
+			keep_in_sgpr(alpha2);
+			keep_in_sgpr(beta);
+			keep_in_sgpr(activation);
+			keep_in_sgpr(K);
+		}
 		__device__ __forceinline__ void load_columns(int k, Columns &c) const
 		{
 #pragma unroll
@@ -136,13 +154,14 @@ namespace avhip
 				c.scale[q] = (MODE == I8_REQUANT && in) ? scale[k + q] : 0.0f;
 			}
 		}
-		template<int ACT>
+		template<int ACT, bool VEC = false>
 		__device__ __forceinline__ void store(int64_t p, int k, const int (&v)[4], const Columns &c) const
 		{
 			/* every fp32 operation below rounds exactly once: a * b + c must not become a fused multiply-add.  The pragma
 			 * governs the expressions written in this block, which is why they use plain operators and no intrinsics. */
 #pragma clang fp contract(off)
-			const int valid = K - k;
+			const bool vec = VEC || this->vec;
+			const int valid = VEC ? 4 : K - k;
 			const int64_t idx = p * K + k;
 			if (MODE == I8_EXACT || MODE == I8_REQUANT)
 			{

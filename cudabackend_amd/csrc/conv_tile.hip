@@ -46,6 +46,12 @@ namespace
 	template<typename TE, typename Epi>
 	__global__ __launch_bounds__(256, 2) void k_conv_tile(const TE *__restrict__ x, const TE *__restrict__ w, TileGeom g, Epi epi)
 	{
+		epi.pin();
+		keep_in_sgpr(g.TW);
+		keep_in_sgpr(g.TH);
+		keep_in_sgpr(g.Ho);
+		keep_in_sgpr(g.Wo);
+		keep_in_sgpr(g.K);
 		__shared__ __attribute__((aligned(16))) char lds[TILE_LDS];
 		char *halo = lds;
 		char *filt = lds + HALO_BYTES;
@@ -232,7 +238,7 @@ namespace
 			const int py = row / g.TW, px = row - py * g.TW;
 			const int oh = oh0 + py, ow = ow0 + px;
 			if (row < g.TH * g.TW && oh < g.Ho && ow < g.Wo && kcol < g.K)
-				epi.template store<ACT_SIMPLE>((static_cast<int64_t>(n) * g.Ho + oh) * g.Wo + ow, kcol, v, columns);
+				epi.template store<ACT_SIMPLE, true>((static_cast<int64_t>(n) * g.Ho + oh) * g.Wo + ow, kcol, v, columns);
 		});
 	}
 
@@ -265,6 +271,8 @@ namespace avhip
 	bool conv_tile_launch(hipStream_t stream, const avhipConvShape &s, const void *x, const void *w, const Epi &epi)
 	{
 		if (s.stride_h != 1 || s.stride_w != 1 || s.dil_h != 1 || s.dil_w != 1)
+			return false;
+		if (!epi.vec) /* the kernel stores whole 4-filter vectors: K is a multiple of 4 and y, z are aligned */
 			return false;
 		TileGeom g;
 		if (!choose_tile(s, g))

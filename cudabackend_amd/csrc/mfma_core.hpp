@@ -305,13 +305,18 @@ namespace avhip
 					for (int j = 0; j < 4; j++)
 						sm[(wm * 32 + 8 * i + 4 * (lane >> 5) + j) * D::pitch + wn * 64 + tn * 32 + (lane & 31)] = acc[tm][tn][4 * i + j];
 			__syncthreads();
+			/* all LDS reads of the pass first, then the stores: the reads are independent and overlap */
+			constexpr int ITERS = D::rows_per_pass / ROW_STEP;
+			Pack<S, 4> vals[ITERS];
 #pragma unroll
-			for (int it = 0; it < D::rows_per_pass / ROW_STEP; it++)
+			for (int it = 0; it < ITERS; it++)
+				vals[it] = *reinterpret_cast<const Pack<S, 4>*>(sm + (tid / D::threads_per_row + it * ROW_STEP) * D::pitch + col);
+#pragma unroll
+			for (int it = 0; it < ITERS; it++)
 			{
 				const int rl = tid / D::threads_per_row + it * ROW_STEP; /* row within this pass */
 				const int row = (rl >> 5) * (TM * 32) + tm * 32 + (rl & 31);
-				const Pack<S, 4> p = *reinterpret_cast<const Pack<S, 4>*>(sm + rl * D::pitch + col);
-				f(row, p.v);
+				f(row, vals[it].v);
 			}
 		}
 	}
