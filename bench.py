@@ -162,10 +162,10 @@ def time_tower(hip, ctx, dtype, steps, warmup):
         tower.step()  # also fills the library's transformed-weight cache, so that nothing allocates during capture
     ctx.synchronize()
     full = hip.capture(stream, tower.step)
-    stem = hip.capture(stream, tower.stem)
+    stem = hip.capture(stream, lambda: [tower.stem() for _ in range(10)])
     hip.sync()
     ms_step = hip.time_graph(full, stream, steps, warmup)
-    ms_stem = hip.time_graph(stem, stream, max(steps, 10), warmup)
+    ms_stem = hip.time_graph(stem, stream, max(steps, 10), warmup) / 10
     ctx.synchronize()
     body_us = (ms_step - ms_stem) * 1e3 / (2 * tower.blocks)
     out = {"ms_per_step": ms_step, "tflops": tower.flops_step / (ms_step * 1e-3) / 1e12, "stem_conv_us": ms_stem * 1e3,
@@ -269,6 +269,19 @@ def copy_bandwidth(hip, ctx, iters=10):
     return 2.0 * nbytes / (ms * 1e-3) / 1e9
 
 
+def counter_calibration(ctx, launches=3):
+    """Launches a plain streaming kernel of known traffic (fp32 -> fp16 conversion of 2^26 elements: 256 MiB read, 128 MiB
+    written).  Under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its reading fixes the factor between the counter and bytes."""
+    lib = cb.load_library()
+    n = 1 << 26
+    a, b = cb.DeviceTensor((n,), cb.DTYPE_FLOAT32), cb.DeviceTensor((n,), cb.DTYPE_FLOAT16)
+    for _ in range(launches):
+        cb.check(lib.cudaChangeType(ctx.handle, b.mem, cb.DTYPE_FLOAT16, a.mem, cb.DTYPE_FLOAT32, n), "cudaChangeType")
+    ctx.synchronize()
+    a.close()
+    b.close()
+
+
 def cpu_baseline(seconds=12.0):
     """fp32 direct convolution of the body layer (128->128, 15x15, 3x3) on a batch slice, all host cores."""
     from oracle import oracle as orc
@@ -297,6 +310,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--quick", action="store_true", help="headline tower only (no side legs, no CPU baseline)")
+    ap.add_argument("--calibrate", action="store_true", help="also launch a streaming kernel of known traffic (for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards over the batch with no collectives)." % args.gpus,
@@ -311,6 +325,8 @@ def main():
     head = time_tower(hip, ctx, args.dtype, args.steps, args.warmup)
     detail = {"headline": head}
     cpu = None
+    if args.calibrate:
+        counter_calibration(ctx)
     if not args.quick:
         it = max(5, args.steps)
         for other in ("f32", "bf16", "f16"):

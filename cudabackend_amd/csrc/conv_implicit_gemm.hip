@@ -250,6 +250,169 @@ namespace
 		}
 	};
 
+	/*
+	 * Few input channels (a network's first layer: 3 or 4 planes): one tap holds far less than a 128-byte k-step, so k is
+	 * taken as the flattened (tap, channel) index of the filter row, R*S*C elements long, and a 16-byte chunk is gathered
+	 * from 16 / PB pieces of PB bytes, each from the tap it falls into.  PB is the largest power of two (2..16) that divides
+	 * the bytes of one pixel, so a piece never straddles two taps.  Which tap a piece belongs to does not depend on the
+	 * output pixel: it is worked out once per k-step; per pixel there is the window origin and the inside-mask as in the
+	 * fast loader.  Same preconditions as the fast loader (zero padding value, 32-bit offsets, at most 32 taps).
+	 */
+	template<int PB> struct Piece;
+	template<> struct Piece<16>
+	{
+		typedef u32x4_t type;
+		__device__ static inline type get(__amdgpu_buffer_rsrc_t r, unsigned int off)
+		{
+			return __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(off), 0, 0);
+		}
+	};
+	template<> struct Piece<8>
+	{
+		typedef __attribute__((__vector_size__(2 * sizeof(unsigned int)))) unsigned int type;
+		__device__ static inline type get(__amdgpu_buffer_rsrc_t r, unsigned int off)
+		{
+			return __builtin_amdgcn_raw_buffer_load_b64(r, static_cast<int>(off), 0, 0);
+		}
+	};
+	template<> struct Piece<4>
+	{
+		typedef unsigned int type;
+		__device__ static inline type get(__amdgpu_buffer_rsrc_t r, unsigned int off)
+		{
+			return __builtin_amdgcn_raw_buffer_load_b32(r, static_cast<int>(off), 0, 0);
+		}
+	};
+	template<> struct Piece<2>
+	{
+		typedef unsigned short type;
+		__device__ static inline type get(__amdgpu_buffer_rsrc_t r, unsigned int off)
+		{
+			return __builtin_amdgcn_raw_buffer_load_b16(r, static_cast<int>(off), 0, 0);
+		}
+	};
+	template<int PB>
+	union PieceChunk
+	{
+		uint4 u;
+		typename Piece<PB>::type piece[16 / PB];
+	};
+
+	template<typename TE, int PB>
+	struct PackedPixelLoader
+	{
+		static constexpr int NP = 16 / PB;
+		__amdgpu_buffer_rsrc_t rsrc;
+		const ConvGeom &g;
+		unsigned int origin[FETCH_PASSES]; /* byte offset of (n, ih0, iw0, 0) */
+		unsigned int inside[FETCH_PASSES]; /* bit t: tap t reads a pixel inside the image */
+		unsigned int rel[NP]; /* byte offset of each piece of the current k-step relative to the window origin */
+		unsigned int bit[NP]; /* the piece's tap as a mask bit; 0 when the piece lies past the end of k */
+		unsigned int k_byte; /* flattened-k byte position of this work-item's chunk in the current step */
+
+		__device__ inline PackedPixelLoader(const TE *x, const ConvGeom &g_, int64_t p0) :
+				g(g_)
+		{
+			rsrc = make_buffer(x, static_cast<unsigned int>(g.images * g.H * g.W * g.C * sizeof(TE)));
+			const unsigned int CB = g.C * sizeof(TE);
+#pragma unroll
+			for (int q = 0; q < FETCH_PASSES; q++)
+			{
+				const unsigned int p = static_cast<unsigned int>(p0) + threadIdx.x / STEP_CHUNKS + FETCH_ROWS * q;
+				const bool ok = p < static_cast<unsigned int>(g.pixels);
+				const unsigned int pp = ok ? p : 0u;
+				const unsigned int row = pp / static_cast<unsigned int>(g.Wo);
+				const int ow = static_cast<int>(pp - row * g.Wo);
+				const unsigned int n = row / static_cast<unsigned int>(g.Ho);
+				const int oh = static_cast<int>(row - n * g.Ho);
+				const int ih0 = oh * g.stride_h + g.pad_h;
+				const int iw0 = ow * g.stride_w + g.pad_w;
+				origin[q] = static_cast<unsigned int>((static_cast<int>(n * g.H + ih0) * g.W + iw0)) * CB;
+				unsigned int m = 0;
+				for (int t = 0; t < g.R * g.S; t++)
+				{
+					int i = t / g.S, j = t - (t / g.S) * g.S;
+					if (g.flip)
+					{
+						i = g.R - 1 - i;
+						j = g.S - 1 - j;
+					}
+					const int ih = ih0 + i * g.dil_h, iw = iw0 + j * g.dil_w;
+					if (ok && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
+						m |= 1u << t;
+				}
+				inside[q] = m;
+			}
+			k_byte = (threadIdx.x % STEP_CHUNKS) * 16;
+			place();
+		}
+		__device__ inline void place()
+		{
+			const unsigned int CB = g.C * sizeof(TE);
+			const unsigned int k_bytes = g.R * g.S * CB;
+#pragma unroll
+			for (int e = 0; e < NP; e++)
+			{
+				const unsigned int b = k_byte + e * PB;
+				const unsigned int tap = b / CB;
+				const unsigned int within = b - tap * CB;
+				int i = tap / g.S, j = tap - (tap / g.S) * g.S;
+				if (g.flip)
+				{
+					i = g.R - 1 - i;
+					j = g.S - 1 - j;
+				}
+				rel[e] = static_cast<unsigned int>((i * g.dil_h) * g.W + j * g.dil_w) * CB + within;
+				bit[e] = b < k_bytes ? 1u << (tap & 31u) : 0u;
+			}
+		}
+		__device__ inline uint4 load(int q, int) const
+		{
+			PieceChunk<PB> c;
+#pragma unroll
+			for (int e = 0; e < NP; e++)
+				c.piece[e] = Piece<PB>::get(rsrc, (inside[q] & bit[e]) != 0u ? origin[q] + rel[e] : OUT_OF_RANGE);
+			return c.u;
+		}
+		__device__ inline void next()
+		{
+			k_byte += STEP_BYTES;
+			place();
+		}
+	};
+	template<typename TE, int PB>
+	struct PackedFilterLoader
+	{
+		static constexpr int NP = 16 / PB;
+		__amdgpu_buffer_rsrc_t rsrc;
+		unsigned int origin[FETCH_PASSES]; /* byte offset of row k of w; OUT_OF_RANGE for k >= K */
+		unsigned int k_byte, k_bytes;
+		__device__ inline PackedFilterLoader(const TE *w, const ConvGeom &g, int k0)
+		{
+			k_bytes = g.R * g.S * g.C * sizeof(TE);
+			rsrc = make_buffer(w, static_cast<unsigned int>(g.K) * k_bytes);
+#pragma unroll
+			for (int q = 0; q < FETCH_PASSES; q++)
+			{
+				const int k = k0 + threadIdx.x / STEP_CHUNKS + FETCH_ROWS * q;
+				origin[q] = k < g.K ? static_cast<unsigned int>(k) * k_bytes : OUT_OF_RANGE;
+			}
+			k_byte = (threadIdx.x % STEP_CHUNKS) * 16;
+		}
+		__device__ inline uint4 load(int q, int) const
+		{
+			PieceChunk<PB> c;
+#pragma unroll
+			for (int e = 0; e < NP; e++)
+				c.piece[e] = Piece<PB>::get(rsrc, k_byte + e * PB < k_bytes ? origin[q] + k_byte + e * PB : OUT_OF_RANGE);
+			return c.u;
+		}
+		__device__ inline void next()
+		{
+			k_byte += STEP_BYTES;
+		}
+	};
+
 	/* One kernel for every epilogue: Epi is FloatEpilogue<TE> or Int8Epilogue<mode>.  FAST instances use the branch-free
 	 * loaders and are launched for LINEAR / RELU only; everything else runs the general instance. */
 	template<typename TE, bool FAST, typename Epi>
@@ -271,6 +434,28 @@ namespace
 			const int64_t p = p0 + r;
 			if (p < g.pixels && k < g.K)
 				epi.template store<FAST ? ACT_SIMPLE : ACT_ANY>(p, k, v, columns);
+		});
+	}
+
+	template<typename TE, int PB, typename Epi>
+	__global__ __launch_bounds__(256, 2) void k_conv_igemm_packed(const TE *__restrict__ x, const TE *__restrict__ w, ConvGeom g, Epi epi)
+	{
+		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
+		const int64_t p0 = static_cast<int64_t>(blockIdx.x) * BLOCK_M;
+		const int k = blockIdx.y * BLOCK_N + drain_column<2>();
+		typename Epi::Columns columns;
+		epi.load_columns(k, columns);
+
+		PackedPixelLoader<TE, PB> la(x, g, p0);
+		PackedFilterLoader<TE, PB> lb(w, g, blockIdx.y * BLOCK_N);
+		typename Mma<TE>::acc_t acc[2][2];
+		block_mma<TE>(lds, (g.R * g.S * g.C * static_cast<int>(sizeof(TE)) + STEP_BYTES - 1) / STEP_BYTES, la, lb, acc);
+
+		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const typename Epi::scalar_t (&v)[4]) __attribute__((always_inline))
+		{
+			const int64_t p = p0 + r;
+			if (p < g.pixels && k < g.K)
+				epi.template store<ACT_SIMPLE>(p, k, v, columns);
 		});
 	}
 
@@ -333,6 +518,34 @@ namespace
 			std::memset(&padv, 0, sizeof(TE));
 		const dim3 grid(ceil_div(g.pixels, BLOCK_M), ceil_div(s.K, BLOCK_N));
 		const bool fast = fast_path_ok<TE>(s, flags, padding_value) && is_simple_activation(epi.activation);
+		/* few input channels: pack (tap, channel) into the k-steps instead of spending a step per tap */
+		const int pixel_bytes = s.C * static_cast<int>(sizeof(TE));
+		if (pixel_bytes <= STEP_BYTES / 2 && s.R * s.S > 1 && fast_path_ok<TE>(s, 1, padding_value) && is_simple_activation(epi.activation))
+		{
+			int pb = 16;
+			while (pb > 1 && (pixel_bytes % pb != 0 || !aligned_to(x, pb) || !aligned_to(w, pb)))
+				pb /= 2;
+			pb = pb < static_cast<int>(sizeof(TE)) ? 0 : pb;
+#define AVHIP_PACKED(PB) hipLaunchKernelGGL((k_conv_igemm_packed<TE, PB, Epi>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi)
+			switch (pb)
+			{
+				case 16:
+					AVHIP_PACKED(16);
+					return 0;
+				case 8:
+					AVHIP_PACKED(8);
+					return 0;
+				case 4:
+					AVHIP_PACKED(4);
+					return 0;
+				case 2:
+					AVHIP_PACKED(2);
+					return 0;
+				default:
+					break;
+			}
+#undef AVHIP_PACKED
+		}
 		/* stride-1 filters with more than one tap first try the kernel that keeps an image tile resident in LDS */
 		if (fast && s.R * s.S > 1 && conv_tile_launch<TE, Epi>(st, s, x, w, epi))
 			return 0;

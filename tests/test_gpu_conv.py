@@ -66,6 +66,46 @@ def test_implicit_gemm_geometry(oracle, dtype, case):
     assert oracle.rel_l2(got, want) < BAR[dtype]
 
 
+FEW_CHANNELS = [
+    dict(x=(3, 15, 15, 4), w=(128, 3, 3, 4), pad=(-1, -1)),                                       # the tower's stem
+    dict(x=(2, 9, 10, 3), w=(24, 3, 3, 3), pad=(-1, -1)),                                         # RGB
+    dict(x=(2, 9, 10, 1), w=(24, 5, 5, 1), pad=(-2, -2), mode=1),                                 # one plane, flipped 5x5
+    dict(x=(2, 11, 9, 2), w=(8, 3, 3, 2), pad=(-1, -1), stride=(2, 1)),
+    dict(x=(2, 12, 12, 8), w=(40, 3, 3, 8), pad=(-2, -2), dilation=(2, 2)),
+    dict(x=(2, 8, 9, 12), w=(136, 3, 3, 12), pad=(-1, -1)),                                       # k spans several steps, two filter blocks
+    dict(x=(1, 7, 7, 16), w=(16, 5, 5, 16), pad=(-2, -2)),
+    dict(x=(1, 7, 7, 5), w=(16, 3, 3, 5), pad=(0, 0)),                                            # valid convolution, odd channel count
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", FEW_CHANNELS, ids=[str(i) for i in range(len(FEW_CHANNELS))])
+def test_implicit_gemm_few_input_channels(oracle, dtype, case):
+    """First-layer shapes: (tap, channel) packed into the k-steps; bias, residual and ReLU fused as in the tower."""
+    g = h.rng(26)
+    x = h.rounded(oracle, g.standard_normal(case["x"]), dtype)
+    w = he(g, case["w"], dtype, oracle)
+    ys = out_shape(oracle, case)
+    b = g.uniform(-0.1, 0.1, ys[3]).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal(ys), dtype)
+    kw = dict(pad=case["pad"], stride=case.get("stride", (1, 1)), dilation=case.get("dilation", (1, 1)), mode=case.get("mode", 0))
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, bias=b, z=z, activation=cb.ACTIVATION_RELU, **kw)
+    want = oracle.conv2d(x, w, b, z, activation=oracle.RELU, **kw)
+    assert got.shape == want.shape
+    assert oracle.rel_l2(got, want) < BAR[dtype]
+
+
+@pytest.mark.parametrize("case", FEW_CHANNELS, ids=[str(i) for i in range(len(FEW_CHANNELS))])
+def test_int8_few_input_channels_bit_exact(oracle, case):
+    g = h.rng(27)
+    x = g.integers(-127, 128, case["x"], dtype=np.int8)
+    w = g.integers(-127, 128, case["w"], dtype=np.int8)
+    b = g.integers(-2 ** 15, 2 ** 15, case["w"][0]).astype(np.int32)
+    kw = dict(pad=case["pad"], stride=case.get("stride", (1, 1)), dilation=case.get("dilation", (1, 1)), mode=case.get("mode", 0))
+    got = h.conv_forward("implicit_gemm", x, w, out_shape(oracle, case), "i8", y_dtype="i32", bias=b, bias_dtype="i32", activation=cb.ACTIVATION_RELU, **kw)
+    np.testing.assert_array_equal(got, oracle.conv2d_i8(x, w, b, activation=cb.ACTIVATION_RELU, **kw))
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_implicit_gemm_full_epilogue(oracle, dtype):
     """alpha1, alpha2, beta, bias, residual and every activation, in the order of the reference's epilogue
