@@ -30,6 +30,10 @@ import cudabackend_amd as cb  # noqa: E402
 PEAK = {"hbm_GBs": 8000.0, "bf16": 2500.0, "f16": 2500.0, "i8": 5000.0, "f32": 157.3}
 DT = {"bf16": cb.DTYPE_BFLOAT16, "f16": cb.DTYPE_FLOAT16, "f32": cb.DTYPE_FLOAT32, "i8": cb.DTYPE_INT8}
 SEED = 0xA70CAD0
+# HBM bytes per launch of the body convolution kernel (read + written, average over the residual and non-residual launches of a
+# pass), from the FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/conv_tile_bf16_cfg2_hbm_traffic.md.  Counters
+# cannot be read from inside this process, so the figure is carried here; it is only reported for the dtype it was taken on.
+COUNTED_TRAFFIC_BYTES = {"bf16": 39.49e6}
 
 
 class Hip:
@@ -349,7 +353,7 @@ def main():
         "config": {"workload": "BASELINE config 2: residual tower N=256 15x15 128ch, stem 4->128 + 10 blocks (21 3x3 convs), NHWC, bias+ReLU+residual fused",
                    "global_batch": 256, "entry": "cudaConvolutionBiasActivationForward"},
         "roofline": {"bound": "mfma", "achieved": head["body_conv_tflops"], "peak": peak, "unit": "TFLOP/s", "frac": head["body_conv_tflops"] / peak,
-                     "traffic": None, "kernel": "body 3x3 conv 128->128: direct-equivalent flops / ((graph-replayed pass - stem) / 20) by HIP events"},
+                     "traffic": COUNTED_TRAFFIC_BYTES.get(args.dtype), "kernel": "body 3x3 conv 128->128: direct-equivalent flops / ((graph-replayed pass - stem) / 20) by HIP events"},
         "cpu_baseline": cpu,
         "detail": detail,
     }
