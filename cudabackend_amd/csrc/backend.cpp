@@ -1428,8 +1428,11 @@ namespace avocado
 				return st;
 			const ConvProblem &p = call.problem;
 			const bool bias_fp32 = call.bias == nullptr || call.bias_dtype == AVOCADO_DTYPE_FLOAT32;
-			/* 3x3 / stride 1 on floating tensors with enough channels to fill the matrix cores: fused Winograd */
-			if (fused_winograd_applicable(p) && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32 && p.shape.Ho == p.shape.H && p.shape.Wo == p.shape.W)
+			/* 3x3 / stride 1 on fp32 tensors with enough channels to fill the matrix cores: fused Winograd, whose 2.25-fold saving
+			 * of multiplications is worth more than its transform work at the fp32 MFMA rate.  At the 16-bit MFMA rate the
+			 * convolution is bound by LDS traffic, not by the matrix cores, and the direct image-tile kernel is faster. */
+			if (fused_winograd_applicable(p) && p.x_dtype == AVOCADO_DTYPE_FLOAT32 && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32
+					&& p.shape.Ho == p.shape.H && p.shape.Wo == p.shape.W)
 			{
 				const avStatus_t fs = run_fused_winograd(call, wMem, yMem, activation);
 				if (fs != AVOCADO_STATUS_NOT_SUPPORTED)

@@ -135,6 +135,77 @@ def test_implicit_gemm_padding_value(oracle):
     assert oracle.rel_l2(got, want) < 1e-5
 
 
+# ---- fused Winograd F(2x2, 3x3) ------------------------------------------------------------------------------------------
+WINOGRAD_BAR = {"f32": 1e-4, "f16": 2e-3, "bf16": 2e-3}
+
+FUSED_CASES = [
+    dict(x=(8, 15, 15, 64), w=(64, 3, 3, 64), pad=(-1, -1)),        # config 1
+    dict(x=(2, 13, 14, 40), w=(21, 3, 3, 40), pad=(-1, -1)),        # odd extents, ragged filters (scalar stores)
+    dict(x=(1, 33, 35, 32), w=(32, 3, 3, 32), pad=(-1, -1)),        # several tile blocks per image, partial ones at the edges
+    dict(x=(2, 9, 9, 136), w=(136, 3, 3, 136), pad=(-1, -1)),       # more than one channel block and more than one filter block
+    dict(x=(2, 12, 11, 32), w=(48, 3, 3, 32), pad=(0, 0)),          # valid convolution: output smaller than input
+    dict(x=(2, 6, 7, 32), w=(32, 3, 3, 32), pad=(-2, -2)),          # full convolution: output larger than input
+    dict(x=(2, 10, 10, 48), w=(40, 3, 3, 48), pad=(-1, -1), mode=1),  # kernel rotated by 180 degrees
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", FUSED_CASES, ids=[str(i) for i in range(len(FUSED_CASES))])
+def test_winograd_fused_geometry(oracle, dtype, case):
+    g = h.rng(30)
+    x = h.rounded(oracle, g.standard_normal(case["x"]), dtype)
+    w = he(g, case["w"], dtype, oracle)
+    ys = out_shape(oracle, case)
+    b = g.uniform(-0.1, 0.1, ys[3]).astype(np.float32).astype(np.float64)
+    kw = dict(pad=case["pad"], mode=case.get("mode", 0))
+    got = h.conv_forward("winograd_fused", x, w, ys, dtype, bias=b, activation=cb.ACTIVATION_RELU, **kw)
+    want = oracle.conv2d(x, w, b, activation=oracle.RELU, **kw)
+    assert got.shape == want.shape
+    err = oracle.rel_l2(got, want)
+    print("fused winograd %s case %s rel-L2 = %.3e" % (dtype, case["x"], err))
+    assert err < WINOGRAD_BAR[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_winograd_fused_full_epilogue(oracle, dtype):
+    g = h.rng(31)
+    x = h.rounded(oracle, g.standard_normal((2, 9, 9, 32)), dtype)
+    w = he(g, (24, 3, 3, 32), dtype, oracle)
+    b = g.uniform(-0.1, 0.1, 24).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal((2, 9, 9, 24)), dtype)
+    y0 = h.rounded(oracle, g.standard_normal((2, 9, 9, 24)), dtype)
+    a1, a2, be = float(np.float32(1.1)), float(np.float32(1.2)), float(np.float32(0.1))
+    for act in range(9):
+        got = h.conv_forward("winograd_fused", x, w, y0.shape, dtype, bias=b, z=z, y0=y0, alpha1=a1, alpha2=a2, beta=be, activation=act)
+        want = oracle.conv2d(x, w, b, z, y0, alpha1=a1, alpha2=a2, beta=be, activation=act)
+        slack = 2 if act == cb.ACTIVATION_EXPONENTIAL else 1  # see test_implicit_gemm_full_epilogue
+        assert oracle.rel_l2(got, want) < WINOGRAD_BAR[dtype] * slack, act
+
+
+def test_winograd_fused_sees_rewritten_weights(oracle):
+    """The transformed weights are cached per memory block and version: a second call after the weights were overwritten
+    through the API must use the new ones."""
+    g = h.rng(32)
+    x = h.rounded(oracle, g.standard_normal((1, 8, 8, 32)), "f32")
+    w1 = he(g, (32, 3, 3, 32), "f32", oracle)
+    w2 = he(g, (32, 3, 3, 32), "f32", oracle)
+    with h.Call() as c:
+        conv = cb.ConvolutionDescriptor(padding=(-1, -1), dtype=cb.DTYPE_FLOAT32)
+        xt, wt, y = c.tensor(x, "f32"), c.tensor(w1, "f32"), c.empty((1, 8, 8, 32), "f32")
+
+        def run():
+            st = c.lib.cudaConvolutionWinogradFusedForward(c.ctx.handle, conv.handle, None, xt.desc, xt.mem, wt.desc, wt.mem, 0, 0, None, 0, 0, None,
+                                                           y.desc, y.mem, cb.ACTIVATION_LINEAR)
+            assert st == cb.STATUS_SUCCESS
+            c.finish()
+            return y.download()
+        first = run()
+        wt.upload(w2)
+        second = run()
+    assert oracle.rel_l2(first, oracle.conv2d(x, w1)) < 1e-4
+    assert oracle.rel_l2(second, oracle.conv2d(x, w2)) < 1e-4
+
+
 # ---- int8 ------------------------------------------------------------------------------------------------------------
 INT8_CASES = [
     dict(x=(4, 20, 20, 128), w=(128, 3, 3, 128), pad=(-1, -1)),      # config 4 at a reduced batch
