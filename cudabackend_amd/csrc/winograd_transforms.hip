@@ -14,7 +14,9 @@
  *  - the matrix dtype is independent of the tensor dtype (fp16 or fp32 matrices for 16-bit tensors keep F(4x4,3x3) usable);
  *  - 16-bit values are computed in fp32 and rounded to nearest even on store.
  */
-#include "common.hpp"
+#include <type_traits>
+
+#include "conv_epilogue.hpp"
 
 namespace
 {
@@ -149,24 +151,33 @@ namespace
 		}
 	}
 
-	template<int M, int R, typename T, typename TM, int V>
+	/* IDX is the integer type of the work-item and tile indices: 32 bits whenever the problem allows it (64-bit divisions
+	 * cost more than the transform itself).  V > 1 instances are launched only when every vector is complete and aligned:
+	 * they have no tail handling, and outside the image they load from a clamped address and select the padding value, so
+	 * the whole work-item is branch-free and all its loads are in flight together. */
+	template<int M, int R, typename T, typename TM, int V, typename IDX>
 	__global__ __launch_bounds__(256) void k_input_transform(const T *__restrict__ x, TM *__restrict__ Vm, int N, int H, int W, int C, int Th, int Tw,
 			int pad_h, int pad_w, typename Traits<T>::compute padv)
 	{
 		typedef typename Traits<T>::compute CT;
 		constexpr int t = M + R - 1;
-		const int CV = (C + V - 1) / V;
-		const size_t tiles = static_cast<size_t>(N) * Th * Tw;
-		const size_t gid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-		const int cv = static_cast<int>(gid % CV);
-		const size_t tile = gid / CV;
+		constexpr bool FULL = V > 1;
+		const IDX CV = static_cast<IDX>((C + V - 1) / V);
+		const IDX tiles = static_cast<IDX>(N) * Th * Tw;
+		const IDX gid = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x;
+		const IDX tile = gid / CV;
+		const int cv = static_cast<int>(gid - tile * CV);
 		if (tile >= tiles)
 			return;
-		const int tw = static_cast<int>(tile % Tw);
-		const int th = static_cast<int>((tile / Tw) % Th);
-		const size_t n = tile / (static_cast<size_t>(Tw) * Th);
+		const IDX row = tile / static_cast<IDX>(Tw);
+		const int tw = static_cast<int>(tile - row * Tw);
+		const IDX n = row / static_cast<IDX>(Th);
+		const int th = static_cast<int>(row - n * Th);
 		const int c = cv * V;
-		const int valid = C - c;
+		const int valid = FULL ? V : C - c;
+		const int ih0 = pad_h + th * M, iw0 = pad_w + tw * M;
+		const T *image = x + static_cast<size_t>(n) * H * W * C + c;
+		typedef typename std::conditional<sizeof(IDX) == 4, int, int64_t>::type OFF; /* offsets inside one image */
 
 		CT d[t * t][V];
 #pragma unroll
@@ -174,10 +185,18 @@ namespace
 #pragma unroll
 			for (int b = 0; b < t; b++)
 			{
-				const int ih = pad_h + th * M + a;
-				const int iw = pad_w + tw * M + b;
-				if (ih >= 0 && ih < H && iw >= 0 && iw < W)
-					load_vec<T, V, CT>(x + ((n * H + ih) * W + iw) * C + c, valid, d[a * t + b]);
+				const int ih = ih0 + a;
+				const int iw = iw0 + b;
+				const bool inside = ih >= 0 && ih < H && iw >= 0 && iw < W;
+				if (FULL)
+				{
+					load_vec<T, V, CT>(image + (inside ? (static_cast<OFF>(ih) * W + iw) * C : 0), V, d[a * t + b]);
+#pragma unroll
+					for (int v = 0; v < V; v++)
+						d[a * t + b][v] = inside ? d[a * t + b][v] : padv;
+				}
+				else if (inside)
+					load_vec<T, V, CT>(image + (static_cast<size_t>(ih) * W + iw) * C, valid, d[a * t + b]);
 				else
 				{
 #pragma unroll
@@ -198,25 +217,27 @@ namespace
 		}
 	}
 
-	template<int M, int R, typename T, typename TM, int V>
+	template<int M, int R, typename T, typename TM, int V, int ACT, typename IDX>
 	__global__ __launch_bounds__(256) void k_output_transform(const TM *__restrict__ Mx, T *y, const typename Traits<T>::compute *__restrict__ bias,
 			const T *z, int N, int H, int W, int K, int Th, int Tw, typename Traits<T>::compute alpha1, typename Traits<T>::compute alpha2,
 			typename Traits<T>::compute beta, int activation)
 	{
 		typedef typename Traits<T>::compute CT;
 		constexpr int t = M + R - 1;
-		const int KV = (K + V - 1) / V;
-		const size_t tiles = static_cast<size_t>(N) * Th * Tw;
-		const size_t gid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-		const int kv = static_cast<int>(gid % KV);
-		const size_t tile = gid / KV;
+		constexpr bool FULL = V > 1;
+		const IDX KV = static_cast<IDX>((K + V - 1) / V);
+		const IDX tiles = static_cast<IDX>(N) * Th * Tw;
+		const IDX gid = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x;
+		const IDX tile = gid / KV;
+		const int kv = static_cast<int>(gid - tile * KV);
 		if (tile >= tiles)
 			return;
-		const int tw = static_cast<int>(tile % Tw);
-		const int th = static_cast<int>((tile / Tw) % Th);
-		const size_t n = tile / (static_cast<size_t>(Tw) * Th);
+		const IDX row = tile / static_cast<IDX>(Tw);
+		const int tw = static_cast<int>(tile - row * Tw);
+		const IDX n = row / static_cast<IDX>(Th);
+		const int th = static_cast<int>(row - n * Th);
 		const int k = kv * V;
-		const int valid = K - k;
+		const int valid = FULL ? V : K - k;
 
 		CT d[t * t][V];
 #pragma unroll
@@ -228,14 +249,14 @@ namespace
 			for (int v = 0; v < V; v++)
 				d[i][v] = static_cast<CT>(tmp[v]);
 		}
-		CT out[M * M][V];
-		sandwich<M, R, 2, M, t, CT, V>(d, out);
-
 		CT bv[V];
 #pragma unroll
 		for (int v = 0; v < V; v++)
 			bv[v] = (bias != nullptr && v < valid) ? bias[k + v] : static_cast<CT>(0);
+		CT out[M * M][V];
+		sandwich<M, R, 2, M, t, CT, V>(d, out);
 
+		const size_t image = static_cast<size_t>(n) * H * W;
 #pragma unroll
 		for (int a = 0; a < M; a++)
 #pragma unroll
@@ -245,7 +266,7 @@ namespace
 				const int ow = tw * M + b;
 				if (oh < H && ow < W)
 				{
-					const size_t idx = ((n * H + oh) * W + ow) * K + k;
+					const size_t idx = (image + static_cast<size_t>(oh * W + ow)) * K + k;
 					CT r[V];
 #pragma unroll
 					for (int v = 0; v < V; v++)
@@ -260,7 +281,7 @@ namespace
 					}
 #pragma unroll
 					for (int v = 0; v < V; v++)
-						r[v] = activation_forward<CT>(activation, r[v]);
+						r[v] = activate<ACT, CT>(activation, r[v]);
 					if (beta != static_cast<CT>(0))
 					{
 						CT yv[V];
@@ -274,22 +295,32 @@ namespace
 			}
 	}
 
-	/* Widest vector (in elements) that keeps every access of a [.., C] tensor of `elem` bytes aligned. */
-	template<typename T, typename TM>
+	/* Channels per work-item: as many as 16 bytes of the wider of the two types hold, but never so many that the t x t tile
+	 * (t*t values per channel, twice during the products) pushes the kernel to one or two wavefronts per SIMD: these kernels
+	 * live on many loads and stores in flight from many wavefronts. */
+#ifndef AVHIP_WINOGRAD_WIDTH_T6
+#  define AVHIP_WINOGRAD_WIDTH_T6 2
+#endif
+#ifndef AVHIP_WINOGRAD_WIDTH_T4
+#  define AVHIP_WINOGRAD_WIDTH_T4 4
+#endif
+	template<int M, int R, typename T, typename TM> struct VecOf
+	{
+		static constexpr int wider = sizeof(T) > sizeof(TM) ? sizeof(T) : sizeof(TM);
+		static constexpr int wide = 4 * sizeof(float) / wider;
+		static constexpr int cap = (M + R - 1 >= 6) ? AVHIP_WINOGRAD_WIDTH_T6 : AVHIP_WINOGRAD_WIDTH_T4;
+		static constexpr int value = wide > cap ? cap : wide;
+	};
+	/* The width to launch with: VecOf's when every access of a [.., C] tensor stays aligned to it, else 1. */
+	template<int M, int R, typename T, typename TM>
 	int pick_vec(int C, const void *p0, const void *p1, const void *p2 = nullptr)
 	{
-		constexpr int V = 4 * sizeof(float) / ((sizeof(T) > sizeof(TM) ? sizeof(T) : sizeof(TM))); // 16 B of the wider type
-		constexpr int VV = V > 4 ? 4 : V; // at most 4 channels per work-item keeps the t*t tile in registers
-		const size_t need = VV * (sizeof(T) > sizeof(TM) ? sizeof(T) : sizeof(TM));
+		constexpr int VV = VecOf<M, R, T, TM>::value;
+		const size_t need = VV * VecOf<M, R, T, TM>::wider;
 		if (VV > 1 && C % VV == 0 && aligned_to(p0, need) && aligned_to(p1, need) && (p2 == nullptr || aligned_to(p2, need)))
 			return VV;
 		return 1;
 	}
-	template<typename T, typename TM> struct VecOf
-	{
-		static constexpr int wide = 4 * sizeof(float) / ((sizeof(T) > sizeof(TM) ? sizeof(T) : sizeof(TM)));
-		static constexpr int value = wide > 4 ? 4 : wide;
-	};
 
 	template<typename T> typename Traits<T>::compute host_scalar(const void *p)
 	{
@@ -301,11 +332,11 @@ namespace
 	template<int M, int R, typename T, typename TM>
 	int launch_weight(hipStream_t s, const void *w, void *U, int K, int C, int invert)
 	{
-		const int V = pick_vec<T, TM>(C, w, U);
+		const int V = pick_vec<M, R, T, TM>(C, w, U);
 		const size_t items = static_cast<size_t>(K) * ((C + V - 1) / V);
 		const dim3 grid(ceil_div(items, 256));
 		if (V > 1)
-			hipLaunchKernelGGL((k_weight_transform<M, R, T, TM, VecOf<T, TM>::value>), grid, dim3(256), 0, s, static_cast<const T*>(w), static_cast<TM*>(U), K, C,
+			hipLaunchKernelGGL((k_weight_transform<M, R, T, TM, VecOf<M, R, T, TM>::value>), grid, dim3(256), 0, s, static_cast<const T*>(w), static_cast<TM*>(U), K, C,
 					invert);
 		else
 			hipLaunchKernelGGL((k_weight_transform<M, R, T, TM, 1>), grid, dim3(256), 0, s, static_cast<const T*>(w), static_cast<TM*>(U), K, C, invert);
@@ -315,16 +346,22 @@ namespace
 	int launch_input(hipStream_t s, const void *x, void *Vm, int N, int H, int W, int C, int pad_h, int pad_w, const void *padding_value)
 	{
 		const int Th = (H + M - 1) / M, Tw = (W + M - 1) / M;
-		const int V = pick_vec<T, TM>(C, x, Vm);
+		const int V = pick_vec<M, R, T, TM>(C, x, Vm);
 		const size_t items = static_cast<size_t>(N) * Th * Tw * ((C + V - 1) / V);
 		const dim3 grid(ceil_div(items, 256));
 		const typename Traits<T>::compute padv = host_scalar<T>(padding_value);
-		if (V > 1)
-			hipLaunchKernelGGL((k_input_transform<M, R, T, TM, VecOf<T, TM>::value>), grid, dim3(256), 0, s, static_cast<const T*>(x), static_cast<TM*>(Vm), N, H, W,
-					C, Th, Tw, pad_h, pad_w, padv);
+		const bool narrow = items < (1ull << 31) && static_cast<uint64_t>(H) * W * C < (1ull << 31);
+#define AVHIP_LAUNCH_INPUT(WIDTH, IDX) hipLaunchKernelGGL((k_input_transform<M, R, T, TM, WIDTH, IDX>), grid, dim3(256), 0, s, static_cast<const T*>(x), \
+		static_cast<TM*>(Vm), N, H, W, C, Th, Tw, pad_h, pad_w, padv)
+		if (V > 1 && narrow)
+			AVHIP_LAUNCH_INPUT((VecOf<M, R, T, TM>::value), uint32_t);
+		else if (V > 1)
+			AVHIP_LAUNCH_INPUT((VecOf<M, R, T, TM>::value), size_t);
+		else if (narrow)
+			AVHIP_LAUNCH_INPUT(1, uint32_t);
 		else
-			hipLaunchKernelGGL((k_input_transform<M, R, T, TM, 1>), grid, dim3(256), 0, s, static_cast<const T*>(x), static_cast<TM*>(Vm), N, H, W, C, Th, Tw,
-					pad_h, pad_w, padv);
+			AVHIP_LAUNCH_INPUT(1, size_t);
+#undef AVHIP_LAUNCH_INPUT
 		return 0;
 	}
 	template<int M, int R, typename T, typename TM>
@@ -333,17 +370,26 @@ namespace
 	{
 		typedef typename Traits<T>::compute CT;
 		const int Th = (H + M - 1) / M, Tw = (W + M - 1) / M;
-		int V = pick_vec<T, TM>(K, Mx, y, z);
+		int V = pick_vec<M, R, T, TM>(K, Mx, y, z);
 		const size_t items = static_cast<size_t>(N) * Th * Tw * ((K + V - 1) / V);
 		const dim3 grid(ceil_div(items, 256));
-		if (V > 1)
-			hipLaunchKernelGGL((k_output_transform<M, R, T, TM, VecOf<T, TM>::value>), grid, dim3(256), 0, s, static_cast<const TM*>(Mx), static_cast<T*>(y),
-					static_cast<const CT*>(bias), static_cast<const T*>(z), N, H, W, K, Th, Tw, static_cast<CT>(alpha1), static_cast<CT>(alpha2),
-					static_cast<CT>(beta), activation);
+#define AVHIP_LAUNCH_OUTPUT(WIDTH, ACT, IDX) hipLaunchKernelGGL((k_output_transform<M, R, T, TM, WIDTH, ACT, IDX>), grid, dim3(256), 0, s, \
+		static_cast<const TM*>(Mx), static_cast<T*>(y), static_cast<const CT*>(bias), static_cast<const T*>(z), N, H, W, K, Th, Tw, static_cast<CT>(alpha1), \
+		static_cast<CT>(alpha2), static_cast<CT>(beta), activation)
+		/* LINEAR / RELU get their own instance: a nine-way switch per element makes the compiler evaluate every function */
+		const bool simple = is_simple_activation(activation);
+		const bool narrow = items < (1ull << 31) && static_cast<uint64_t>(H) * W < (1ull << 31);
+		if (V > 1 && simple && narrow)
+			AVHIP_LAUNCH_OUTPUT((VecOf<M, R, T, TM>::value), ACT_SIMPLE, uint32_t);
+		else if (V > 1 && narrow)
+			AVHIP_LAUNCH_OUTPUT((VecOf<M, R, T, TM>::value), ACT_ANY, uint32_t);
+		else if (V > 1)
+			AVHIP_LAUNCH_OUTPUT((VecOf<M, R, T, TM>::value), ACT_ANY, size_t);
+		else if (narrow)
+			AVHIP_LAUNCH_OUTPUT(1, ACT_ANY, uint32_t);
 		else
-			hipLaunchKernelGGL((k_output_transform<M, R, T, TM, 1>), grid, dim3(256), 0, s, static_cast<const TM*>(Mx), static_cast<T*>(y),
-					static_cast<const CT*>(bias), static_cast<const T*>(z), N, H, W, K, Th, Tw, static_cast<CT>(alpha1), static_cast<CT>(alpha2),
-					static_cast<CT>(beta), activation);
+			AVHIP_LAUNCH_OUTPUT(1, ACT_ANY, size_t);
+#undef AVHIP_LAUNCH_OUTPUT
 		return 0;
 	}
 
