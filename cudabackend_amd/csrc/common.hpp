@@ -119,16 +119,26 @@ namespace avhip
 				out[i] = (i < valid) ? static_cast<CT>(Traits<T>::load(ptr[i])) : static_cast<CT>(0);
 		}
 	}
-	template<typename T, int V, typename CT>
+	/* STREAM: the pack is written with a non-temporal store.  For tensors that the writing kernel never reads back this
+	 * lets the caches drain them while the kernel still runs instead of at its end. */
+	template<typename T, int V, typename CT, bool STREAM = false>
 	__device__ inline void store_vec(T *ptr, int valid, const CT (&in)[V], bool allow_vector = true)
 	{
 		if (V > 1 && valid >= V && allow_vector)
 		{
-			Pack<T, V> p;
+			typedef unsigned int words_t __attribute__((ext_vector_type((sizeof(T) * V + 3) / 4)));
+			union
+			{
+				Pack<T, V> p;
+				words_t words;
+			} u;
 #pragma unroll
 			for (int i = 0; i < V; i++)
-				p.v[i] = Traits<T>::store(in[i]);
-			*reinterpret_cast<Pack<T, V>*>(ptr) = p;
+				u.p.v[i] = Traits<T>::store(in[i]);
+			if (STREAM && sizeof(T) * V >= 4)
+				__builtin_nontemporal_store(u.words, reinterpret_cast<words_t*>(ptr));
+			else
+				*reinterpret_cast<Pack<T, V>*>(ptr) = u.p;
 		}
 		else
 		{

@@ -102,7 +102,7 @@ namespace avhip
 				for (int q = 0; q < 4; q++)
 					t[q] += beta * yv[q];
 			}
-			store_vec<TE, 4, float>(y + idx, valid, t, vec);
+			store_vec<TE, 4, float, VEC>(y + idx, valid, t, vec);
 		}
 	};
 
@@ -177,7 +177,12 @@ namespace avhip
 				{
 					int *dst = static_cast<int*>(y) + idx;
 					if (vec && valid >= 4)
-						*reinterpret_cast<int4*>(dst) = make_int4(t[0], t[1], t[2], t[3]);
+					{
+						/* streaming store: the kernel never reads y back, so the caches may drain it while the kernel runs */
+						typedef int i32x4 __attribute__((ext_vector_type(4)));
+						const i32x4 pack = { t[0], t[1], t[2], t[3] };
+						__builtin_nontemporal_store(pack, reinterpret_cast<i32x4*>(dst));
+					}
 					else
 					{
 #pragma unroll
@@ -194,7 +199,11 @@ namespace avhip
 						o[q] = static_cast<int8_t>(round_saturate(static_cast<float>(t[q]) * c.scale[q], -128.0f, 127.0f));
 					int8_t *dst = static_cast<int8_t*>(y) + idx;
 					if (vec && valid >= 4)
-						*reinterpret_cast<char4*>(dst) = make_char4(o[0], o[1], o[2], o[3]);
+					{
+						const unsigned int pack = (static_cast<unsigned int>(static_cast<unsigned char>(o[0]))) | (static_cast<unsigned int>(static_cast<unsigned char>(o[1])) << 8)
+								| (static_cast<unsigned int>(static_cast<unsigned char>(o[2])) << 16) | (static_cast<unsigned int>(static_cast<unsigned char>(o[3])) << 24);
+						__builtin_nontemporal_store(pack, reinterpret_cast<unsigned int*>(dst));
+					}
 					else
 					{
 #pragma unroll

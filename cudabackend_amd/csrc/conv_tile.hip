@@ -11,7 +11,7 @@
  *     straight from the halo at a per-tap uniform offset: the input is read from L2 about once per slice, not R*S times;
  *   - only the weights stream: 64 filters x 128 bytes per step, fetched two steps ahead into registers and double buffered
  *     in LDS exactly as in the general engine;
- *   - the halo of the next channel slice is fetched during the last tap of the current one.
+ *   - the halo of the next channel slice is fetched during the third tap of the current one and held in registers.
  * Four wavefronts stack in M (64 pixels x 64 filters each, 2 x 2 MFMA tiles of 32 x 32); 60 KB of LDS and <= 256 registers
  * let two workgroups share a CU.  k order is (channel slice, tap), which sums the same products as (tap, channel).
  */
@@ -114,6 +114,7 @@ namespace
 
 		const int taps = g.R * g.S;
 		const int total = g.slices * taps;
+		const int prefetch_tap = taps > 2 ? 2 : taps - 1;
 		typename Mma<TE>::acc_t acc[2][2];
 #pragma unroll
 		for (int i = 0; i < 2; i++)
@@ -205,9 +206,11 @@ namespace
 		{
 			__syncthreads(); /* filters of step s and the current halo are visible; everyone is done with step s - 1 */
 			fetch_filters(mine); /* step s + 2 */
-			const bool last_tap = (c_i == g.R - 1) & (c_j == g.S - 1);
+			/* the halo of the next channel slice is requested early in the current one (its registers are free from the
+			 * moment the current halo went to LDS), so that its latency is spent under several taps of MFMAs */
+			const bool prefetch_now = c_i * g.S + c_j == prefetch_tap;
 			const bool more_slices = c_slice + 1 < g.slices;
-			if (last_tap & more_slices)
+			if (prefetch_now & more_slices)
 				fetch_halo(c_slice + 1, hr);
 			if (s < total)
 				multiply(buffer);
