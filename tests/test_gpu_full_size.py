@@ -1,0 +1,133 @@
+"""Parity at BASELINE's full sizes.  The CPU oracle cannot redo these in seconds, so every case combines
+  (a) the oracle on a handful of whole images picked from the batch (images are independent in a forward convolution, so this
+      is an exact check of those images at the real launch geometry: full grids, every tile position, 32-bit offset ranges), with
+  (b) size-independent properties over the WHOLE output: invariance under a permutation of the batch (bit-exact), linearity in
+      the weights and delta kernels (int8, bit-exact), agreement of independent kernels (Winograd vs implicit GEMM)."""
+import numpy as np
+import pytest
+
+import cudabackend_amd as cb
+import helpers as h
+
+pytestmark = pytest.mark.gpu
+
+BAR = {"f32": 1e-5, "f16": 2e-3, "bf16": 2e-3}
+
+
+def he(g, shape):
+    K, R, S, Cin = shape
+    return g.standard_normal(shape) * np.sqrt(2.0 / (R * S * Cin))
+
+
+def check_images(oracle, got, x, w, b, z, images, bar, **kw):
+    for n in images:
+        want = oracle.conv2d(x[n:n + 1], w, b, None if z is None else z[n:n + 1], activation=oracle.RELU, **kw)
+        err = oracle.rel_l2(got[n:n + 1], want)
+        assert err < bar, "image %d: rel-L2 %.3e" % (n, err)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_config2_body_convolution(oracle, dtype):
+    """N=256, 15x15, 128->128, bias + residual + ReLU, through the dispatcher (what the tower calls)."""
+    g = h.rng(40)
+    N = 256
+    x = h.rounded(oracle, g.standard_normal((N, 15, 15, 128)), dtype)
+    w = h.rounded(oracle, he(g, (128, 3, 3, 128)), dtype)
+    b = g.uniform(-0.1, 0.1, 128).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal((N, 15, 15, 128)), dtype)
+    got = h.conv_forward("dispatch", x, w, x.shape, dtype, bias=b, z=z, activation=cb.ACTIVATION_RELU)
+    bar = 1e-4 if dtype == "f32" else BAR[dtype]  # the dispatcher runs fp32 through the fused Winograd kernel
+    check_images(oracle, got, x, w, b, z, (0, 1, 100, 255), bar)
+    perm = g.permutation(N)
+    again = h.conv_forward("dispatch", x[perm], w, x.shape, dtype, bias=b, z=z[perm], activation=cb.ACTIVATION_RELU)
+    np.testing.assert_array_equal(again, got[perm])
+    if dtype == "f32":
+        direct = h.conv_forward("implicit_gemm", x, w, x.shape, dtype, bias=b, z=z, activation=cb.ACTIVATION_RELU)
+        check_images(oracle, direct, x, w, b, z, (0, 255), BAR["f32"])
+        assert oracle.rel_l2(got, direct) < 1e-4
+
+
+def test_config2_stem_and_nonfused_winograd(oracle):
+    """Stem 4->128 on sparse 0/1 planes (bf16), and the four-call non-fused F(4x4,3x3) sequence on the fp32 body shape."""
+    g = h.rng(41)
+    N = 256
+    x0 = (g.random((N, 15, 15, 4)) < 0.15).astype(np.float64)
+    w0 = h.rounded(oracle, he(g, (128, 3, 3, 4)), "bf16")
+    b = g.uniform(-0.1, 0.1, 128).astype(np.float32).astype(np.float64)
+    got = h.conv_forward("dispatch", x0, w0, (N, 15, 15, 128), "bf16", bias=b, activation=cb.ACTIVATION_RELU)
+    check_images(oracle, got, x0, w0, b, None, (0, 17, 255), BAR["bf16"])
+
+    x = h.rounded(oracle, g.standard_normal((N, 15, 15, 128)), "f32")
+    w = h.rounded(oracle, he(g, (128, 3, 3, 128)), "f32")
+    U = h.winograd_weight_transform(w, "f32", 4)
+    V = h.winograd_input_transform(x, w.shape, "f32", 4, (-1, -1))
+    M = h.gemm(V, U, np.zeros((36, V.shape[1], 128)), "f32", opB=True, batched=True)
+    y = h.winograd_output_transform(M, x.shape, w.shape, "f32", 4, bias=b, activation=cb.ACTIVATION_RELU)
+    check_images(oracle, y, x, w, b, None, (0, 128, 255), 1e-4)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_config3_large_spatial(oracle, dtype):
+    """N=64, 56x56, 256->256: implicit GEMM and fused Winograd against the oracle on sampled images, and against each other."""
+    g = h.rng(42)
+    N = 64
+    x = h.rounded(oracle, g.standard_normal((N, 56, 56, 256)), dtype)
+    w = h.rounded(oracle, he(g, (256, 3, 3, 256)), dtype)
+    b = g.uniform(-0.1, 0.1, 256).astype(np.float32).astype(np.float64)
+    direct = h.conv_forward("implicit_gemm", x, w, x.shape, dtype, bias=b, activation=cb.ACTIVATION_RELU)
+    check_images(oracle, direct, x, w, b, None, (0, 63), BAR[dtype])
+    fused = h.conv_forward("winograd_fused", x, w, x.shape, dtype, bias=b, activation=cb.ACTIVATION_RELU)
+    check_images(oracle, fused, x, w, b, None, (31,), BAR[dtype])
+    assert oracle.rel_l2(fused, direct) < 2 * BAR[dtype]
+
+
+def test_config4_int8(oracle):
+    """N=128, 20x20, 128->128 int8: sampled images exact, requantised exact, linearity in the weights and delta kernels exact."""
+    g = h.rng(43)
+    N = 128
+    x = g.integers(-127, 128, (N, 20, 20, 128), dtype=np.int8)
+    b = g.integers(-2 ** 15, 2 ** 15, 128).astype(np.int32)
+    scale = g.uniform(1e-4, 1e-3, 128).astype(np.float32)
+    for R, pad in ((3, (-1, -1)), (1, (0, 0))):
+        w = g.integers(-127, 128, (128, R, R, 128), dtype=np.int8)
+        got = h.conv_forward("implicit_gemm", x, w, (N, 20, 20, 128), "i8", y_dtype="i32", bias=b, bias_dtype="i32", pad=pad)
+        for n in (0, 64, 127):
+            np.testing.assert_array_equal(got[n:n + 1], oracle.conv2d_i8(x[n:n + 1], w, b, pad=pad))
+        q = h.conv_forward("requant", x, w, (N, 20, 20, 128), "i8", y_dtype="i8", bias=b, bias_dtype="i32", scale=scale, pad=pad)
+        np.testing.assert_array_equal(q, oracle.requant_i8(got, scale))
+        # linearity: conv(x, w1) + conv(x, w2) == conv(x, w1 + w2) in exact integer arithmetic (no bias)
+        w1 = g.integers(-60, 61, w.shape, dtype=np.int8)
+        w2 = g.integers(-60, 61, w.shape, dtype=np.int8)
+        y1 = h.conv_forward("implicit_gemm", x, w1, (N, 20, 20, 128), "i8", y_dtype="i32", pad=pad)
+        y2 = h.conv_forward("implicit_gemm", x, w2, (N, 20, 20, 128), "i8", y_dtype="i32", pad=pad)
+        y12 = h.conv_forward("implicit_gemm", x, (w1 + w2).astype(np.int8), (N, 20, 20, 128), "i8", y_dtype="i32", pad=pad)
+        np.testing.assert_array_equal(y1 + y2, y12)
+    # delta kernel at tap (0, 0) of a 3x3 filter with offset -1: y[n, oh, ow, k] = 3 * x[n, oh - 1, ow - 1, k]
+    wd = np.zeros((128, 3, 3, 128), dtype=np.int8)
+    wd[np.arange(128), 0, 0, np.arange(128)] = 3
+    yd = h.conv_forward("implicit_gemm", x, wd, (N, 20, 20, 128), "i8", y_dtype="i32")
+    want = np.zeros((N, 20, 20, 128), dtype=np.int32)
+    want[:, 1:, 1:, :] = 3 * x[:, :-1, :-1, :].astype(np.int32)
+    np.testing.assert_array_equal(yd, want)
+
+
+CONFIG5 = [
+    dict(x=(64, 56, 56, 128), w=(256, 3, 3, 128), pad=(-1, -1), stride=(2, 2)),
+    dict(x=(64, 28, 28, 256), w=(512, 1, 1, 256), pad=(0, 0), stride=(1, 1)),
+    dict(x=(64, 32, 32, 64), w=(64, 5, 5, 64), pad=(-2, -2), stride=(1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", CONFIG5, ids=["3x3s2", "1x1", "5x5"])
+def test_config5_bf16(oracle, case):
+    g = h.rng(44)
+    x = h.rounded(oracle, g.standard_normal(case["x"]), "bf16")
+    w = h.rounded(oracle, he(g, case["w"]), "bf16")
+    K = case["w"][0]
+    b = g.uniform(-0.1, 0.1, K).astype(np.float32).astype(np.float64)
+    Ho, Wo = oracle.conv_output_shape(case["x"][1], case["x"][2], case["w"][1], case["w"][2], case["pad"], case["stride"])
+    got = h.conv_forward("dispatch", x, w, (case["x"][0], Ho, Wo, K), "bf16", bias=b, activation=cb.ACTIVATION_RELU, pad=case["pad"], stride=case["stride"])
+    check_images(oracle, got, x, w, b, None, (0, 63), BAR["bf16"], pad=case["pad"], stride=case["stride"])
+    perm = g.permutation(case["x"][0])
+    again = h.conv_forward("dispatch", x[perm], w, got.shape, "bf16", bias=b, activation=cb.ACTIVATION_RELU, pad=case["pad"], stride=case["stride"])
+    np.testing.assert_array_equal(again, got[perm])
