@@ -273,6 +273,60 @@ def copy_bandwidth(hip, ctx, iters=10):
     return 2.0 * nbytes / (ms * 1e-3) / 1e9
 
 
+def mfma_rates(hip, ctx):
+    """What the matrix cores sustain with register-resident operands and no memory traffic (avhip_mfma_rate_probe), per
+    dtype, in T(FL)OP/s: the clock under sustained MFMA load is below the boost clock the datasheet peak assumes."""
+    lib = cb.load_library()
+    lib.avhip_mfma_rate_probe.restype = C.c_int
+    lib.avhip_mfma_rate_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    workgroups, iterations = 256 * 8, 4096
+    sink = cb.DeviceTensor((workgroups * 256,), cb.DTYPE_FLOAT32)
+    out = {}
+    for name, k, per_call in (("bf16", 16, 1), ("f16", 16, 1), ("i8", 32, 1), ("f32", 2, 4)):
+        def call():
+            assert lib.avhip_mfma_rate_probe(ctx.stream(), DT[name], workgroups, iterations, sink.pointer()) == 0
+        ms = time_calls(hip, ctx, call, 4, warmup=1)
+        ops = workgroups * 4.0 * iterations * 8 * per_call * 2 * 32 * 32 * k
+        out[name] = ops / (ms * 1e-3) / 1e12
+    sink.close()
+    return out
+
+
+def other_configs(hip, ctx, iters):
+    """BASELINE configs 1, 3 and 5 through the dispatcher (bias + ReLU fused), one timing each."""
+    lib = cb.load_library()
+    g = np.random.default_rng(SEED + 7)
+    cases = [("cfg1_f32_3x3_15x15_64", "f32", (8, 15, 15, 64), (64, 3, 3, 64), -1, 1),
+             ("cfg3_bf16_3x3_56x56_256", "bf16", (64, 56, 56, 256), (256, 3, 3, 256), -1, 1),
+             ("cfg3_f16_3x3_56x56_256", "f16", (64, 56, 56, 256), (256, 3, 3, 256), -1, 1),
+             ("cfg5_bf16_3x3_stride2_128_256", "bf16", (64, 56, 56, 128), (256, 3, 3, 128), -1, 2),
+             ("cfg5_bf16_1x1_256_512", "bf16", (64, 28, 28, 256), (512, 1, 1, 256), 0, 1),
+             ("cfg5_bf16_5x5_64_64", "bf16", (64, 32, 32, 64), (64, 5, 5, 64), -2, 1)]
+    out = {}
+    for name, dtype, xs, ws, pad, stride in cases:
+        d = DT[dtype]
+        N, H, W, Cin = xs
+        K, R, S, _ = ws
+        Ho = (H - 2 * pad - R) // stride + 1
+        x = cb.DeviceTensor.from_numpy(g.standard_normal(xs).astype(np.float32), d)
+        w = cb.DeviceTensor.from_numpy((g.standard_normal(ws) * np.sqrt(2.0 / (R * S * Cin))).astype(np.float32), d)
+        b = cb.DeviceTensor.from_numpy(g.uniform(-0.1, 0.1, K).astype(np.float32), cb.DTYPE_FLOAT32)
+        y = cb.DeviceTensor((N, Ho, Ho, K), d)
+        conv = cb.ConvolutionDescriptor(padding=(pad, pad), strides=(stride, stride), dtype=d)
+        need = C.c_int64(0)
+        cb.check(lib.cudaGetConvolutionWorkspaceSize(ctx.handle, conv.handle, x.desc, w.desc, b.desc, C.byref(need)), "workspace size")
+        ws_mem = cb.DeviceTensor((max(int(need.value), 256),), cb.DTYPE_UINT8)
+
+        def call():
+            cb.check(lib.cudaConvolutionBiasActivationForward(ctx.handle, conv.handle, None, x.desc, x.mem, w.desc, w.mem, b.desc, b.mem, None, 0, 0, None,
+                                                              y.desc, y.mem, cb.ACTIVATION_RELU, ws_mem.mem), "conv")
+        ms = time_calls(hip, ctx, call, iters)
+        out[name] = {"us": ms * 1e3, "tflops": conv_flops(N, Ho, Ho, K, Cin, R, S) / (ms * 1e-3) / 1e12}
+        for t in (x, w, b, y, ws_mem):
+            t.close()
+    return out
+
+
 def counter_calibration(ctx, launches=3):
     """Launches a plain streaming kernel of known traffic (fp32 -> fp16 conversion of 2^26 elements: 256 MiB read, 128 MiB
     written).  Under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its reading fixes the factor between the counter and bytes."""
@@ -340,6 +394,8 @@ def main():
         detail["nonfused_winograd_f32_F4"] = nonfused_stages(hip, ctx, "f32", "f32", 4, it)
         detail["nonfused_winograd_bf16_F2_fp16mat"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it)
         detail["copy_GBs_measured"] = copy_bandwidth(hip, ctx)
+        detail["mfma_rate_measured"] = mfma_rates(hip, ctx)
+        detail["other_configs"] = other_configs(hip, ctx, it)
         if "tower_bf16" in detail or args.dtype == "bf16":
             bf = head if args.dtype == "bf16" else detail["tower_bf16"]
             detail["int8_over_bf16_throughput"] = detail["int8_config4"]["3x3"]["tops"] / bf["body_conv_tflops"]

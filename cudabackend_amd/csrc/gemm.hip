@@ -228,6 +228,63 @@ namespace
 	}
 }
 
+namespace
+{
+	/* Eight independent accumulators per wavefront: enough MFMAs in flight to cover the pipeline depth without any memory
+	 * access in the loop.  The operands are arbitrary register contents derived from the lane number. */
+	template<typename TE>
+	__global__ __launch_bounds__(256) void k_mfma_rate_probe(int iterations, typename Mma<TE>::scalar_t *sink)
+	{
+		typename Mma<TE>::acc_t acc[8];
+#pragma unroll
+		for (int i = 0; i < 8; i++)
+#pragma unroll
+			for (int v = 0; v < 16; v++)
+				acc[i][v] = 0;
+		Chunk a, b;
+		a.u = make_uint4(threadIdx.x, 0u, 0u, 0u);
+		b.u = make_uint4(0u, threadIdx.x & 1u, 0u, 0u);
+		for (int it = 0; it < iterations; it++)
+		{
+#pragma unroll
+			for (int i = 0; i < 8; i++)
+				Mma<TE>::run(a, b, acc[i]);
+		}
+		typename Mma<TE>::scalar_t total = 0;
+#pragma unroll
+		for (int i = 0; i < 8; i++)
+#pragma unroll
+			for (int v = 0; v < 16; v++)
+				total += acc[i][v];
+		sink[static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x] = total;
+	}
+}
+
+extern "C" int avhip_mfma_rate_probe(void *stream, int dtype, int workgroups, int iterations, void *sink)
+{
+	if (workgroups <= 0 || iterations <= 0 || sink == nullptr)
+		return AVHIP_BAD_PARAM;
+	hipStream_t st = static_cast<hipStream_t>(stream);
+	switch (dtype)
+	{
+		case DT_FLOAT16:
+			hipLaunchKernelGGL((k_mfma_rate_probe<f16_t>), dim3(workgroups), dim3(256), 0, st, iterations, static_cast<float*>(sink));
+			return 0;
+		case DT_BFLOAT16:
+			hipLaunchKernelGGL((k_mfma_rate_probe<bf16_t>), dim3(workgroups), dim3(256), 0, st, iterations, static_cast<float*>(sink));
+			return 0;
+		case DT_INT8:
+			hipLaunchKernelGGL((k_mfma_rate_probe<int8_t>), dim3(workgroups), dim3(256), 0, st, iterations, static_cast<int*>(sink));
+			return 0;
+		case DT_FLOAT32:
+			/* Mma<float>::run issues four 32x32x2 MFMAs per call */
+			hipLaunchKernelGGL((k_mfma_rate_probe<float>), dim3(workgroups), dim3(256), 0, st, iterations, static_cast<float*>(sink));
+			return 0;
+		default:
+			return AVHIP_UNSUPPORTED_DATATYPE;
+	}
+}
+
 extern "C" int avhip_gemm_batched(void *stream, int ab_dtype, int c_dtype, int opA, int opB, const void *A, const void *B, void *C, int batch, int M,
 		int N, int K, int lda, int ldb, int ldc, int64_t strideA, int64_t strideB, int64_t strideC, double alpha, double beta)
 {
