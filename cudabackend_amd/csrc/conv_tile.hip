@@ -28,10 +28,11 @@ namespace
 	constexpr int HALO_MAX = 300; /* halo pixels that fit */
 	constexpr int HALO_BYTES = HALO_MAX * PIXEL_PITCH;
 	constexpr int FILTER_TILE = TILE_N * LDS_ROW;
-	constexpr int TILE_LDS = HALO_BYTES + 2 * FILTER_TILE;
+	constexpr int ROW_TABLE = HALO_BYTES + 2 * FILTER_TILE; /* offset of the table: tile row -> (y << 16 | x) inside the tile, -1 past it */
+	constexpr int TILE_LDS = ROW_TABLE + TILE_M * 4;
 	constexpr int HALO_FETCHES = (HALO_MAX * STEP_CHUNKS + 255) / 256; /* 16-byte chunks of the halo per work-item */
 	constexpr int FILTER_FETCHES = TILE_N * STEP_CHUNKS / 256;
-	static_assert(DrainShape<1>::bytes <= TILE_LDS, "the drain buffer reuses the operand buffers");
+	static_assert(DrainShape<1>::bytes <= ROW_TABLE, "the drain buffer reuses the operand buffers");
 
 	struct TileGeom
 	{
@@ -79,16 +80,34 @@ namespace
 		const __amdgpu_buffer_rsrc_t rw = make_buffer(w, static_cast<unsigned int>(g.K) * g.R * g.S * g.C * SZ);
 
 		/* where this work-item's halo chunks come from (slice 0) and go to */
+		/* Integer division by a run-time divisor costs about thirty instructions: the work-item divides once and then walks. */
+		int *row_table = reinterpret_cast<int*>(lds + ROW_TABLE);
+		{
+			const int py = tid / g.TW, px = tid - py * g.TW;
+			row_table[tid] = tid < g.TH * g.TW ? ((py << 16) | px) : -1;
+		}
 		unsigned int halo_src[HALO_FETCHES];
 		const int halo_pixels = g.HH * g.HW;
-#pragma unroll
-		for (int f = 0; f < HALO_FETCHES; f++)
 		{
-			const int h = tid / STEP_CHUNKS + f * (256 / STEP_CHUNKS);
-			const int hy = h / g.HW, hx = h - hy * g.HW;
-			const int ih = oh0 + g.pad_h + hy, iw = ow0 + g.pad_w + hx;
-			const bool inside = (h < halo_pixels) & (ih >= 0) & (ih < g.H) & (iw >= 0) & (iw < g.W);
-			halo_src[f] = inside ? static_cast<unsigned int>(((n * g.H + ih) * g.W + iw) * g.C + chunk_channel) * SZ : OUT_OF_RANGE;
+			constexpr int STRIDE = 256 / STEP_CHUNKS; /* halo pixels between two fetches of a work-item */
+			const int dy = STRIDE / g.HW, dx = STRIDE - dy * g.HW;
+			int h = tid / STEP_CHUNKS;
+			int hy = h / g.HW, hx = h - hy * g.HW;
+#pragma unroll
+			for (int f = 0; f < HALO_FETCHES; f++)
+			{
+				const int ih = oh0 + g.pad_h + hy, iw = ow0 + g.pad_w + hx;
+				const bool inside = (h < halo_pixels) & (ih >= 0) & (ih < g.H) & (iw >= 0) & (iw < g.W);
+				halo_src[f] = inside ? static_cast<unsigned int>(((n * g.H + ih) * g.W + iw) * g.C + chunk_channel) * SZ : OUT_OF_RANGE;
+				h += STRIDE;
+				hy += dy;
+				hx += dx;
+				if (hx >= g.HW)
+				{
+					hx -= g.HW;
+					hy++;
+				}
+			}
 		}
 		const int halo_dst = (tid / STEP_CHUNKS) * PIXEL_PITCH + part * 16;
 		unsigned int filt_src[FILTER_FETCHES];
@@ -101,15 +120,7 @@ namespace
 		const int filt_dst = (tid / STEP_CHUNKS) * LDS_ROW + part * 16;
 
 		/* MFMA operand addresses: lane l supplies row (l % 32) of a 32-row tile and k-chunk (l / 32) */
-		int a_off[2];
-#pragma unroll
-		for (int tm = 0; tm < 2; tm++)
-		{
-			const int row = wave * 64 + tm * 32 + (lane & 31);
-			const int py = row / g.TW, px = row - py * g.TW;
-			const int pix = row < g.TH * g.TW ? py * g.HW + px : 0; /* rows past the tile read pixel 0 and are never stored */
-			a_off[tm] = pix * PIXEL_PITCH + (lane >> 5) * 16;
-		}
+		int a_off[2]; /* filled from the row table once it is visible */
 		const int b_off = (lane & 31) * LDS_ROW + (lane >> 5) * 16;
 
 		const int taps = g.R * g.S;
@@ -197,6 +208,14 @@ namespace
 		fetch_halo(0, hr);
 		fetch_filters(fr[0]);
 		fetch_filters(fr[1]);
+		__syncthreads(); /* row table complete */
+#pragma unroll
+		for (int tm = 0; tm < 2; tm++)
+		{
+			const int e = row_table[wave * 64 + tm * 32 + (lane & 31)];
+			const int pix = e >= 0 ? (e >> 16) * g.HW + (e & 0xFFFF) : 0; /* rows past the tile read pixel 0 and are never stored */
+			a_off[tm] = pix * PIXEL_PITCH + (lane >> 5) * 16;
+		}
 		stash_halo(hr);
 		stash_filters(0, fr[0]);
 
@@ -238,9 +257,9 @@ namespace
 
 		drain_tile<TE, 2, 1>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[4]) __attribute__((always_inline))
 		{
-			const int py = row / g.TW, px = row - py * g.TW;
-			const int oh = oh0 + py, ow = ow0 + px;
-			if (row < g.TH * g.TW && oh < g.Ho && ow < g.Wo && kcol < g.K)
+			const int e = row_table[row];
+			const int oh = oh0 + (e >> 16), ow = ow0 + (e & 0xFFFF);
+			if (e >= 0 && oh < g.Ho && ow < g.Wo && kcol < g.K)
 				epi.template store<ACT_SIMPLE, true>((static_cast<int64_t>(n) * g.Ho + oh) * g.Wo + ow, kcol, v, columns);
 		});
 	}
