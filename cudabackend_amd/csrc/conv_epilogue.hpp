@@ -76,9 +76,14 @@ namespace avhip
 		template<int ACT, bool VEC = false>
 		__device__ __forceinline__ void store(int64_t p, int k, const float (&v)[4], const Columns &c) const
 		{
+			store_at<ACT, VEC>(p * K + k, k, v, c);
+		}
+		/* idx: element index of (pixel, filter k) in y and z, for callers that keep it cheaper than p * K + k */
+		template<int ACT, bool VEC = false>
+		__device__ __forceinline__ void store_at(int64_t idx, int k, const float (&v)[4], const Columns &c) const
+		{
 			const bool vec = VEC || this->vec;
 			const int valid = VEC ? 4 : K - k;
-			const int64_t idx = p * K + k;
 			float t[4];
 #pragma unroll
 			for (int q = 0; q < 4; q++)
@@ -157,12 +162,16 @@ namespace avhip
 		template<int ACT, bool VEC = false>
 		__device__ __forceinline__ void store(int64_t p, int k, const int (&v)[4], const Columns &c) const
 		{
+			store_at<ACT, VEC>(p * K + k, k, v, c);
+		}
+		template<int ACT, bool VEC = false>
+		__device__ __forceinline__ void store_at(int64_t idx, int k, const int (&v)[4], const Columns &c) const
+		{
 			/* every fp32 operation below rounds exactly once: a * b + c must not become a fused multiply-add.  The pragma
 			 * governs the expressions written in this block, which is why they use plain operators and no intrinsics. */
 #pragma clang fp contract(off)
 			const bool vec = VEC || this->vec;
 			const int valid = VEC ? 4 : K - k;
-			const int64_t idx = p * K + k;
 			if (MODE == I8_EXACT || MODE == I8_REQUANT)
 			{
 				int t[4];

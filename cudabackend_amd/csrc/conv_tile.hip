@@ -9,11 +9,17 @@
  *   - for each 128-byte slice of input channels it loads the (TH+R-1) x (TW+S-1) input halo ONCE into LDS (pixels outside
  *     the image come back as zeros from the buffer load) and then walks the R*S taps, reading the A operand of tap (i, j)
  *     straight from the halo at a per-tap uniform offset: the input is read from L2 about once per slice, not R*S times;
- *   - only the weights stream: 64 filters x 128 bytes per step, fetched two steps ahead into registers and double buffered
- *     in LDS exactly as in the general engine;
+ *   - only the weights stream: 64 filters x 128 bytes per step, fetched three steps ahead into registers (three sets) and
+ *     double buffered in LDS;
  *   - the halo of the next channel slice is fetched during the third tap of the current one and held in registers.
- * Four wavefronts stack in M (64 pixels x 64 filters each, 2 x 2 MFMA tiles of 32 x 32); 60 KB of LDS and <= 256 registers
+ * Four wavefronts stack in M (64 pixels x 64 filters each, 2 x 2 MFMA tiles of 32 x 32); 61 KB of LDS and <= 256 registers
  * let two workgroups share a CU.  k order is (channel slice, tap), which sums the same products as (tap, channel).
+ *
+ * The 256 rows of the workgroup's GEMM tile are NOT the TH x TW output pixels in raster order: row q stands for halo
+ * position q (halo rows are HW = TW + S - 1 pixels long), so S - 1 rows at the end of every tile row compute values that
+ * nobody stores.  In exchange the A operand of tap (i, j) for row q is halo pixel q + i * HW + j: the 32 rows of an MFMA
+ * tile always read 32 CONSECUTIVE halo pixels, whatever the tap, and with the 144-byte pixel pitch that is free of LDS
+ * bank conflicts.  Raster order would break the run at every tile-row end and serialise most reads two-fold.
  */
 #include "conv_tile.hpp"
 #include "mfma_core.hpp"
@@ -83,8 +89,10 @@ namespace
 		/* Integer division by a run-time divisor costs about thirty instructions: the work-item divides once and then walks. */
 		int *row_table = reinterpret_cast<int*>(lds + ROW_TABLE);
 		{
-			const int py = tid / g.TW, px = tid - py * g.TW;
-			row_table[tid] = tid < g.TH * g.TW ? ((py << 16) | px) : -1;
+			/* GEMM row -> offset of its output pixel inside the image, in pixels; -1 for rows that are not stored */
+			const int py = tid / g.HW, px = tid - py * g.HW;
+			const int oh = oh0 + py, ow = ow0 + px;
+			row_table[tid] = (py < g.TH && px < g.TW && oh < g.Ho && ow < g.Wo) ? oh * g.Wo + ow : -1;
 		}
 		unsigned int halo_src[HALO_FETCHES];
 		const int halo_pixels = g.HH * g.HW;
@@ -120,7 +128,7 @@ namespace
 		const int filt_dst = (tid / STEP_CHUNKS) * LDS_ROW + part * 16;
 
 		/* MFMA operand addresses: lane l supplies row (l % 32) of a 32-row tile and k-chunk (l / 32) */
-		int a_off[2]; /* filled from the row table once it is visible */
+		int a_off[2];
 		const int b_off = (lane & 31) * LDS_ROW + (lane >> 5) * 16;
 
 		const int taps = g.R * g.S;
@@ -204,27 +212,25 @@ namespace
 		};
 
 		uint4 hr[HALO_FETCHES];
-		uint4 fr[2][FILTER_FETCHES];
+		uint4 fr[3][FILTER_FETCHES];
 		fetch_halo(0, hr);
 		fetch_filters(fr[0]);
 		fetch_filters(fr[1]);
-		__syncthreads(); /* row table complete */
+		fetch_filters(fr[2]);
 #pragma unroll
 		for (int tm = 0; tm < 2; tm++)
-		{
-			const int e = row_table[wave * 64 + tm * 32 + (lane & 31)];
-			const int pix = e >= 0 ? (e >> 16) * g.HW + (e & 0xFFFF) : 0; /* rows past the tile read pixel 0 and are never stored */
-			a_off[tm] = pix * PIXEL_PITCH + (lane >> 5) * 16;
-		}
+			a_off[tm] = (wave * 64 + tm * 32 + (lane & 31)) * PIXEL_PITCH + (lane >> 5) * 16;
 		stash_halo(hr);
 		stash_filters(0, fr[0]);
 
-		/* One step = one tap of one channel slice.  Steps run in pairs so that the two register sets and the two LDS
-		 * buffers alternate with compile-time indices; fetches past the last step return zeros and are never multiplied. */
-		auto step = [&](int s, int buffer, uint4 (&mine)[FILTER_FETCHES], uint4 (&other)[FILTER_FETCHES]) __attribute__((always_inline))
+		/* One step = one tap of one channel slice.  The filters of step t are requested at step t - 3 into register set t % 3,
+		 * go to LDS buffer t % 2 at the end of step t - 1 and are multiplied at step t: a load from L2 has two full steps of
+		 * MFMAs to arrive.  Six steps per trip keep the set and buffer indices compile-time constants; fetches past the last
+		 * step return zeros and steps past it are not multiplied. */
+		auto step = [&](int s, int buffer, uint4 (&mine)[FILTER_FETCHES], uint4 (&next)[FILTER_FETCHES]) __attribute__((always_inline))
 		{
 			__syncthreads(); /* filters of step s and the current halo are visible; everyone is done with step s - 1 */
-			fetch_filters(mine); /* step s + 2 */
+			fetch_filters(mine); /* step s + 3: this set held step s, which went to LDS during step s - 1 */
 			/* the halo of the next channel slice is requested early in the current one (its registers are free from the
 			 * moment the current halo went to LDS), so that its latency is spent under several taps of MFMAs */
 			const bool prefetch_now = c_i * g.S + c_j == prefetch_tap;
@@ -233,7 +239,7 @@ namespace
 				fetch_halo(c_slice + 1, hr);
 			if (s < total)
 				multiply(buffer);
-			stash_filters(buffer ^ 1, other); /* step s + 1 */
+			stash_filters(buffer ^ 1, next); /* step s + 1 */
 			if (++c_j == g.S)
 			{
 				c_j = 0;
@@ -249,30 +255,41 @@ namespace
 				}
 			}
 		};
-		for (int s = 0; s < total; s += 2)
+		for (int s = 0; s < total; s += 6)
 		{
 			step(s, 0, fr[0], fr[1]);
-			step(s + 1, 1, fr[1], fr[0]);
+			step(s + 1, 1, fr[1], fr[2]);
+			step(s + 2, 0, fr[2], fr[0]);
+			step(s + 3, 1, fr[0], fr[1]);
+			step(s + 4, 0, fr[1], fr[2]);
+			step(s + 5, 1, fr[2], fr[0]);
 		}
 
+		/* element index of (image n, pixel 0, filter kcol); one image of y is below 2^31 elements (checked by the launcher) */
+		const int64_t image_base = static_cast<int64_t>(n) * g.Ho * g.Wo * g.K + kcol;
 		drain_tile<TE, 2, 1>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[4]) __attribute__((always_inline))
 		{
 			const int e = row_table[row];
-			const int oh = oh0 + (e >> 16), ow = ow0 + (e & 0xFFFF);
-			if (e >= 0 && oh < g.Ho && ow < g.Wo && kcol < g.K)
-				epi.template store<ACT_SIMPLE, true>((static_cast<int64_t>(n) * g.Ho + oh) * g.Wo + ow, kcol, v, columns);
+			if (e >= 0 && kcol < g.K)
+				epi.template store_at<ACT_SIMPLE, true>(image_base + e * g.K, kcol, v, columns);
 		});
 	}
 
-	/* Picks the output tile: as few tiles per image as possible with TH * TW <= 256 and the halo within HALO_MAX. */
+	/* Picks the output tile: as few tiles per image as possible such that the tile's rows in halo order fit the 256 GEMM rows,
+	 * the halo fits its LDS area and the reads of the never-stored rows stay inside the kernel's LDS. */
 	bool choose_tile(const avhipConvShape &s, TileGeom &g)
 	{
+		constexpr int LDS_PIXELS = (HALO_BYTES + 2 * FILTER_TILE) / PIXEL_PITCH;
 		int best_tiles = 0, best_halo = 0;
 		for (int tw = 1; tw <= s.Wo && tw <= TILE_M; tw++)
-			for (int th = 1; th <= s.Ho && th * tw <= TILE_M; th++)
+			for (int th = 1; th <= s.Ho; th++)
 			{
-				const int halo = (th + s.R - 1) * (tw + s.S - 1);
-				if (halo > HALO_MAX)
+				const int hw = tw + s.S - 1;
+				const int rows = (th - 1) * hw + tw;
+				const int halo = (th + s.R - 1) * hw;
+				if (rows > TILE_M)
+					break;
+				if (halo > HALO_MAX || TILE_M + (s.R - 1) * hw + s.S > LDS_PIXELS)
 					continue;
 				const int tiles = ((s.Ho + th - 1) / th) * ((s.Wo + tw - 1) / tw);
 				if (best_tiles == 0 || tiles < best_tiles || (tiles == best_tiles && halo < best_halo))
@@ -319,6 +336,8 @@ namespace avhip
 		/* the gather kernel wastes nothing on partially filled tiles: keep it when tiles would be mostly padding */
 		const double fill = static_cast<double>(s.Ho) * s.Wo / (static_cast<double>(g.tiles_h) * g.tiles_w * TILE_M);
 		if (fill < 0.5)
+			return false;
+		if (static_cast<int64_t>(s.Ho) * s.Wo * s.K >= (1ll << 31))
 			return false;
 		const int64_t blocks = static_cast<int64_t>(s.N) * g.tiles_h * g.tiles_w;
 		const int64_t filter_blocks = (static_cast<int64_t>(s.K) + TILE_N - 1) / TILE_N;
