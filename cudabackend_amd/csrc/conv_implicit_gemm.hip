@@ -433,7 +433,7 @@ namespace
 		{
 			const int64_t p = p0 + r;
 			if (p < g.pixels && k < g.K)
-				epi.template store<FAST ? ACT_SIMPLE : ACT_ANY>(p, k, v, columns);
+				epi.template store<FAST ? ACT_SIMPLE : ACT_ANY, FAST>(p, k, v, columns); /* fast instances store whole 4-filter vectors */
 		});
 	}
 
@@ -455,7 +455,7 @@ namespace
 		{
 			const int64_t p = p0 + r;
 			if (p < g.pixels && k < g.K)
-				epi.template store<ACT_SIMPLE>(p, k, v, columns);
+				epi.template store<ACT_SIMPLE, true>(p, k, v, columns);
 		});
 	}
 
@@ -517,10 +517,11 @@ namespace
 		else
 			std::memset(&padv, 0, sizeof(TE));
 		const dim3 grid(ceil_div(g.pixels, BLOCK_M), ceil_div(s.K, BLOCK_N));
-		const bool fast = fast_path_ok<TE>(s, flags, padding_value) && is_simple_activation(epi.activation);
+		/* the branch-free instances also store whole 4-filter vectors (streaming stores): K % 4 == 0 and y, z aligned (bit 1) */
+		const bool fast = fast_path_ok<TE>(s, flags, padding_value) && is_simple_activation(epi.activation) && (flags & 2) != 0;
 		/* few input channels: pack (tap, channel) into the k-steps instead of spending a step per tap */
 		const int pixel_bytes = s.C * static_cast<int>(sizeof(TE));
-		if (pixel_bytes <= STEP_BYTES / 2 && s.R * s.S > 1 && fast_path_ok<TE>(s, 1, padding_value) && is_simple_activation(epi.activation))
+		if (pixel_bytes <= STEP_BYTES / 2 && s.R * s.S > 1 && fast_path_ok<TE>(s, 1, padding_value) && is_simple_activation(epi.activation) && (flags & 2) != 0)
 		{
 			int pb = 16;
 			while (pb > 1 && (pixel_bytes % pb != 0 || !aligned_to(x, pb) || !aligned_to(w, pb)))
