@@ -56,6 +56,26 @@ namespace
 		}
 	};
 
+	/* Bit t = i * S + j of the result: tap (i, j) of the window whose origin is (ih0, iw0) reads a pixel inside the image.
+	 * Rows and columns are tested separately (R + S tests, no division) and combined. */
+	__device__ inline unsigned int inside_mask(const ConvGeom &g, int ih0, int iw0)
+	{
+		unsigned int columns = 0, m = 0;
+		for (int j = 0; j < g.S; j++)
+		{
+			const int iw = iw0 + (g.flip ? g.S - 1 - j : j) * g.dil_w;
+			if (iw >= 0 && iw < g.W)
+				columns |= 1u << j;
+		}
+		for (int i = 0; i < g.R; i++)
+		{
+			const int ih = ih0 + (g.flip ? g.R - 1 - i : i) * g.dil_h;
+			if (ih >= 0 && ih < g.H)
+				m |= columns << (i * g.S);
+		}
+		return m;
+	}
+
 	/* Rows of A are output pixels; a chunk is 16 bytes of channels of the input pixel that tap (i, j) reads.
 	 * General form: any alignment, any channel count, any padding value. */
 	template<typename TE, bool FAST>
@@ -146,20 +166,7 @@ namespace
 				const int ih0 = oh * g.stride_h + g.pad_h;
 				const int iw0 = ow * g.stride_w + g.pad_w;
 				origin[q] = static_cast<unsigned int>((static_cast<int>(n * g.H + ih0) * g.W + iw0) * g.C + chunk_channel) * static_cast<unsigned int>(sizeof(TE));
-				unsigned int m = 0;
-				for (int t = 0; t < g.R * g.S; t++)
-				{
-					int i = t / g.S, j = t - (t / g.S) * g.S;
-					if (g.flip)
-					{
-						i = g.R - 1 - i;
-						j = g.S - 1 - j;
-					}
-					const int ih = ih0 + i * g.dil_h, iw = iw0 + j * g.dil_w;
-					if (ok && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
-						m |= 1u << t;
-				}
-				inside[q] = m;
+				inside[q] = ok ? inside_mask(g, ih0, iw0) : 0u;
 			}
 			set_tap();
 		}
@@ -328,20 +335,7 @@ namespace
 				const int ih0 = oh * g.stride_h + g.pad_h;
 				const int iw0 = ow * g.stride_w + g.pad_w;
 				origin[q] = static_cast<unsigned int>((static_cast<int>(n * g.H + ih0) * g.W + iw0)) * CB;
-				unsigned int m = 0;
-				for (int t = 0; t < g.R * g.S; t++)
-				{
-					int i = t / g.S, j = t - (t / g.S) * g.S;
-					if (g.flip)
-					{
-						i = g.R - 1 - i;
-						j = g.S - 1 - j;
-					}
-					const int ih = ih0 + i * g.dil_h, iw = iw0 + j * g.dil_w;
-					if (ok && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
-						m |= 1u << t;
-				}
-				inside[q] = m;
+				inside[q] = ok ? inside_mask(g, ih0, iw0) : 0u;
 			}
 			k_byte = (threadIdx.x % STEP_CHUNKS) * 16;
 			place();
