@@ -213,7 +213,7 @@ namespace
 #pragma unroll
 			for (int v = 0; v < V; v++)
 				o[v] = static_cast<typename Traits<TM>::compute>(out[i][v]);
-			store_vec<TM, V>(Vm + (static_cast<size_t>(i) * tiles + tile) * C + c, valid, o);
+			store_vec<TM, V, typename Traits<TM>::compute, FULL>(Vm + (static_cast<size_t>(i) * tiles + tile) * C + c, valid, o);
 		}
 	}
 
@@ -290,7 +290,7 @@ namespace
 						for (int v = 0; v < V; v++)
 							r[v] += beta * yv[v];
 					}
-					store_vec<T, V>(y + idx, valid, r);
+					store_vec<T, V, CT, FULL>(y + idx, valid, r);
 				}
 			}
 	}
