@@ -116,3 +116,35 @@ def test_copy_possible_only_within_one_device():
     cb.check(lib.cudaIsCopyPossible(0, 1, C.byref(r)))
     assert not r.value
     assert lib.cudaIsCopyPossible(0, 0, None) == cb.STATUS_BAD_PARAM
+
+
+def test_headers_compile_as_c_and_cxx_and_link(tmp_path):
+    """A front-end written in C or C++ includes <Avocado/cuda_backend.h> and links the shared library: the headers must be
+    valid in both languages and every entry point must resolve at link time (the program only calls what works without a GPU)."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib_dir = os.path.join(root, "cudabackend_amd")
+    if not os.path.exists(os.path.join(lib_dir, "libavocado_hip.so")):
+        pytest.skip("library not built")
+    c_src = tmp_path / "front_end.c"
+    c_src.write_text('#include <stdio.h>\n#include "avocado_hip_backend.h"\n#include "avocado_hip_kernels.h"\n'
+                     'int main(void) {\n'
+                     '  avTensorDescriptor_t t; int dims[4] = {2, 3, 4, 5};\n'
+                     '  if (cudaCreateTensorDescriptor(&t) != AVOCADO_STATUS_SUCCESS) return 1;\n'
+                     '  if (cudaSetTensorDescriptor(t, AVOCADO_DTYPE_FLOAT32, 4, dims) != AVOCADO_STATUS_SUCCESS) return 2;\n'
+                     '  if (cudaDestroyTensorDescriptor(t) != AVOCADO_STATUS_SUCCESS) return 3;\n'
+                     '  printf("devices %d\\n", cudaGetNumberOfDevices());\n'
+                     '  return avhip_conv2d_implicit_gemm(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1.0, 1.0, 0.0, 0, 0) == AVHIP_BAD_PARAM ? 0 : 4;\n}\n')
+    cxx_src = tmp_path / "front_end.cpp"
+    cxx_src.write_text('#include <Avocado/cuda_backend.h>\nusing namespace avocado::backend;\n'
+                       'int main() { avConvolutionDescriptor_t c; if (cudaCreateConvolutionDescriptor(&c) != AVOCADO_STATUS_SUCCESS) return 1;\n'
+                       '  return cudaDestroyConvolutionDescriptor(c) == AVOCADO_STATUS_SUCCESS ? 0 : 2; }\n')
+    env = dict(os.environ, LD_LIBRARY_PATH=lib_dir + ":/opt/rocm/lib:" + os.environ.get("LD_LIBRARY_PATH", ""))
+    for compiler, src, exe in (("gcc", c_src, tmp_path / "c_front"), ("g++", cxx_src, tmp_path / "cxx_front")):
+        cmd = [compiler, "-Wall", "-Werror", "-I", os.path.join(root, "include"), str(src), "-o", str(exe), "-L", lib_dir, "-lavocado_hip",
+               "-Wl,-rpath," + lib_dir, "-Wl,-rpath-link,/opt/rocm/lib"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        assert r.returncode == 0, r.stdout + r.stderr
+        r = subprocess.run([str(exe)], capture_output=True, text=True, env=env)
+        assert r.returncode == 0, "exit %d: %s%s" % (r.returncode, r.stdout, r.stderr)
