@@ -1431,8 +1431,12 @@ namespace avocado
 			/* 3x3 / stride 1 on fp32 tensors with enough channels to fill the matrix cores: fused Winograd, whose 2.25-fold saving
 			 * of multiplications is worth more than its transform work at the fp32 MFMA rate.  At the 16-bit MFMA rate the
 			 * convolution is bound by LDS traffic, not by the matrix cores, and the direct image-tile kernel is faster. */
+			/* its workgroups cover 16 x 16 pixels x 128 filters: a problem with too few of them is left to the implicit-GEMM
+			 * kernels, which can cut it finer */
+			const av_int64 fused_workgroups = static_cast<av_int64>(p.shape.N) * ((p.shape.Ho + 15) / 16) * ((p.shape.Wo + 15) / 16)
+					* ((p.shape.K + 127) / 128);
 			if (fused_winograd_applicable(p) && p.x_dtype == AVOCADO_DTYPE_FLOAT32 && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32
-					&& p.shape.Ho == p.shape.H && p.shape.Wo == p.shape.W)
+					&& p.shape.Ho == p.shape.H && p.shape.Wo == p.shape.W && fused_workgroups >= 128)
 			{
 				const avStatus_t fs = run_fused_winograd(call, wMem, yMem, activation);
 				if (fs != AVOCADO_STATUS_NOT_SUPPORTED)

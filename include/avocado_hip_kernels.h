@@ -99,6 +99,11 @@ extern "C"
 	 * src/descriptors.cu:22-39. */
 	AVHIP_API int avhip_set_memory(void *stream, void *dst, int64_t bytes, const void *pattern, int pattern_size);
 
+	/* Tuning knob without a counterpart in the reference.  The implicit-GEMM launcher sends a convolution to the kernel with
+	 * one 32 x 32 tile per wavefront when its 128 x 128 tiling would yield fewer than this many workgroups (default 192 on
+	 * the 256 compute units of an MI355X; 0 never uses that kernel).  Returns the previous value.  Process-wide. */
+	AVHIP_API int avhip_set_small_problem_threshold(int workgroups);
+
 	/* Measurement aid without a counterpart in the reference: keeps every matrix core busy with register-resident
 	 * 32x32 MFMAs of `dtype` (FLOAT16, BFLOAT16, INT8 or FLOAT32) and nothing else, so that a harness can time the rate the
 	 * matrix cores sustain on this machine (clock under load included) next to the datasheet peak.  Launches `workgroups`
