@@ -194,24 +194,48 @@ def time_calls(hip, ctx, fn, iters, warmup=3):
 
 
 def int8_leg(hip, ctx, iters):
-    """Config 4: int8 x int8 -> int32, N=128, 20x20, 128->128, 3x3 offset -1 and 1x1."""
+    """Config 4: N=128, 20x20, 128->128, 3x3 offset -1 and 1x1: int8 x int8 -> int32 (bit-exact path), int8 -> int8
+    requantised by a per-filter fp32 scale, and the same shapes in bf16 for the throughput ratio on equal work."""
     lib = cb.load_library()
     g = np.random.default_rng(SEED + 4)
     out = {}
-    x = cb.DeviceTensor.from_numpy(g.integers(-127, 128, (128, 20, 20, 128), dtype=np.int8), cb.DTYPE_INT8)
+    shape = (128, 20, 20, 128)
+    x = cb.DeviceTensor.from_numpy(g.integers(-127, 128, shape, dtype=np.int8), cb.DTYPE_INT8)
     b = cb.DeviceTensor.from_numpy(g.integers(-2 ** 15, 2 ** 15, 128).astype(np.int32), cb.DTYPE_INT32)
-    y = cb.DeviceTensor((128, 20, 20, 128), cb.DTYPE_INT32)
+    scale = cb.DeviceTensor.from_numpy(g.uniform(1e-4, 1e-3, 128).astype(np.float32), cb.DTYPE_FLOAT32)
+    y = cb.DeviceTensor(shape, cb.DTYPE_INT32)
+    q = cb.DeviceTensor(shape, cb.DTYPE_INT8)
+    xb = cb.DeviceTensor.from_numpy(g.standard_normal(shape).astype(np.float32), cb.DTYPE_BFLOAT16)
+    bb = cb.DeviceTensor.from_numpy(g.uniform(-0.1, 0.1, 128).astype(np.float32), cb.DTYPE_FLOAT32)
+    yb = cb.DeviceTensor(shape, cb.DTYPE_BFLOAT16)
     for r, pad in ((3, -1), (1, 0)):
         w = cb.DeviceTensor.from_numpy(g.integers(-127, 128, (128, r, r, 128), dtype=np.int8), cb.DTYPE_INT8)
+        wb = cb.DeviceTensor.from_numpy((g.standard_normal((128, r, r, 128)) * np.sqrt(2.0 / (r * r * 128))).astype(np.float32), cb.DTYPE_BFLOAT16)
         conv = cb.ConvolutionDescriptor(padding=(pad, pad), dtype=cb.DTYPE_INT8)
+        convb = cb.ConvolutionDescriptor(padding=(pad, pad), dtype=cb.DTYPE_BFLOAT16)
 
-        def call():
+        def exact():
             cb.check(lib.cudaConvolutionImplicitGemmForward(ctx.handle, conv.handle, None, x.desc, x.mem, w.desc, w.mem, b.desc, b.mem, None, 0, 0, None,
                                                             y.desc, y.mem, cb.ACTIVATION_LINEAR), "int8 conv")
-        ms = time_calls(hip, ctx, call, iters)
-        out["%dx%d" % (r, r)] = {"us": ms * 1e3, "tops": conv_flops(128, 20, 20, 128, 128, r, r) / (ms * 1e-3) / 1e12}
+
+        def requant():
+            cb.check(lib.avhipConvolutionRequantForward(ctx.handle, conv.handle, x.desc, x.mem, w.desc, w.mem, b.desc, b.mem, scale.desc, scale.mem,
+                                                        q.desc, q.mem, cb.ACTIVATION_RELU), "int8 requant conv")
+
+        def bf16():
+            cb.check(lib.cudaConvolutionImplicitGemmForward(ctx.handle, convb.handle, None, xb.desc, xb.mem, wb.desc, wb.mem, bb.desc, bb.mem, None, 0, 0,
+                                                            None, yb.desc, yb.mem, cb.ACTIVATION_RELU), "bf16 conv")
+        ops = conv_flops(128, 20, 20, 128, 128, r, r)
+        rec = {}
+        for name, fn in (("int32_out", exact), ("int8_requant_out", requant), ("bf16_same_shape", bf16)):
+            ms = time_calls(hip, ctx, fn, iters)
+            rec[name] = {"us": ms * 1e3, "tops": ops / (ms * 1e-3) / 1e12}
+        rec["int8_over_bf16"] = {"int32_out": rec["bf16_same_shape"]["us"] / rec["int32_out"]["us"],
+                                 "int8_requant_out": rec["bf16_same_shape"]["us"] / rec["int8_requant_out"]["us"]}
+        out["%dx%d" % (r, r)] = rec
         w.close()
-    for t in (x, b, y):
+        wb.close()
+    for t in (x, b, scale, y, q, xb, bb, yb):
         t.close()
     return out
 
@@ -396,9 +420,6 @@ def main():
         detail["copy_GBs_measured"] = copy_bandwidth(hip, ctx)
         detail["mfma_rate_measured"] = mfma_rates(hip, ctx)
         detail["other_configs"] = other_configs(hip, ctx, it)
-        if "tower_bf16" in detail or args.dtype == "bf16":
-            bf = head if args.dtype == "bf16" else detail["tower_bf16"]
-            detail["int8_over_bf16_throughput"] = detail["int8_config4"]["3x3"]["tops"] / bf["body_conv_tflops"]
         cpu = cpu_baseline()
     ctx.close()
     peak = PEAK[args.dtype]

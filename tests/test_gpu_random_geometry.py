@@ -1,0 +1,99 @@
+"""Seeded random sweep over convolution geometries, data types, epilogue terms and kernel selections, against the CPU oracle.
+The hand-picked cases of the other files pin known edges; this sweep looks for the ones nobody thought of (ragged channel and
+filter counts, windows hanging over any border, non-square filters with asymmetric offsets, strides and dilations that do not
+divide the image).  Bars as everywhere: int8 bit-exact, fp32 1e-5 (1e-4 through Winograd), fp16 / bf16 2e-3."""
+import numpy as np
+import pytest
+
+import cudabackend_amd as cb
+import helpers as h
+
+pytestmark = pytest.mark.gpu
+
+CHANNELS = [1, 2, 3, 4, 5, 8, 12, 16, 20, 32, 36, 64, 72, 136]
+FILTERS = [1, 3, 4, 8, 20, 32, 40, 64, 132]
+
+
+def random_case(g):
+    R, S = int(g.choice([1, 2, 3, 5])), int(g.choice([1, 2, 3, 5]))
+    dil = (int(g.choice([1, 1, 2])), int(g.choice([1, 1, 2])))
+    stride = (int(g.choice([1, 1, 2, 3])), int(g.choice([1, 1, 2, 3])))
+    H, W = int(g.integers(3, 21)), int(g.integers(3, 21))
+    pad = (-int(g.integers(0, (R - 1) * dil[0] + 1)), -int(g.integers(0, (S - 1) * dil[1] + 1)))  # up to the full convolution
+    return dict(x=(int(g.integers(1, 4)), H, W, int(g.choice(CHANNELS))), w=(int(g.choice(FILTERS)), R, S), pad=pad, stride=stride, dilation=dil,
+                mode=int(g.integers(0, 2)))
+
+
+def output_shape(orc, c):
+    N, H, W, _ = c["x"]
+    K, R, S = c["w"]
+    Ho = (H - 2 * c["pad"][0] - ((R - 1) * c["dilation"][0] + 1)) // c["stride"][0] + 1
+    Wo = (W - 2 * c["pad"][1] - ((S - 1) * c["dilation"][1] + 1)) // c["stride"][1] + 1
+    return (N, Ho, Wo, K)
+
+
+@pytest.mark.parametrize("tiling", ["wavefront_tiles", "workgroup_tiles"])
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_random_geometries_floating(oracle, dtype, tiling):
+    lib = cb.load_library()
+    lib.avhip_set_small_problem_threshold.restype = int
+    previous = lib.avhip_set_small_problem_threshold(192 if tiling == "wavefront_tiles" else 0)
+    try:
+        g = h.rng(50 + ["f32", "f16", "bf16"].index(dtype))
+        done = 0
+        while done < 120:
+            c = random_case(g)
+            ys = output_shape(oracle, c)
+            if ys[1] < 1 or ys[2] < 1:
+                continue
+            done += 1
+            x = h.rounded(oracle, g.standard_normal(c["x"]), dtype)
+            ws = (c["w"][0], c["w"][1], c["w"][2], c["x"][3])
+            w = h.rounded(oracle, g.standard_normal(ws) * np.sqrt(2.0 / (ws[1] * ws[2] * ws[3])), dtype)
+            b = g.uniform(-0.1, 0.1, ws[0]).astype(np.float32).astype(np.float64) if g.random() < 0.7 else None
+            z = h.rounded(oracle, g.standard_normal(ys), dtype) if g.random() < 0.5 else None
+            act = int(g.choice([cb.ACTIVATION_LINEAR, cb.ACTIVATION_RELU, cb.ACTIVATION_RELU, cb.ACTIVATION_TANH]))
+            kw = dict(pad=c["pad"], stride=c["stride"], dilation=c["dilation"], mode=c["mode"])
+            want = oracle.conv2d(x, w, b, z, activation=act, **kw)
+            assert want.shape == ys, (c, want.shape, ys)
+            for entry in ("implicit_gemm", "dispatch"):
+                got = h.conv_forward(entry, x, w, ys, dtype, bias=b, z=z, activation=act, **kw)
+                bar = {"f32": 1e-4 if entry == "dispatch" else 1e-5, "f16": 2e-3, "bf16": 2e-3}[dtype]
+                err = oracle.rel_l2(got, want)
+                assert err < bar, "case %d %s %s: rel-L2 %.3e  %r bias=%s z=%s act=%d" % (done, entry, dtype, err, c, b is not None, z is not None, act)
+            if ws[1] == 3 and ws[2] == 3 and c["stride"] == (1, 1) and c["dilation"] == (1, 1) and ws[3] % (4 if dtype == "f32" else 8) == 0:
+                got = h.conv_forward("winograd_fused", x, w, ys, dtype, bias=b, z=z, activation=act, pad=c["pad"], mode=c["mode"])
+                err = oracle.rel_l2(got, want)
+                assert err < (1e-4 if dtype == "f32" else 2e-3), "case %d fused %s: rel-L2 %.3e  %r" % (done, dtype, err, c)
+    finally:
+        lib.avhip_set_small_problem_threshold(previous)
+
+
+@pytest.mark.parametrize("tiling", ["wavefront_tiles", "workgroup_tiles"])
+def test_random_geometries_int8(oracle, tiling):
+    lib = cb.load_library()
+    lib.avhip_set_small_problem_threshold.restype = int
+    previous = lib.avhip_set_small_problem_threshold(192 if tiling == "wavefront_tiles" else 0)
+    try:
+        g = h.rng(53)
+        done = 0
+        while done < 120:
+            c = random_case(g)
+            ys = output_shape(oracle, c)
+            if ys[1] < 1 or ys[2] < 1:
+                continue
+            done += 1
+            ws = (c["w"][0], c["w"][1], c["w"][2], c["x"][3])
+            x = g.integers(-127, 128, c["x"], dtype=np.int8)
+            w = g.integers(-127, 128, ws, dtype=np.int8)
+            b = g.integers(-2 ** 15, 2 ** 15, ws[0]).astype(np.int32)
+            scale = g.uniform(1e-4, 1e-3, ws[0]).astype(np.float32)
+            act = int(g.choice([cb.ACTIVATION_LINEAR, cb.ACTIVATION_RELU]))
+            kw = dict(pad=c["pad"], stride=c["stride"], dilation=c["dilation"], mode=c["mode"])
+            want = oracle.conv2d_i8(x, w, b, activation=act, **kw)
+            got = h.conv_forward("implicit_gemm", x, w, ys, "i8", y_dtype="i32", bias=b, bias_dtype="i32", activation=act, **kw)
+            np.testing.assert_array_equal(got, want, err_msg="case %d %r" % (done, c))
+            q = h.conv_forward("requant", x, w, ys, "i8", y_dtype="i8", bias=b, bias_dtype="i32", scale=scale, activation=act, **kw)
+            np.testing.assert_array_equal(q, oracle.requant_i8(want, scale), err_msg="requant case %d %r" % (done, c))
+    finally:
+        lib.avhip_set_small_problem_threshold(previous)
