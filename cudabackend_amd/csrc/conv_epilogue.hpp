@@ -46,10 +46,13 @@ namespace avhip
 	struct FloatEpilogue
 	{
 		typedef float scalar_t;
-		struct Columns
+		/* widest run of filters one work-item can store with a single 16-byte instruction */
+		static constexpr int wide = sizeof(TE) >= 4 ? 4 : 8;
+		template<int W> struct ColumnsT
 		{
-			float bias[4];
+			float bias[W];
 		};
+		typedef ColumnsT<4> Columns;
 		const float *bias;
 		const TE *z;
 		TE *y;
@@ -66,49 +69,60 @@ namespace avhip
 			keep_in_sgpr(activation);
 			keep_in_sgpr(K);
 		}
-		__device__ __forceinline__ void load_columns(int k, Columns &c) const
+		template<int W>
+		__device__ __forceinline__ void load_columns(int k, ColumnsT<W> &c) const
 		{
 #pragma unroll
-			for (int q = 0; q < 4; q++)
+			for (int q = 0; q < W; q++)
 				c.bias[q] = (bias != nullptr && k + q < K) ? bias[k + q] : 0.0f;
 		}
-		/* p: index of the output pixel (row of y), k: first of the four filters.  VEC instances require `vec`. */
+		/* p: index of the output pixel (row of y), k: first of the W filters.  VEC instances require whole, aligned vectors. */
 		template<int ACT, bool VEC = false>
 		__device__ __forceinline__ void store(int64_t p, int k, const float (&v)[4], const Columns &c) const
 		{
-			store_at<ACT, VEC>(p * K + k, k, v, c);
+			store_at<ACT, VEC, 4>(p * K + k, k, v, c);
 		}
 		/* idx: element index of (pixel, filter k) in y and z, for callers that keep it cheaper than p * K + k */
-		template<int ACT, bool VEC = false>
-		__device__ __forceinline__ void store_at(int64_t idx, int k, const float (&v)[4], const Columns &c) const
+		template<int ACT, bool VEC = false, int W = 4>
+		__device__ __forceinline__ void store_at(int64_t idx, int k, const float (&v)[W], const ColumnsT<W> &c) const
 		{
+			static_assert(VEC || W == 4, "`vec` vouches for 4-element vectors only; wider runs are for callers that checked");
 			const bool vec = VEC || this->vec;
-			const int valid = VEC ? 4 : K - k;
-			float t[4];
+			const int valid = VEC ? W : K - k;
+			float t[W];
 #pragma unroll
-			for (int q = 0; q < 4; q++)
+			for (int q = 0; q < W; q++)
 				t[q] = alpha1 * v[q] + c.bias[q];
 			if (z != nullptr)
 			{
-				float zv[4];
-				load_vec<TE, 4, float>(z + idx, valid, zv, vec);
+				float zv[W];
+				load_vec<TE, W, float>(z + idx, valid, zv, vec);
 #pragma unroll
-				for (int q = 0; q < 4; q++)
+				for (int q = 0; q < W; q++)
 					t[q] += alpha2 * zv[q];
 			}
 #pragma unroll
-			for (int q = 0; q < 4; q++)
+			for (int q = 0; q < W; q++)
 				t[q] = activate<ACT, float>(activation, t[q]);
 			if (beta != 0.0f)
 			{
-				float yv[4];
-				load_vec<TE, 4, float>(y + idx, valid, yv, vec);
+				float yv[W];
+				load_vec<TE, W, float>(y + idx, valid, yv, vec);
 #pragma unroll
-				for (int q = 0; q < 4; q++)
+				for (int q = 0; q < W; q++)
 					t[q] += beta * yv[q];
 			}
-			store_vec<TE, 4, float, VEC>(y + idx, valid, t, vec);
+			store_vec<TE, W, float, VEC>(y + idx, valid, t, vec);
 		}
+	};
+
+	template<int N> struct Words
+	{
+		typedef int type __attribute__((ext_vector_type(N)));
+	};
+	template<> struct Words<1>
+	{
+		typedef int type;
 	};
 
 	enum Int8Mode
@@ -127,12 +141,14 @@ namespace avhip
 	struct Int8Epilogue
 	{
 		typedef int scalar_t;
-		struct Columns
+		static constexpr int wide = MODE == I8_REQUANT ? 8 : 4;
+		template<int W> struct ColumnsT
 		{
-			int ibias[4];
-			float fbias[4];
-			float scale[4];
+			int ibias[W];
+			float fbias[W];
+			float scale[W];
 		};
+		typedef ColumnsT<4> Columns;
 		const void *bias, *z;
 		void *y;
 		const float *scale;
@@ -148,84 +164,99 @@ namespace avhip
 			keep_in_sgpr(activation);
 			keep_in_sgpr(K);
 		}
-		__device__ __forceinline__ void load_columns(int k, Columns &c) const
+		template<int W>
+		__device__ __forceinline__ void load_columns(int k, ColumnsT<W> &c) const
 		{
 #pragma unroll
-			for (int q = 0; q < 4; q++)
+			for (int q = 0; q < W; q++)
 			{
 				const bool in = k + q < K;
 				c.ibias[q] = (MODE <= I8_REQUANT && bias != nullptr && in) ? static_cast<const int*>(bias)[k + q] : 0;
 				c.fbias[q] = (MODE > I8_REQUANT && bias != nullptr && in) ? static_cast<const float*>(bias)[k + q] : 0.0f;
-				c.scale[q] = (MODE == I8_REQUANT && in) ? scale[k + q] : 0.0f;
+				/* Requantisation multiplies a finite fp32 value by the scale and clamps.  A NaN scale gives NaN -> 0 for every
+				 * sum, exactly what a zero scale gives; an infinite scale saturates every non-zero sum and gives NaN -> 0 for
+				 * a zero sum, exactly what the largest finite scale gives.  Replacing them here, once per filter, leaves the
+				 * per-element path free of NaN handling. */
+				float sc = (MODE == I8_REQUANT && in) ? scale[k + q] : 0.0f;
+				sc = (sc == sc) ? sc : 0.0f;
+				sc = sc > 3.0e38f ? 3.0e38f : (sc < -3.0e38f ? -3.0e38f : sc);
+				c.scale[q] = sc;
 			}
 		}
 		template<int ACT, bool VEC = false>
 		__device__ __forceinline__ void store(int64_t p, int k, const int (&v)[4], const Columns &c) const
 		{
-			store_at<ACT, VEC>(p * K + k, k, v, c);
+			store_at<ACT, VEC, 4>(p * K + k, k, v, c);
 		}
-		template<int ACT, bool VEC = false>
-		__device__ __forceinline__ void store_at(int64_t idx, int k, const int (&v)[4], const Columns &c) const
+		template<int ACT, bool VEC = false, int W = 4>
+		__device__ __forceinline__ void store_at(int64_t idx, int k, const int (&v)[W], const ColumnsT<W> &c) const
 		{
 			/* every fp32 operation below rounds exactly once: a * b + c must not become a fused multiply-add.  The pragma
 			 * governs the expressions written in this block, which is why they use plain operators and no intrinsics. */
 #pragma clang fp contract(off)
+			static_assert(VEC || W == 4, "`vec` vouches for 4-element vectors only; wider runs are for callers that checked");
 			const bool vec = VEC || this->vec;
-			const int valid = VEC ? 4 : K - k;
+			const int valid = VEC ? W : K - k;
 			if (MODE == I8_EXACT || MODE == I8_REQUANT)
 			{
-				int t[4];
+				int t[W];
 #pragma unroll
-				for (int q = 0; q < 4; q++)
+				for (int q = 0; q < W; q++)
 				{
 					t[q] = v[q] + c.ibias[q];
 					if (activation == ACT_RELU && t[q] < 0)
 						t[q] = 0;
 				}
+				/* whole runs leave as streaming vector stores: the kernel never reads y back, so the caches may drain it while
+				 * the kernel runs */
+				typedef typename Words<W / 4>::type words_t; /* W int8 values as 32-bit words */
 				if (MODE == I8_EXACT)
 				{
 					int *dst = static_cast<int*>(y) + idx;
-					if (vec && valid >= 4)
+					if (vec && valid >= W)
 					{
-						/* streaming store: the kernel never reads y back, so the caches may drain it while the kernel runs */
-						typedef int i32x4 __attribute__((ext_vector_type(4)));
-						const i32x4 pack = { t[0], t[1], t[2], t[3] };
-						__builtin_nontemporal_store(pack, reinterpret_cast<i32x4*>(dst));
+#pragma unroll
+						for (int part = 0; part < W / 4; part++)
+						{
+							typedef int i32x4 __attribute__((ext_vector_type(4)));
+							const i32x4 pack = { t[4 * part], t[4 * part + 1], t[4 * part + 2], t[4 * part + 3] };
+							__builtin_nontemporal_store(pack, reinterpret_cast<i32x4*>(dst) + part);
+						}
 					}
 					else
 					{
 #pragma unroll
-						for (int q = 0; q < 4; q++)
+						for (int q = 0; q < W; q++)
 							if (q < valid)
 								dst[q] = t[q];
 					}
 				}
 				else
 				{
-					int8_t o[4];
-#pragma unroll
-					for (int q = 0; q < 4; q++)
-						o[q] = static_cast<int8_t>(round_saturate(static_cast<float>(t[q]) * c.scale[q], -128.0f, 127.0f));
-					int8_t *dst = static_cast<int8_t*>(y) + idx;
-					if (vec && valid >= 4)
+					union
 					{
-						const unsigned int pack = (static_cast<unsigned int>(static_cast<unsigned char>(o[0]))) | (static_cast<unsigned int>(static_cast<unsigned char>(o[1])) << 8)
-								| (static_cast<unsigned int>(static_cast<unsigned char>(o[2])) << 16) | (static_cast<unsigned int>(static_cast<unsigned char>(o[3])) << 24);
-						__builtin_nontemporal_store(pack, reinterpret_cast<unsigned int*>(dst));
-					}
+						int8_t b[W];
+						words_t w;
+					} o;
+#pragma unroll
+					for (int q = 0; q < W; q++)
+						o.b[q] = static_cast<int8_t>(static_cast<int>(__builtin_amdgcn_fmed3f(rintf(static_cast<float>(t[q]) * c.scale[q]), -128.0f, 127.0f)));
+					int8_t *dst = static_cast<int8_t*>(y) + idx;
+					if (vec && valid >= W)
+						__builtin_nontemporal_store(o.w, reinterpret_cast<words_t*>(dst));
 					else
 					{
 #pragma unroll
-						for (int q = 0; q < 4; q++)
+						for (int q = 0; q < W; q++)
 							if (q < valid)
-								dst[q] = o[q];
+								dst[q] = o.b[q];
 					}
 				}
 			}
 			else
 			{
 #pragma unroll
-				for (int q = 0; q < 4; q++)
+				for (int q = 0; q < W; q++)
 				{
 					if (q >= valid)
 						continue;

@@ -78,8 +78,9 @@ namespace
 		const int n = b / g.tiles_h;
 		const int oh0 = th * g.TH, ow0 = tw * g.TW;
 		const int k0 = blockIdx.y * TILE_N;
-		const int kcol = k0 + drain_column<1>();
-		typename Epi::Columns columns;
+		constexpr int W = Epi::wide; /* filters per work-item in the epilogue: one 16-byte store each */
+		const int kcol = k0 + drain_column<1, W>();
+		typename Epi::template ColumnsT<W> columns;
 		epi.load_columns(kcol, columns);
 
 		const __amdgpu_buffer_rsrc_t rx = make_buffer(x, static_cast<unsigned int>(g.images) * g.H * g.W * g.C * SZ);
@@ -267,11 +268,11 @@ namespace
 
 		/* element index of (image n, pixel 0, filter kcol); one image of y is below 2^31 elements (checked by the launcher) */
 		const int64_t image_base = static_cast<int64_t>(n) * g.Ho * g.Wo * g.K + kcol;
-		drain_tile<TE, 2, 1>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[4]) __attribute__((always_inline))
+		drain_tile<TE, 2, 1, W>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[W]) __attribute__((always_inline))
 		{
 			const int e = row_table[row];
 			if (e >= 0 && kcol < g.K)
-				epi.template store_at<ACT_SIMPLE, true>(image_base + e * g.K, kcol, v, columns);
+				epi.template store_at<ACT_SIMPLE, true, W>(image_base + e * g.K, kcol, v, columns);
 		});
 	}
 
@@ -311,7 +312,8 @@ namespace avhip
 	{
 		if (s.stride_h != 1 || s.stride_w != 1 || s.dil_h != 1 || s.dil_w != 1)
 			return false;
-		if (!epi.vec) /* the kernel stores whole 4-filter vectors: K is a multiple of 4 and y, z are aligned */
+		/* the kernel stores whole runs of Epi::wide filters with one 16-byte instruction */
+		if (!epi.vec || s.K % Epi::wide != 0 || !aligned_to(epi.y, 16) || (epi.z != nullptr && !aligned_to(epi.z, 16)))
 			return false;
 		TileGeom g;
 		if (!choose_tile(s, g))

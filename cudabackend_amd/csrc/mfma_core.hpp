@@ -263,35 +263,37 @@ namespace avhip
 	 * 64 columns when they are stacked (WAVES_N = 1).  The accumulators go through LDS in TM passes so that afterwards each
 	 * work-item owns 4 consecutive columns of a row and neighbouring work-items cover a whole row: global stores are
 	 * contiguous rows.  A work-item always gets the same 4 columns (drain_column()), so per-column constants can be loaded
-	 * once, up front.  f(row, v) is called with the tile-relative row and the four accumulators v[0..3].
+	 * once, up front.  f(row, v) is called with the tile-relative row and the CPL accumulators v[0..CPL-1] (CPL = 4 unless the
+ * caller asks for 8 or 16 columns per work-item, which makes 16-byte stores of 2-byte and 1-byte outputs possible).
 	 * Must be called by all 256 work-items, after the last LDS read of the k loop; `lds` needs drain_bytes<WAVES_N>().
 	 */
-	template<int WAVES_N> struct DrainShape
+	template<int WAVES_N, int CPL = 4> struct DrainShape
 	{
 		static constexpr int cols = 64 * WAVES_N; /* columns of the workgroup tile */
 		static constexpr int pitch = cols + 4; /* words per LDS row: keeps rows 16-byte aligned and staggers banks */
 		static constexpr int rows_per_pass = 32 * (4 / WAVES_N); /* one 32-row MFMA tile of every wavefront row */
-		static constexpr int threads_per_row = cols / 4;
+		static constexpr int threads_per_row = cols / CPL; /* CPL: consecutive columns handed to one work-item (4, 8 or 16) */
 		static constexpr int bytes = rows_per_pass * pitch * 4;
 	};
-	template<int WAVES_N>
+	template<int WAVES_N, int CPL = 4>
 	__device__ inline int drain_column()
 	{
-		return (threadIdx.x % DrainShape<WAVES_N>::threads_per_row) * 4;
+		return (threadIdx.x % DrainShape<WAVES_N, CPL>::threads_per_row) * CPL;
 	}
-	template<typename TE, int TM, int WAVES_N, typename F>
+	template<typename TE, int TM, int WAVES_N, int CPL = 4, typename F>
 	__device__ __forceinline__ void drain_tile(char *lds, const typename Mma<TE>::acc_t (&acc)[TM][2], const F &f)
 	{
 		typedef typename Mma<TE>::scalar_t S;
-		typedef DrainShape<WAVES_N> D;
+		typedef DrainShape<WAVES_N, CPL> D;
 		static_assert(sizeof(S) == 4, "accumulators are 32-bit");
+		static_assert(CPL == 4 || CPL == 8 || CPL == 16, "a work-item takes 4, 8 or 16 consecutive columns");
 		S *sm = reinterpret_cast<S*>(lds);
 		const int tid = threadIdx.x;
 		const int lane = tid & 63;
 		const int wave = tid >> 6;
 		const int wm = WAVES_N == 2 ? (wave >> 1) : wave;
 		const int wn = WAVES_N == 2 ? (wave & 1) : 0;
-		const int col = drain_column<WAVES_N>();
+		const int col = drain_column<WAVES_N, CPL>();
 		constexpr int ROW_STEP = 256 / D::threads_per_row; /* rows covered by one sweep of the workgroup */
 #pragma unroll
 		for (int tm = 0; tm < TM; tm++)
@@ -307,16 +309,22 @@ namespace avhip
 			__syncthreads();
 			/* all LDS reads of the pass first, then the stores: the reads are independent and overlap */
 			constexpr int ITERS = D::rows_per_pass / ROW_STEP;
-			Pack<S, 4> vals[ITERS];
+			Pack<S, 4> vals[ITERS][CPL / 4];
 #pragma unroll
 			for (int it = 0; it < ITERS; it++)
-				vals[it] = *reinterpret_cast<const Pack<S, 4>*>(sm + (tid / D::threads_per_row + it * ROW_STEP) * D::pitch + col);
+#pragma unroll
+				for (int part = 0; part < CPL / 4; part++)
+					vals[it][part] = *reinterpret_cast<const Pack<S, 4>*>(sm + (tid / D::threads_per_row + it * ROW_STEP) * D::pitch + col + 4 * part);
 #pragma unroll
 			for (int it = 0; it < ITERS; it++)
 			{
 				const int rl = tid / D::threads_per_row + it * ROW_STEP; /* row within this pass */
 				const int row = (rl >> 5) * (TM * 32) + tm * 32 + (rl & 31);
-				f(row, vals[it].v);
+				S v[CPL];
+#pragma unroll
+				for (int q = 0; q < CPL; q++)
+					v[q] = vals[it][q / 4].v[q % 4];
+				f(row, v);
 			}
 		}
 	}
