@@ -62,6 +62,8 @@ PROTOTYPES = {
     "cudaSetConvolutionDescriptor": (i32, [i64, i32, i32, ip, ip, ip, i32, vp]),
     "cudaGetConvolutionDescriptor": (i32, [i64, ip, ip, ip, ip, ip, ip, vp]),
     "cudaChangeType": (i32, [i64, i64, i32, i64, i32, i64]),
+    "cudaAffineForward": (i32, [i64, i32, i64, i64, i64, i64, vp, i64, i64, vp, i64, i64]),
+    "cudaBatchNormInference": (i32, [i64, i32, vp, i64, i64, vp, i64, i64, i64, i64, i64, i64, i64, C.c_double]),
     "cudaAddBias": (i32, [i64, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, vp, i64, i32]),
     "cudaGemm": (i32, [i64, i32, i32, vp, i64, i64, i64, i64, vp, i64, i64]),
     "cudaGemmBatched": (i32, [i64, i32, i32, vp, i64, i64, i64, i64, vp, i64, i64]),
@@ -82,7 +84,8 @@ PROTOTYPES = {
 # the thin kernel layer of include/avocado_hip_kernels.h (exported, bound only for the symbol check)
 KERNEL_LAYER_SYMBOLS = ["avhip_winograd_weight_transform", "avhip_winograd_input_transform", "avhip_winograd_output_transform", "avhip_gemm_batched",
                         "avhip_conv2d_implicit_gemm", "avhip_conv2d_winograd_fused", "avhip_add_bias", "avhip_im2row", "avhip_change_type",
-                        "avhip_set_memory", "avhip_mfma_rate_probe", "avhip_set_small_problem_threshold"]
+                        "avhip_set_memory", "avhip_mfma_rate_probe", "avhip_set_small_problem_threshold",
+                        "avhip_affine_forward", "avhip_batchnorm_inference"]
 
 _lib = None
 

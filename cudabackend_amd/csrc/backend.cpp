@@ -699,6 +699,26 @@ namespace
 		}
 		return from_launcher(rc);
 	}
+
+	/* Shared validation of the two per-channel transforms: the parameter tensors hold one value per element of x's
+	 * trailing dimensions (volume(params) must divide volume(x)); fp32 parameters for 16-bit and fp32 tensors, fp64 for fp64. */
+	avStatus_t per_channel_view(const Tensor *x, const Tensor *y, const Tensor *params, av_int64 &first, av_int64 &last)
+	{
+		if (x == nullptr || y == nullptr || params == nullptr || x->nb_dims == 0)
+			return AVOCADO_STATUS_BAD_PARAM;
+		if (!is_floating(x->dtype))
+			return AVOCADO_STATUS_UNSUPPORTED_DATATYPE;
+		if (x->dtype != y->dtype || x->volume() != y->volume())
+			return AVOCADO_STATUS_BAD_PARAM;
+		const avDataType_t param_type = (x->dtype == AVOCADO_DTYPE_FLOAT64) ? AVOCADO_DTYPE_FLOAT64 : AVOCADO_DTYPE_FLOAT32;
+		if (params->dtype != param_type)
+			return AVOCADO_STATUS_UNSUPPORTED_DATATYPE;
+		last = params->volume();
+		if (last <= 0 || x->volume() % last != 0)
+			return AVOCADO_STATUS_BAD_PARAM;
+		first = x->volume() / last;
+		return AVOCADO_STATUS_SUCCESS;
+	}
 }
 
 namespace avocado
@@ -1165,6 +1185,62 @@ namespace avocado
 				return AVOCADO_STATUS_EXECUTION_FAILED;
 			touch(yMem);
 			return from_launcher(avhip_add_bias(ctx.stream, y->dtype, xm->data, bm->data, z, ym->data, first, last, a1, a2, b1, b2, b3, activation));
+		}
+
+		avStatus_t cudaAffineForward(avContextDescriptor_t context, avActivationType_t activation, const avTensorDescriptor_t wDesc,
+				const avMemoryDescriptor_t wMem, const avTensorDescriptor_t bDesc, const avMemoryDescriptor_t bMem, const void *alpha,
+				const avTensorDescriptor_t xDesc, const avMemoryDescriptor_t xMem, const void *beta, const avTensorDescriptor_t yDesc,
+				avMemoryDescriptor_t yMem)
+		{
+			Context ctx;
+			if (!get_context(context, ctx))
+				return AVOCADO_STATUS_BAD_PARAM;
+			const Tensor *x = get_tensor(xDesc), *y = get_tensor(yDesc), *w = get_tensor(wDesc), *b = get_tensor(bDesc);
+			av_int64 first = 0, last = 0;
+			const avStatus_t st = per_channel_view(x, y, b, first, last);
+			if (st != AVOCADO_STATUS_SUCCESS)
+				return st;
+			if (w == nullptr || w->dtype != b->dtype || w->volume() != last)
+				return AVOCADO_STATUS_BAD_PARAM;
+			Memory *xm = get_memory(xMem), *ym = get_memory(yMem), *wm = get_memory(wMem), *bm = get_memory(bMem);
+			const av_int64 bytes = x->volume() * size_of(x->dtype), param_bytes = last * size_of(b->dtype);
+			if (!fits(xm, bytes) || !fits(ym, bytes) || !fits(wm, param_bytes) || !fits(bm, param_bytes))
+				return AVOCADO_STATUS_BAD_PARAM;
+			if (hipSetDevice(ctx.device) != hipSuccess)
+				return AVOCADO_STATUS_EXECUTION_FAILED;
+			touch(yMem);
+			return from_launcher(avhip_affine_forward(ctx.stream, x->dtype, xm->data, ym->data, wm->data, bm->data, first, last,
+					scalar_or(alpha, x->dtype, 1.0), scalar_or(beta, x->dtype, 0.0), activation));
+		}
+
+		avStatus_t cudaBatchNormInference(avContextDescriptor_t context, avActivationType_t activation, const void *alpha, const avTensorDescriptor_t xDesc,
+				const avMemoryDescriptor_t xMem, const void *beta, const avTensorDescriptor_t yDesc, avMemoryDescriptor_t yMem,
+				const avTensorDescriptor_t scaleBiasMeanVarDesc, const avMemoryDescriptor_t scaleMem, const avMemoryDescriptor_t biasMem,
+				const avMemoryDescriptor_t meanMem, const avMemoryDescriptor_t varianceMem, double epsilon)
+		{
+			Context ctx;
+			if (!get_context(context, ctx))
+				return AVOCADO_STATUS_BAD_PARAM;
+			const Tensor *x = get_tensor(xDesc), *y = get_tensor(yDesc), *params = get_tensor(scaleBiasMeanVarDesc);
+			av_int64 first = 0, last = 0;
+			const avStatus_t st = per_channel_view(x, y, params, first, last);
+			if (st != AVOCADO_STATUS_SUCCESS)
+				return st;
+			if (!(epsilon >= 0.0))
+				return AVOCADO_STATUS_BAD_PARAM;
+			Memory *xm = get_memory(xMem), *ym = get_memory(yMem);
+			Memory *pm[4] = { get_memory(scaleMem), get_memory(biasMem), get_memory(meanMem), get_memory(varianceMem) };
+			const av_int64 bytes = x->volume() * size_of(x->dtype), param_bytes = last * size_of(params->dtype);
+			if (!fits(xm, bytes) || !fits(ym, bytes))
+				return AVOCADO_STATUS_BAD_PARAM;
+			for (int i = 0; i < 4; i++)
+				if (!fits(pm[i], param_bytes))
+					return AVOCADO_STATUS_BAD_PARAM;
+			if (hipSetDevice(ctx.device) != hipSuccess)
+				return AVOCADO_STATUS_EXECUTION_FAILED;
+			touch(yMem);
+			return from_launcher(avhip_batchnorm_inference(ctx.stream, x->dtype, xm->data, ym->data, pm[0]->data, pm[1]->data, pm[2]->data, pm[3]->data,
+					first, last, scalar_or(alpha, x->dtype, 1.0), scalar_or(beta, x->dtype, 0.0), epsilon, activation));
 		}
 
 		avStatus_t cudaGemm(avContextDescriptor_t context, avGemmOperation_t aOp, avGemmOperation_t bOp, const void *alpha,

@@ -79,6 +79,102 @@ namespace
 		return 0;
 	}
 
+	/* y = alpha * act(x * scale[j] + shift[j]) + beta * y over a [first, last] view, j the last index.
+	 * BN = false: scale = p0, shift = p1 (affine transform).  BN = true: the folded form of batch normalisation in
+	 * inference, scale = p0 / sqrt(p3 + epsilon), shift = p1 - p2 * scale with p0..p3 = scale, bias, mean, variance
+	 * (src/batchnorm.cu:28-69 of the reference: same operations in the same order). */
+	template<typename T, int V, bool BN>
+	__global__ __launch_bounds__(256) void k_affine(const T *__restrict__ x, T *y, const typename Traits<T>::compute *__restrict__ p0,
+			const typename Traits<T>::compute *__restrict__ p1, const typename Traits<T>::compute *__restrict__ p2,
+			const typename Traits<T>::compute *__restrict__ p3, int64_t first, int last, typename Traits<T>::compute alpha,
+			typename Traits<T>::compute beta, typename Traits<T>::compute epsilon, int activation)
+	{
+		typedef typename Traits<T>::compute CT;
+		const int LV = (last + V - 1) / V;
+		const int64_t gid = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+		const int64_t row = gid / LV;
+		if (row >= first)
+			return;
+		const int j = static_cast<int>(gid - row * LV) * V;
+		const int valid = last - j;
+		const int64_t idx = row * last + j;
+
+		CT xv[V], t[V];
+		load_vec<T, V, CT>(x + idx, valid, xv);
+#pragma unroll
+		for (int v = 0; v < V; v++)
+		{
+			CT scale = static_cast<CT>(0), shift = static_cast<CT>(0);
+			if (v < valid)
+			{
+				if (BN)
+				{
+					scale = p0[j + v] / sqrt(p3[j + v] + epsilon);
+					shift = p1[j + v] - p2[j + v] * scale;
+				}
+				else
+				{
+					scale = p0[j + v];
+					shift = p1[j + v];
+				}
+			}
+			t[v] = alpha * activation_forward<CT>(activation, xv[v] * scale + shift);
+		}
+		if (beta != static_cast<CT>(0))
+		{
+			CT yv[V];
+			load_vec<T, V, CT>(y + idx, valid, yv);
+#pragma unroll
+			for (int v = 0; v < V; v++)
+				t[v] += beta * yv[v];
+		}
+		store_vec<T, V, CT>(y + idx, valid, t);
+	}
+	template<typename T, bool BN>
+	int launch_affine(hipStream_t s, const void *x, void *y, const void *p0, const void *p1, const void *p2, const void *p3, int64_t first, int last,
+			double alpha, double beta, double epsilon, int activation)
+	{
+		typedef typename Traits<T>::compute CT;
+		constexpr int V = 16 / sizeof(T) > 4 ? 4 : 16 / sizeof(T);
+		const bool vec = last % V == 0 && aligned_to(x, V * sizeof(T)) && aligned_to(y, V * sizeof(T));
+		const int v = vec ? V : 1;
+		const int64_t items = first * ((last + v - 1) / v);
+		const dim3 grid(ceil_div(items, 256));
+#define ARGS static_cast<const T*>(x), static_cast<T*>(y), static_cast<const CT*>(p0), static_cast<const CT*>(p1), static_cast<const CT*>(p2), \
+		static_cast<const CT*>(p3), first, last, static_cast<CT>(alpha), static_cast<CT>(beta), static_cast<CT>(epsilon), activation
+		if (vec)
+			hipLaunchKernelGGL((k_affine<T, V, BN>), grid, dim3(256), 0, s, ARGS);
+		else
+			hipLaunchKernelGGL((k_affine<T, 1, BN>), grid, dim3(256), 0, s, ARGS);
+#undef ARGS
+		return 0;
+	}
+	template<bool BN>
+	int dispatch_affine(void *stream, int dtype, const void *x, void *y, const void *p0, const void *p1, const void *p2, const void *p3, int64_t first,
+			int64_t last, double alpha, double beta, double epsilon, int activation)
+	{
+		if (x == nullptr || y == nullptr || p0 == nullptr || p1 == nullptr || (BN && (p2 == nullptr || p3 == nullptr)) || first < 0 || last <= 0
+				|| last > 0x7FFFFFFF)
+			return AVHIP_BAD_PARAM;
+		if (first == 0)
+			return 0;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+		const int l = static_cast<int>(last);
+		switch (dtype)
+		{
+			case DT_FLOAT16:
+				return launch_affine<f16_t, BN>(s, x, y, p0, p1, p2, p3, first, l, alpha, beta, epsilon, activation);
+			case DT_BFLOAT16:
+				return launch_affine<bf16_t, BN>(s, x, y, p0, p1, p2, p3, first, l, alpha, beta, epsilon, activation);
+			case DT_FLOAT32:
+				return launch_affine<float, BN>(s, x, y, p0, p1, p2, p3, first, l, alpha, beta, epsilon, activation);
+			case DT_FLOAT64:
+				return launch_affine<double, BN>(s, x, y, p0, p1, p2, p3, first, l, alpha, beta, epsilon, activation);
+			default:
+				return AVHIP_UNSUPPORTED_DATATYPE;
+		}
+	}
+
 	/* rows[pixel, (i*S + j)*C + c] = x[n, pad_h + oh + i', pad_w + ow + j', c]; one work-item per element of `rows`. */
 	template<typename E>
 	__global__ __launch_bounds__(256) void k_im2row(const E *__restrict__ x, E *__restrict__ rows, avhipConvShape s, E padv, int64_t total)
@@ -279,6 +375,17 @@ extern "C"
 			default:
 				return AVHIP_UNSUPPORTED_DATATYPE;
 		}
+	}
+
+	int avhip_affine_forward(void *stream, int dtype, const void *x, void *y, const void *weight, const void *bias, int64_t first, int64_t last,
+			double alpha, double beta, int activation)
+	{
+		return dispatch_affine<false>(stream, dtype, x, y, weight, bias, nullptr, nullptr, first, last, alpha, beta, 0.0, activation);
+	}
+	int avhip_batchnorm_inference(void *stream, int dtype, const void *x, void *y, const void *scale, const void *bias, const void *mean,
+			const void *variance, int64_t first, int64_t last, double alpha, double beta, double epsilon, int activation)
+	{
+		return dispatch_affine<true>(stream, dtype, x, y, scale, bias, mean, variance, first, last, alpha, beta, epsilon, activation);
 	}
 
 	int avhip_set_memory(void *stream, void *dst, int64_t bytes, const void *pattern, int pattern_size)

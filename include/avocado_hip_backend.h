@@ -109,6 +109,21 @@ namespace avocado
 					avMemoryDescriptor_t yMem, const void *beta1, const void *beta2, const void *beta3, const avMemoryDescriptor_t zMem,
 					avActivationType_t activation);
 
+			/* cuda_backend.h:591.  y = alpha * activation(x * w + b) + beta * y with w, b broadcast over the trailing dimensions of
+			 * x that they span (src/batchnorm.cu:28-48, 315-340).  fp16 / bf16 / fp32 tensors with fp32 parameters, fp64 with fp64. */
+			DLL_PUBLIC avStatus_t cudaAffineForward(avContextDescriptor_t context, avActivationType_t activation, const avTensorDescriptor_t wDesc,
+					const avMemoryDescriptor_t wMem, const avTensorDescriptor_t bDesc, const avMemoryDescriptor_t bMem, const void *alpha,
+					const avTensorDescriptor_t xDesc, const avMemoryDescriptor_t xMem, const void *beta, const avTensorDescriptor_t yDesc,
+					avMemoryDescriptor_t yMem);
+
+			/* cuda_backend.h:612.  Batch normalisation with stored statistics: y = alpha * activation((x - mean) / sqrt(variance +
+			 * epsilon) * scale + bias) + beta * y, evaluated as x * s + t with s = scale / sqrt(variance + epsilon), t = bias - mean * s
+			 * (src/batchnorm.cu:51-69, 342-370).  Same data types as cudaAffineForward. */
+			DLL_PUBLIC avStatus_t cudaBatchNormInference(avContextDescriptor_t context, avActivationType_t activation, const void *alpha,
+					const avTensorDescriptor_t xDesc, const avMemoryDescriptor_t xMem, const void *beta, const avTensorDescriptor_t yDesc,
+					avMemoryDescriptor_t yMem, const avTensorDescriptor_t scaleBiasMeanVarDesc, const avMemoryDescriptor_t scaleMem,
+					const avMemoryDescriptor_t biasMem, const avMemoryDescriptor_t meanMem, const avMemoryDescriptor_t varianceMem, double epsilon);
+
 			/* cuda_backend.h:442.  C = alpha * opA(A) opB(B) + beta * C, row-major.  fp16 / bf16 / fp32 / fp64, and
 			 * int8 x int8 -> int32 with alpha, beta in {0, 1} and leading dimensions that are multiples of 4 (src/gemm.cpp:42-57). */
 			DLL_PUBLIC avStatus_t cudaGemm(avContextDescriptor_t context, avGemmOperation_t aOp, avGemmOperation_t bOp, const void *alpha,

@@ -91,6 +91,16 @@ extern "C"
 	/* Explicit im2row, stride 1.  Replaces kernel_im2row_conv2d, src/im2row.cu:29-66.  elem_size in bytes. */
 	AVHIP_API int avhip_im2row(void *stream, int elem_size, const avhipConvShape *shape, const void *x, void *rows, const void *padding_value);
 
+	/* y = alpha * act(x * weight[j] + bias[j]) + beta * y over a [first, last] view of x (j = last index).  Replaces
+	 * kernel_affine_forward, src/batchnorm.cu:28-48.  weight, bias: fp32 (fp64 for fp64 tensors). */
+	AVHIP_API int avhip_affine_forward(void *stream, int dtype, const void *x, void *y, const void *weight, const void *bias, int64_t first, int64_t last,
+			double alpha, double beta, int activation);
+
+	/* Batch normalisation in inference: the affine transform above with weight = scale / sqrt(variance + epsilon) and
+	 * bias = bias - mean * weight, computed on the fly.  Replaces kernel_batchnorm_forward, src/batchnorm.cu:51-69. */
+	AVHIP_API int avhip_batchnorm_inference(void *stream, int dtype, const void *x, void *y, const void *scale, const void *bias, const void *mean,
+			const void *variance, int64_t first, int64_t last, double alpha, double beta, double epsilon, int activation);
+
 	/* Element type conversion with round-to-nearest-even and saturation.  Replaces cudaChangeType's kernels,
 	 * src/conversions.cu:253-258. */
 	AVHIP_API int avhip_change_type(void *stream, void *dst, int dst_dtype, const void *src, int src_dtype, int64_t elements);

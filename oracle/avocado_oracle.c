@@ -25,6 +25,9 @@
  *   orc_add_bias              pinned: numpy restatement of the documented formula in two algebraic
  *                             forms; operation order from the reference kernel.
  *   orc_im2row                pinned: rows times flattened weights == orc_conv2d_f64.
+ *   orc_affine_forward        pinned: with weight 1 it is orc_add_bias (itself pinned); numpy broadcast form.
+ *   orc_batchnorm_inference   pinned: torch.nn.functional.batch_norm(training=False) in fp64; equals
+ *                             orc_affine_forward on the folded parameters.
  *   orc_conv2d_i8_float_epilogue  parity unpinned: the float epilogue on integer tensors follows
  *                             the header's prose convention only.
  *
@@ -39,6 +42,7 @@
  *   src/tensor_op.cu:199-228                 add-bias operation order
  *   src/gemm.cpp:126-145                     batched GEMM operand/shape mapping
  *   src/im2row.cu:29-66                      im2row slot order
+ *   src/batchnorm.cu:28-69                   affine forward and batch normalisation in inference
  */
 #include <math.h>
 #include <stdint.h>
@@ -497,6 +501,45 @@ void orc_add_bias(const double *x, const double *b, const double *z, double *y, 
 				t += beta3 * y[idx];
 			y[idx] = t;
 		}
+}
+
+/*
+ * y = alpha * act(x * weight[j] + bias[j]) + beta * y over a [first, last] view (src/batchnorm.cu:28-48).
+ */
+void orc_affine_forward(const double *x, const double *weight, const double *bias, double *y, int64_t first, int64_t last, double alpha, double beta,
+		int activation)
+{
+	for (int64_t i = 0; i < first; i++)
+		for (int64_t j = 0; j < last; j++)
+		{
+			const int64_t idx = i * last + j;
+			double t = alpha * activation_forward(activation, x[idx] * weight[j] + bias[j]);
+			if (beta != 0.0)
+				t += beta * y[idx];
+			y[idx] = t;
+		}
+}
+
+/*
+ * Batch normalisation with stored statistics (src/batchnorm.cu:51-69): per channel j
+ *   s = scale[j] / sqrt(variance[j] + epsilon),  t = bias[j] - mean[j] * s,  y = alpha * act(x * s + t) + beta * y.
+ */
+void orc_batchnorm_inference(const double *x, const double *scale, const double *bias, const double *mean, const double *variance, double *y,
+		int64_t first, int64_t last, double alpha, double beta, double epsilon, int activation)
+{
+	for (int64_t j = 0; j < last; j++)
+	{
+		const double s = scale[j] / sqrt(variance[j] + epsilon);
+		const double t = bias[j] - mean[j] * s;
+		for (int64_t i = 0; i < first; i++)
+		{
+			const int64_t idx = i * last + j;
+			double r = alpha * activation_forward(activation, x[idx] * s + t);
+			if (beta != 0.0)
+				r += beta * y[idx];
+			y[idx] = r;
+		}
+	}
 }
 
 /*

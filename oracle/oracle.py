@@ -220,6 +220,25 @@ def add_bias(x, b, z=None, y=None, alpha1=1.0, alpha2=1.0, beta1=0.0, beta2=0.0,
     return out
 
 
+def affine_forward(x, weight, bias, y=None, alpha=1.0, beta=0.0, activation=LINEAR):
+    """y = alpha * act(x * weight + bias) + beta * y, weight and bias spanning the trailing dimensions of x."""
+    x, weight, bias = _f64(x), _f64(weight), _f64(bias)
+    last = weight.size
+    out = np.zeros(x.shape, dtype=np.float64) if y is None else np.array(y, dtype=np.float64).reshape(x.shape)
+    lib().orc_affine_forward(_p(x), _p(weight), _p(bias), _p(out), C.c_int64(x.size // last), C.c_int64(last), C.c_double(alpha), C.c_double(beta),
+                             activation)
+    return out
+
+
+def batchnorm_inference(x, scale, bias, mean, variance, y=None, alpha=1.0, beta=0.0, epsilon=1e-5, activation=LINEAR):
+    x, scale, bias, mean, variance = _f64(x), _f64(scale), _f64(bias), _f64(mean), _f64(variance)
+    last = scale.size
+    out = np.zeros(x.shape, dtype=np.float64) if y is None else np.array(y, dtype=np.float64).reshape(x.shape)
+    lib().orc_batchnorm_inference(_p(x), _p(scale), _p(bias), _p(mean), _p(variance), _p(out), C.c_int64(x.size // last), C.c_int64(last),
+                                  C.c_double(alpha), C.c_double(beta), C.c_double(epsilon), activation)
+    return out
+
+
 def im2row(x, R, S, pad, mode=CONVOLUTION, padding_value=0.0):
     x = _f64(x)
     N, H, W, Cin = x.shape

@@ -185,3 +185,30 @@ def add_bias(x, b, dtype, z=None, y0=None, alpha1=None, alpha2=None, beta1=None,
         assert st == expect, cb.STATUS_NAMES[st]
         c.finish()
         return y.download() if st == cb.STATUS_SUCCESS else None
+
+
+def affine_forward(x, w, b, dtype, y0=None, alpha=None, beta=None, activation=0, expect=cb.STATUS_SUCCESS):
+    pdt = "f64" if dtype == "f64" else "f32"
+    with Call() as c:
+        xt, wt, bt = c.tensor(x, dtype), c.tensor(w, pdt), c.tensor(b, pdt)
+        y = c.tensor(y0, dtype) if y0 is not None else c.empty(x.shape, dtype)
+        d = DT[dtype]
+        st = c.lib.cudaAffineForward(c.ctx.handle, activation, wt.desc, wt.mem, bt.desc, bt.mem, cb.scalar(alpha, d), xt.desc, xt.mem, cb.scalar(beta, d),
+                                     y.desc, y.mem)
+        assert st == expect, cb.STATUS_NAMES[st]
+        c.finish()
+        return y.download() if st == cb.STATUS_SUCCESS else None
+
+
+def batchnorm_inference(x, scale, bias, mean, var, dtype, y0=None, alpha=None, beta=None, epsilon=1e-5, activation=0, expect=cb.STATUS_SUCCESS):
+    pdt = "f64" if dtype == "f64" else "f32"
+    with Call() as c:
+        xt = c.tensor(x, dtype)
+        ps = [c.tensor(p, pdt) for p in (scale, bias, mean, var)]
+        y = c.tensor(y0, dtype) if y0 is not None else c.empty(x.shape, dtype)
+        d = DT[dtype]
+        st = c.lib.cudaBatchNormInference(c.ctx.handle, activation, cb.scalar(alpha, d), xt.desc, xt.mem, cb.scalar(beta, d), y.desc, y.mem, ps[0].desc,
+                                          ps[0].mem, ps[1].mem, ps[2].mem, ps[3].mem, epsilon)
+        assert st == expect, cb.STATUS_NAMES[st]
+        c.finish()
+        return y.download() if st == cb.STATUS_SUCCESS else None

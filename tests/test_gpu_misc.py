@@ -130,3 +130,25 @@ def test_memory_entries():
     assert lib.cudaDestroyMemoryDescriptor(m.value) == cb.STATUS_BAD_PARAM
     assert lib.cudaDestroyContextDescriptor(dflt) == cb.STATUS_BAD_PARAM                                # the default context cannot be destroyed
     ctx.close()
+
+
+@pytest.mark.parametrize("dtype,tol", [("f16", 1e-3), ("bf16", 1e-2), ("f32", 1e-6), ("f64", 1e-13)])
+def test_affine_forward_and_batchnorm_inference(oracle, dtype, tol):
+    """src/batchnorm.cu:28-69: y = alpha * act(x * s + t) + beta * y per channel; folded batch normalisation.  Ragged and
+    vector-friendly channel counts, parameters spanning one or two trailing dimensions."""
+    g = h.rng(60)
+    sfun = (lambda v: v) if dtype == "f64" else (lambda v: float(np.float32(v)))
+    par = (lambda a: a) if dtype == "f64" else (lambda a: a.astype(np.float32).astype(np.float64))
+    for shape, pshape in (((3, 7, 5, 13), (13,)), ((4, 6, 6, 64), (64,)), ((5, 3, 8), (3, 8))):
+        x = h.rounded(oracle, g.standard_normal(shape), dtype)
+        y0 = h.rounded(oracle, g.standard_normal(shape), dtype)
+        w, b, mean = par(g.standard_normal(pshape)), par(g.standard_normal(pshape)), par(g.standard_normal(pshape))
+        var = par(g.uniform(0.2, 2.0, pshape))
+        for act in (cb.ACTIVATION_LINEAR, cb.ACTIVATION_RELU, cb.ACTIVATION_SIGMOID):
+            got = h.affine_forward(x, w, b, dtype, y0, sfun(1.1), sfun(0.3), activation=act)
+            assert oracle.rel_l2(got, oracle.affine_forward(x, w, b, y0, sfun(1.1), sfun(0.3), activation=act)) < tol
+            got = h.batchnorm_inference(x, w, b, mean, var, dtype, None, None, None, 1e-3, activation=act)
+            assert oracle.rel_l2(got, oracle.batchnorm_inference(x, w, b, mean, var, epsilon=1e-3, activation=act)) < tol * 3
+    x = np.zeros((2, 4, 8))
+    h.affine_forward(x, np.zeros(5), np.zeros(5), "f32", expect=cb.STATUS_BAD_PARAM)  # 5 does not divide 64
+    h.affine_forward(x.astype(np.int32), np.zeros(8), np.zeros(8), "i32", expect=cb.STATUS_UNSUPPORTED_DATATYPE)

@@ -257,3 +257,45 @@ def test_bf16_rounding_helpers(oracle):
     np.testing.assert_array_equal(back, t)
     big = RNG.standard_normal(10000).astype(np.float32)
     np.testing.assert_array_equal(oracle.bf16_bits_to_f32(oracle.f32_to_bf16_bits(big)), torch.tensor(big).to(torch.bfloat16).to(torch.float32).numpy())
+
+
+# ---- per-channel transforms: affine forward and batch normalisation in inference (src/batchnorm.cu:28-69) ---------------
+def test_affine_forward_reduces_to_add_bias_and_broadcast_form(oracle):
+    g = np.random.default_rng(77)
+    x = g.standard_normal((5, 6, 7, 12))
+    w = g.standard_normal(12)
+    b = g.standard_normal(12)
+    y0 = g.standard_normal(x.shape)
+    for act in (oracle.LINEAR, oracle.RELU, oracle.TANH):
+        # weight 1: the add-bias routine, which has its own pins (y = alpha1 * act(x + b) + beta3 * y)
+        got = oracle.affine_forward(x, np.ones(12), b, y0, alpha=1.3, beta=0.4, activation=act)
+        want = oracle.add_bias(x, b, None, y0, alpha1=1.3, alpha2=1.0, beta3=0.4, activation=act)
+        np.testing.assert_allclose(got, want, rtol=0, atol=1e-14)
+        # general weight: x * w is x with its channels pre-scaled
+        got = oracle.affine_forward(x, w, b, None, alpha=0.7, activation=act)
+        want = oracle.add_bias(x * w, b, alpha1=0.7, activation=act)
+        np.testing.assert_allclose(got, want, rtol=0, atol=1e-14)
+    # parameters spanning the two trailing dimensions
+    w2, b2 = g.standard_normal((7, 12)), g.standard_normal((7, 12))
+    np.testing.assert_allclose(oracle.affine_forward(x, w2, b2), x * w2 + b2, rtol=0, atol=1e-14)
+
+
+def test_batchnorm_inference_matches_torch_and_folded_affine(oracle):
+    import torch
+    g = np.random.default_rng(78)
+    x = g.standard_normal((4, 5, 6, 16)) * 2 + 0.5
+    scale, bias, mean = g.standard_normal(16), g.standard_normal(16), g.standard_normal(16)
+    var = g.uniform(0.1, 2.0, 16)
+    eps = 1e-3
+    got = oracle.batchnorm_inference(x, scale, bias, mean, var, epsilon=eps)
+    # independent library routine: channels-last data moved to torch's channel-second layout
+    t = torch.nn.functional.batch_norm(torch.from_numpy(x).permute(0, 3, 1, 2), torch.from_numpy(mean), torch.from_numpy(var), torch.from_numpy(scale),
+                                       torch.from_numpy(bias), training=False, eps=eps)
+    np.testing.assert_allclose(got, t.permute(0, 2, 3, 1).numpy(), rtol=0, atol=1e-12)
+    s = scale / np.sqrt(var + eps)
+    y0 = g.standard_normal(x.shape)
+    got = oracle.batchnorm_inference(x, scale, bias, mean, var, y0, alpha=1.1, beta=0.3, epsilon=eps, activation=oracle.RELU)
+    want = oracle.affine_forward(x, s, bias - mean * s, y0, alpha=1.1, beta=0.3, activation=oracle.RELU)
+    np.testing.assert_allclose(got, want, rtol=0, atol=1e-13)
+    # identity statistics leave x unchanged
+    np.testing.assert_allclose(oracle.batchnorm_inference(x, np.ones(16), np.zeros(16), np.zeros(16), np.ones(16), epsilon=0.0), x, rtol=0, atol=0)
