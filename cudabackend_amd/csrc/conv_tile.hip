@@ -86,38 +86,6 @@ namespace
 		const __amdgpu_buffer_rsrc_t rx = make_buffer(x, static_cast<unsigned int>(g.images) * g.H * g.W * g.C * SZ);
 		const __amdgpu_buffer_rsrc_t rw = make_buffer(w, static_cast<unsigned int>(g.K) * g.R * g.S * g.C * SZ);
 
-		/* where this work-item's halo chunks come from (slice 0) and go to */
-		/* Integer division by a run-time divisor costs about thirty instructions: the work-item divides once and then walks. */
-		int *row_table = reinterpret_cast<int*>(lds + ROW_TABLE);
-		{
-			/* GEMM row -> offset of its output pixel inside the image, in pixels; -1 for rows that are not stored */
-			const int py = tid / g.HW, px = tid - py * g.HW;
-			const int oh = oh0 + py, ow = ow0 + px;
-			row_table[tid] = (py < g.TH && px < g.TW && oh < g.Ho && ow < g.Wo) ? oh * g.Wo + ow : -1;
-		}
-		unsigned int halo_src[HALO_FETCHES];
-		const int halo_pixels = g.HH * g.HW;
-		{
-			constexpr int STRIDE = 256 / STEP_CHUNKS; /* halo pixels between two fetches of a work-item */
-			const int dy = STRIDE / g.HW, dx = STRIDE - dy * g.HW;
-			int h = tid / STEP_CHUNKS;
-			int hy = h / g.HW, hx = h - hy * g.HW;
-#pragma unroll
-			for (int f = 0; f < HALO_FETCHES; f++)
-			{
-				const int ih = oh0 + g.pad_h + hy, iw = ow0 + g.pad_w + hx;
-				const bool inside = (h < halo_pixels) & (ih >= 0) & (ih < g.H) & (iw >= 0) & (iw < g.W);
-				halo_src[f] = inside ? static_cast<unsigned int>(((n * g.H + ih) * g.W + iw) * g.C + chunk_channel) * SZ : OUT_OF_RANGE;
-				h += STRIDE;
-				hy += dy;
-				hx += dx;
-				if (hx >= g.HW)
-				{
-					hx -= g.HW;
-					hy++;
-				}
-			}
-		}
 		const int halo_dst = (tid / STEP_CHUNKS) * PIXEL_PITCH + part * 16;
 		unsigned int filt_src[FILTER_FETCHES];
 #pragma unroll
@@ -127,24 +95,15 @@ namespace
 			filt_src[f] = k < g.K ? static_cast<unsigned int>(k * g.R * g.S * g.C + chunk_channel) * SZ : OUT_OF_RANGE;
 		}
 		const int filt_dst = (tid / STEP_CHUNKS) * LDS_ROW + part * 16;
-
-		/* MFMA operand addresses: lane l supplies row (l % 32) of a 32-row tile and k-chunk (l / 32) */
-		int a_off[2];
-		const int b_off = (lane & 31) * LDS_ROW + (lane >> 5) * 16;
-
+		unsigned int halo_src[HALO_FETCHES];
+		const int halo_pixels = g.HH * g.HW;
 		const int taps = g.R * g.S;
 		const int total = g.slices * taps;
 		const int prefetch_tap = taps > 2 ? 2 : taps - 1;
-		typename Mma<TE>::acc_t acc[2][2];
-#pragma unroll
-		for (int i = 0; i < 2; i++)
-#pragma unroll
-			for (int j = 0; j < 2; j++)
-#pragma unroll
-				for (int v = 0; v < 16; v++)
-					acc[i][j][v] = 0;
 
-		/* fetch side: runs two steps ahead of the MFMAs */
+		/* fetch side: runs three steps ahead of the MFMAs.  The first requests go out before anything else is computed: the
+		 * addresses of the filters are the cheapest to form, the halo's follow, and the bookkeeping that needs no memory (row
+		 * table, accumulators) is done while they travel. */
 		int f_slice = 0, f_tap = 0;
 		auto fetch_filters = [&](uint4 (&r)[FILTER_FETCHES]) __attribute__((always_inline))
 		{
@@ -179,6 +138,56 @@ namespace
 				if (tid / STEP_CHUNKS + f * (256 / STEP_CHUNKS) < HALO_MAX)
 					*reinterpret_cast<uint4*>(halo + halo_dst + f * (256 / STEP_CHUNKS) * PIXEL_PITCH) = r[f];
 		};
+		uint4 hr[HALO_FETCHES];
+		uint4 fr[3][FILTER_FETCHES];
+		fetch_filters(fr[0]);
+		fetch_filters(fr[1]);
+		fetch_filters(fr[2]);
+		/* where this work-item's halo chunks come from (slice 0).  Integer division by a run-time divisor costs about thirty
+		 * instructions: the work-item divides once and then walks. */
+		{
+			constexpr int STRIDE = 256 / STEP_CHUNKS; /* halo pixels between two fetches of a work-item */
+			const int dy = STRIDE / g.HW, dx = STRIDE - dy * g.HW;
+			int h = tid / STEP_CHUNKS;
+			int hy = h / g.HW, hx = h - hy * g.HW;
+#pragma unroll
+			for (int f = 0; f < HALO_FETCHES; f++)
+			{
+				const int ih = oh0 + g.pad_h + hy, iw = ow0 + g.pad_w + hx;
+				const bool inside = (h < halo_pixels) & (ih >= 0) & (ih < g.H) & (iw >= 0) & (iw < g.W);
+				halo_src[f] = inside ? static_cast<unsigned int>(((n * g.H + ih) * g.W + iw) * g.C + chunk_channel) * SZ : OUT_OF_RANGE;
+				h += STRIDE;
+				hy += dy;
+				hx += dx;
+				if (hx >= g.HW)
+				{
+					hx -= g.HW;
+					hy++;
+				}
+			}
+		}
+		fetch_halo(0, hr);
+		int *row_table = reinterpret_cast<int*>(lds + ROW_TABLE);
+		{
+			/* GEMM row -> offset of its output pixel inside the image, in pixels; -1 for rows that are not stored */
+			const int py = tid / g.HW, px = tid - py * g.HW;
+			const int oh = oh0 + py, ow = ow0 + px;
+			row_table[tid] = (py < g.TH && px < g.TW && oh < g.Ho && ow < g.Wo) ? oh * g.Wo + ow : -1;
+		}
+
+		/* MFMA operand addresses: lane l supplies row (l % 32) of a 32-row tile and k-chunk (l / 32) */
+		int a_off[2];
+		const int b_off = (lane & 31) * LDS_ROW + (lane >> 5) * 16;
+
+		typename Mma<TE>::acc_t acc[2][2];
+#pragma unroll
+		for (int i = 0; i < 2; i++)
+#pragma unroll
+			for (int j = 0; j < 2; j++)
+#pragma unroll
+				for (int v = 0; v < 16; v++)
+					acc[i][j][v] = 0;
+
 		/* compute side */
 		int c_slice = 0, c_i = 0, c_j = 0;
 		auto multiply = [&](int buffer) __attribute__((always_inline))
@@ -212,12 +221,6 @@ namespace
 			}
 		};
 
-		uint4 hr[HALO_FETCHES];
-		uint4 fr[3][FILTER_FETCHES];
-		fetch_halo(0, hr);
-		fetch_filters(fr[0]);
-		fetch_filters(fr[1]);
-		fetch_filters(fr[2]);
 #pragma unroll
 		for (int tm = 0; tm < 2; tm++)
 			a_off[tm] = (wave * 64 + tm * 32 + (lane & 31)) * PIXEL_PITCH + (lane >> 5) * 16;
