@@ -82,9 +82,21 @@ namespace avhip
 		{
 			store_at<ACT, VEC, 4>(p * K + k, k, v, c);
 		}
+		/* W values of the residual z, fetched ahead of the epilogue by callers that know their rows early: a load issued
+		 * inside the store loop cannot pass the stores before it (y and z may alias) and its latency adds up row by row. */
+		template<int W> struct Residual
+		{
+			Pack<TE, W> raw;
+		};
+		template<int W>
+		__device__ __forceinline__ void load_residual(int64_t idx, Residual<W> &r) const
+		{
+			if (z != nullptr)
+				r.raw = *reinterpret_cast<const Pack<TE, W>*>(z + idx); /* whole, aligned runs only (VEC callers) */
+		}
 		/* idx: element index of (pixel, filter k) in y and z, for callers that keep it cheaper than p * K + k */
 		template<int ACT, bool VEC = false, int W = 4>
-		__device__ __forceinline__ void store_at(int64_t idx, int k, const float (&v)[W], const ColumnsT<W> &c) const
+		__device__ __forceinline__ void store_at(int64_t idx, int k, const float (&v)[W], const ColumnsT<W> &c, const Residual<W> *fetched = nullptr) const
 		{
 			static_assert(VEC || W == 4, "`vec` vouches for 4-element vectors only; wider runs are for callers that checked");
 			const bool vec = VEC || this->vec;
@@ -96,7 +108,14 @@ namespace avhip
 			if (z != nullptr)
 			{
 				float zv[W];
-				load_vec<TE, W, float>(z + idx, valid, zv, vec);
+				if (fetched != nullptr)
+				{
+#pragma unroll
+					for (int q = 0; q < W; q++)
+						zv[q] = Traits<TE>::load(fetched->raw.v[q]);
+				}
+				else
+					load_vec<TE, W, float>(z + idx, valid, zv, vec);
 #pragma unroll
 				for (int q = 0; q < W; q++)
 					t[q] += alpha2 * zv[q];
@@ -188,8 +207,15 @@ namespace avhip
 		{
 			store_at<ACT, VEC, 4>(p * K + k, k, v, c);
 		}
+		template<int W> struct Residual /* nothing is fetched ahead on the integer paths */
+		{
+		};
+		template<int W>
+		__device__ __forceinline__ void load_residual(int64_t, Residual<W>&) const
+		{
+		}
 		template<int ACT, bool VEC = false, int W = 4>
-		__device__ __forceinline__ void store_at(int64_t idx, int k, const int (&v)[W], const ColumnsT<W> &c) const
+		__device__ __forceinline__ void store_at(int64_t idx, int k, const int (&v)[W], const ColumnsT<W> &c, const Residual<W>* = nullptr) const
 		{
 			/* every fp32 operation below rounds exactly once: a * b + c must not become a fused multiply-add.  The pragma
 			 * governs the expressions written in this block, which is why they use plain operators and no intrinsics. */

@@ -424,7 +424,7 @@ namespace
 		typename Mma<TE>::acc_t acc[2][2];
 		block_mma<TE>(lds, g.R * g.S * g.steps_per_tap, la, lb, acc);
 
-		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const typename Epi::scalar_t (&v)[4]) __attribute__((always_inline))
+		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const typename Epi::scalar_t (&v)[4], int) __attribute__((always_inline))
 		{
 			const int64_t p = p0 + r;
 			if (p < g.pixels && k < g.K)
@@ -446,7 +446,7 @@ namespace
 		typename Mma<TE>::acc_t acc[2][2];
 		block_mma<TE>(lds, (g.R * g.S * g.C * static_cast<int>(sizeof(TE)) + STEP_BYTES - 1) / STEP_BYTES, la, lb, acc);
 
-		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const typename Epi::scalar_t (&v)[4]) __attribute__((always_inline))
+		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const typename Epi::scalar_t (&v)[4], int) __attribute__((always_inline))
 		{
 			const int64_t p = p0 + r;
 			if (p < g.pixels && k < g.K)

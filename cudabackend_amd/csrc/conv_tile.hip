@@ -227,6 +227,23 @@ namespace
 		stash_halo(hr);
 		stash_filters(0, fr[0]);
 
+		/* The residual of every row this work-item will store is requested during the last channel slice: its latency and its
+		 * HBM traffic run under the MFMAs of that slice instead of in the epilogue, and the registers are held for half the
+		 * loop only. */
+		typedef DrainRows<2, 1, W> Rows;
+		const int64_t image_base = static_cast<int64_t>(n) * g.Ho * g.Wo * g.K + kcol; /* element index of (image n, pixel 0, filter kcol); one image of y is below 2^31 elements (checked by the launcher) */
+		typename Epi::template Residual<W> residual[Rows::slots];
+		auto fetch_residual = [&]() __attribute__((always_inline))
+		{
+#pragma unroll
+			for (int slot = 0; slot < Rows::slots; slot++)
+			{
+				const int e = row_table[Rows::row(slot)];
+				if (e >= 0 && kcol < g.K)
+					epi.load_residual(image_base + e * g.K, residual[slot]);
+			}
+		};
+
 		/* One step = one tap of one channel slice.  The filters of step t are requested at step t - 3 into register set t % 3,
 		 * go to LDS buffer t % 2 at the end of step t - 1 and are multiplied at step t: a load from L2 has two full steps of
 		 * MFMAs to arrive.  Six steps per trip keep the set and buffer indices compile-time constants; fetches past the last
@@ -241,6 +258,8 @@ namespace
 			const bool more_slices = c_slice + 1 < g.slices;
 			if (prefetch_now & more_slices)
 				fetch_halo(c_slice + 1, hr);
+			if (prefetch_now & !more_slices)
+				fetch_residual(); /* after the barrier above, so the row table is complete */
 			if (s < total)
 				multiply(buffer);
 			stash_filters(buffer ^ 1, next); /* step s + 1 */
@@ -269,13 +288,11 @@ namespace
 			step(s + 5, 1, fr[2], fr[0]);
 		}
 
-		/* element index of (image n, pixel 0, filter kcol); one image of y is below 2^31 elements (checked by the launcher) */
-		const int64_t image_base = static_cast<int64_t>(n) * g.Ho * g.Wo * g.K + kcol;
-		drain_tile<TE, 2, 1, W>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[W]) __attribute__((always_inline))
+		drain_tile<TE, 2, 1, W>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[W], int slot) __attribute__((always_inline))
 		{
 			const int e = row_table[row];
 			if (e >= 0 && kcol < g.K)
-				epi.template store_at<ACT_SIMPLE, true, W>(image_base + e * g.K, kcol, v, columns);
+				epi.template store_at<ACT_SIMPLE, true, W>(image_base + e * g.K, kcol, v, columns, &residual[slot]);
 		});
 	}
 

@@ -349,7 +349,7 @@ namespace
 			for (int b = 0; b < 2; b++)
 			{
 				typename Kernel::acc_t plane[1][2] = { { kn.Y[a][b][0], kn.Y[a][b][1] } };
-				drain_tile<TL, 1, 2>(lds, plane, [&](int row, const float (&v)[4]) __attribute__((always_inline))
+				drain_tile<TL, 1, 2>(lds, plane, [&](int row, const float (&v)[4], int) __attribute__((always_inline))
 				{
 					const int th = TILE_BLOCK * block_h + (row >> 3), tw = TILE_BLOCK * block_w + (row & 7);
 					const int oh = 2 * th + a, ow = 2 * tw + b;

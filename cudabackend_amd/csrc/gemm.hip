@@ -132,7 +132,7 @@ namespace
 		TC *c = C + batch * strideC;
 		const bool vec_c = (vec_ok & 2) != 0;
 		const int cc = n0 + drain_column<2>();
-		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const typename Mma<TE>::scalar_t (&v)[4]) __attribute__((always_inline))
+		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const typename Mma<TE>::scalar_t (&v)[4], int) __attribute__((always_inline))
 		{
 			const int row = m0 + r;
 			if (row < M && cc < N)

@@ -263,8 +263,9 @@ namespace avhip
 	 * 64 columns when they are stacked (WAVES_N = 1).  The accumulators go through LDS in TM passes so that afterwards each
 	 * work-item owns 4 consecutive columns of a row and neighbouring work-items cover a whole row: global stores are
 	 * contiguous rows.  A work-item always gets the same 4 columns (drain_column()), so per-column constants can be loaded
-	 * once, up front.  f(row, v) is called with the tile-relative row and the CPL accumulators v[0..CPL-1] (CPL = 4 unless the
- * caller asks for 8 or 16 columns per work-item, which makes 16-byte stores of 2-byte and 1-byte outputs possible).
+	 * once, up front.  f(row, v, slot) is called with the tile-relative row, the CPL accumulators v[0..CPL-1] (CPL = 4 unless the
+ * caller asks for 8 or 16 columns per work-item, which makes 16-byte stores of 2-byte and 1-byte outputs possible) and the
+	 * number of the call (DrainRows<...>::row(slot) is that row: a caller can prefetch per-row data long before the drain).
 	 * Must be called by all 256 work-items, after the last LDS read of the k loop; `lds` needs drain_bytes<WAVES_N>().
 	 */
 	template<int WAVES_N, int CPL = 4> struct DrainShape
@@ -280,6 +281,20 @@ namespace avhip
 	{
 		return (threadIdx.x % DrainShape<WAVES_N, CPL>::threads_per_row) * CPL;
 	}
+	/* The rows a work-item is handed by drain_tile, in the order of its calls: slot = tm * iterations + it. */
+	template<int TM, int WAVES_N, int CPL = 4> struct DrainRows
+	{
+		typedef DrainShape<WAVES_N, CPL> D;
+		static constexpr int row_step = 256 / D::threads_per_row; /* rows covered by one sweep of the workgroup */
+		static constexpr int iterations = D::rows_per_pass / row_step;
+		static constexpr int slots = TM * iterations;
+		__device__ static inline int row(int slot)
+		{
+			const int tm = slot / iterations, it = slot - tm * iterations;
+			const int rl = threadIdx.x / D::threads_per_row + it * row_step; /* row within the pass */
+			return (rl >> 5) * (TM * 32) + tm * 32 + (rl & 31);
+		}
+	};
 	template<typename TE, int TM, int WAVES_N, int CPL = 4, typename F>
 	__device__ __forceinline__ void drain_tile(char *lds, const typename Mma<TE>::acc_t (&acc)[TM][2], const F &f)
 	{
@@ -318,13 +333,11 @@ namespace avhip
 #pragma unroll
 			for (int it = 0; it < ITERS; it++)
 			{
-				const int rl = tid / D::threads_per_row + it * ROW_STEP; /* row within this pass */
-				const int row = (rl >> 5) * (TM * 32) + tm * 32 + (rl & 31);
 				S v[CPL];
 #pragma unroll
 				for (int q = 0; q < CPL; q++)
 					v[q] = vals[it][q / 4].v[q % 4];
-				f(row, v);
+				f(DrainRows<TM, WAVES_N, CPL>::row(tm * ITERS + it), v, tm * ITERS + it);
 			}
 		}
 	}
