@@ -393,6 +393,7 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--quick", action="store_true", help="headline tower only (no side legs, no CPU baseline)")
     ap.add_argument("--calibrate", action="store_true", help="also launch a streaming kernel of known traffic (for counter runs)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (for counter runs, where only the GPU side matters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards over the batch with no collectives)." % args.gpus,
@@ -420,7 +421,7 @@ def main():
         detail["copy_GBs_measured"] = copy_bandwidth(hip, ctx)
         detail["mfma_rate_measured"] = mfma_rates(hip, ctx)
         detail["other_configs"] = other_configs(hip, ctx, it)
-        cpu = cpu_baseline()
+        cpu = None if args.no_cpu else cpu_baseline()
     ctx.close()
     peak = PEAK[args.dtype]
     line = {

@@ -159,6 +159,17 @@ namespace avhip
 		asm volatile("" : "+s"(v));
 	}
 
+	/* Workgroups of a grid are handed to the eight XCDs of the chip round-robin (workgroup b runs on XCD b % 8) and every
+	 * XCD has its own L2.  Kernels whose neighbouring blocks of work share input (tiles with halos, pixel blocks whose filter
+	 * windows overlap) renumber their workgroups so that each XCD owns a contiguous eighth of the blocks: workgroup b of nb
+	 * takes block (b % 8) * (nb / 8) + b / 8; the last nb % 8 workgroups keep their own number. */
+	__device__ inline unsigned int xcd_block(unsigned int b, unsigned int nb)
+	{
+		constexpr unsigned int XCDS = 8;
+		const unsigned int per_xcd = nb / XCDS;
+		return b < per_xcd * XCDS ? (b % XCDS) * per_xcd + b / XCDS : b;
+	}
+
 	/* Forward activations, src/activations.cuh:202-425 of the reference. */
 	template<typename CT>
 	__device__ inline CT activation_forward(int act, CT x)

@@ -414,7 +414,8 @@ namespace
 	__global__ __launch_bounds__(256, 2) void k_conv_igemm(const TE *__restrict__ x, const TE *__restrict__ w, ConvGeom g, TE padv, int vec_ok, Epi epi)
 	{
 		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
-		const int64_t p0 = static_cast<int64_t>(blockIdx.x) * BLOCK_M;
+		/* neighbouring pixel blocks read overlapping input windows: one XCD (one L2) gets a contiguous run of them */
+		const int64_t p0 = static_cast<int64_t>(xcd_block(blockIdx.x, gridDim.x)) * BLOCK_M;
 		const int k = blockIdx.y * BLOCK_N + drain_column<2>();
 		typename Epi::Columns columns;
 		epi.load_columns(k, columns); /* issued before the k loop: its latency is hidden behind the whole convolution */
@@ -436,7 +437,8 @@ namespace
 	__global__ __launch_bounds__(256, 2) void k_conv_igemm_packed(const TE *__restrict__ x, const TE *__restrict__ w, ConvGeom g, Epi epi)
 	{
 		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
-		const int64_t p0 = static_cast<int64_t>(blockIdx.x) * BLOCK_M;
+		/* neighbouring pixel blocks read overlapping input windows: one XCD (one L2) gets a contiguous run of them */
+		const int64_t p0 = static_cast<int64_t>(xcd_block(blockIdx.x, gridDim.x)) * BLOCK_M;
 		const int k = blockIdx.y * BLOCK_N + drain_column<2>();
 		typename Epi::Columns columns;
 		epi.load_columns(k, columns);

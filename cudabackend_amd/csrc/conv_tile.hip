@@ -71,7 +71,7 @@ namespace
 		const int part = tid % STEP_CHUNKS;
 		const int chunk_channel = part * E;
 
-		int b = blockIdx.x;
+		int b = static_cast<int>(xcd_block(blockIdx.x, gridDim.x)); /* tiles of an image share halo pixels: one XCD, one L2 */
 		const int tw = b % g.tiles_w;
 		b /= g.tiles_w;
 		const int th = b % g.tiles_h;

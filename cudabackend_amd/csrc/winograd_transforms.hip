@@ -164,7 +164,8 @@ namespace
 		constexpr bool FULL = V > 1;
 		const IDX CV = static_cast<IDX>((C + V - 1) / V);
 		const IDX tiles = static_cast<IDX>(N) * Th * Tw;
-		const IDX gid = static_cast<IDX>(blockIdx.x) * 256 + threadIdx.x;
+		/* neighbouring tiles share input pixels: consecutive runs of tiles go to one XCD, whose L2 then serves the overlap */
+		const IDX gid = static_cast<IDX>(xcd_block(blockIdx.x, gridDim.x)) * 256 + threadIdx.x;
 		const IDX tile = gid / CV;
 		const int cv = static_cast<int>(gid - tile * CV);
 		if (tile >= tiles)
