@@ -91,7 +91,7 @@ namespace
 			for (int q = 0; q < 4; q++)
 				v[q] += beta * old[q];
 		}
-		store_vec<TC, 4, float>(p, valid, v, vec);
+		store_vec<TC, 4, float, true>(p, valid, v, vec); /* streaming: C is not read back by this kernel */
 	}
 	__device__ inline void store_c(int *p, int valid, bool vec, const int (&acc)[4], int alpha, int beta)
 	{
