@@ -38,7 +38,8 @@ namespace
 		const int lane = threadIdx.x;
 		const int r = lane & 31;
 		const unsigned int half = (lane >> 5) * 16;
-		const int p0 = blockIdx.x * SMALL_TILE, k0 = blockIdx.y * SMALL_TILE;
+		/* neighbouring pixel tiles read overlapping windows: a contiguous run of them goes to one XCD and its L2 */
+		const int p0 = static_cast<int>(xcd_block(blockIdx.x, gridDim.x)) * SMALL_TILE, k0 = blockIdx.y * SMALL_TILE;
 		const int kcol = k0 + (lane & 7) * 4;
 		typename Epi::Columns columns;
 		epi.load_columns(kcol, columns);
