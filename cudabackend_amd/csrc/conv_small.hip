@@ -30,17 +30,20 @@ namespace
 		int pixels, images;
 	};
 
-	template<typename TE, typename Epi>
-	__global__ __launch_bounds__(64) void k_conv_small(const TE *__restrict__ x, const TE *__restrict__ w, SmallGeom g, Epi epi)
+	/* KW wavefronts share one tile: each takes a contiguous KW-th of the k range and the partial tiles are summed through LDS.
+	 * KW = 4 when even the 32 x 32 tiling leaves most SIMDs without a wavefront. */
+	template<typename TE, typename Epi, int KW>
+	__global__ __launch_bounds__(64 * KW) void k_conv_small(const TE *__restrict__ x, const TE *__restrict__ w, SmallGeom g, Epi epi)
 	{
-		__shared__ __attribute__((aligned(16))) typename Epi::scalar_t sm[SMALL_TILE * SMALL_PITCH];
+		__shared__ __attribute__((aligned(16))) typename Epi::scalar_t sm[KW * SMALL_TILE * SMALL_PITCH];
 		constexpr unsigned int SZ = sizeof(TE);
-		const int lane = threadIdx.x;
+		const int lane = threadIdx.x & 63;
+		const int wave = threadIdx.x >> 6;
 		const int r = lane & 31;
 		const unsigned int half = (lane >> 5) * 16;
 		/* neighbouring pixel tiles read overlapping windows: a contiguous run of them goes to one XCD and its L2 */
 		const int p0 = static_cast<int>(xcd_block(blockIdx.x, gridDim.x)) * SMALL_TILE, k0 = blockIdx.y * SMALL_TILE;
-		const int kcol = k0 + (lane & 7) * 4;
+		const int kcol = k0 + (threadIdx.x & 7) * 4;
 		typename Epi::Columns columns;
 		epi.load_columns(kcol, columns);
 
@@ -83,8 +86,13 @@ namespace
 			acc[v] = 0;
 
 		/* k walks (tap, slab); everything about the position is wavefront-uniform */
-		int f_tap = 0, f_i = 0, f_j = 0, f_slab = 0;
 		const int taps = g.R * g.S;
+		const int groups_all = (taps * g.slabs_per_tap + GROUP - 1) / GROUP;
+		const int groups = (groups_all + KW - 1) / KW; /* groups of this wavefront: [wave * groups, (wave + 1) * groups) */
+		const int first_slab = wave * groups * GROUP;
+		int f_tap = first_slab / g.slabs_per_tap, f_slab = first_slab - f_tap * g.slabs_per_tap;
+		int f_i = f_tap / g.S, f_j = f_tap - f_i * g.S;
+		int left = groups * GROUP; /* slabs this wavefront may still fetch */
 		auto fetch = [&](uint4 (&a)[GROUP], uint4 (&b)[GROUP]) __attribute__((always_inline))
 		{
 #pragma unroll
@@ -92,7 +100,8 @@ namespace
 			{
 				const int i = g.flip ? g.R - 1 - f_i : f_i, j = g.flip ? g.S - 1 - f_j : f_j;
 				const unsigned int cb = static_cast<unsigned int>(f_slab) * 32u;
-				const bool live = (f_tap < taps) & (cb + half < c_bytes);
+				const bool live = (left > 0) & (f_tap < taps) & (cb + half < c_bytes);
+				left--;
 				const unsigned int a_tap = static_cast<unsigned int>((i * g.dil_h) * g.W + j * g.dil_w) * c_bytes + cb;
 				const unsigned int b_tap = static_cast<unsigned int>(f_tap) * c_bytes + cb;
 				a[q] = buffer_fetch(rx, (live && ((inside >> (f_tap & 31)) & 1u)) ? a_origin + a_tap : OUT_OF_RANGE);
@@ -120,7 +129,6 @@ namespace
 				Mma<TE>::run(ca, cb, acc);
 			}
 		};
-		const int groups = (taps * g.slabs_per_tap + GROUP - 1) / GROUP;
 		uint4 a0[GROUP], b0[GROUP], a1[GROUP], b1[GROUP];
 		fetch(a0, b0);
 		for (int s = 0; s < groups; s += 2)
@@ -131,18 +139,29 @@ namespace
 			multiply(a1, b1);
 		}
 
-		/* lane holds column r, rows 8 i + 4 (lane / 32) + j; after the transpose: 4 consecutive columns of a row */
+		/* lane holds column r, rows 8 i + 4 (lane / 32) + j of its wavefront's partial tile; after the transpose through LDS a
+		 * work-item owns 4 consecutive columns of a row and adds up the KW partial tiles */
+		typename Epi::scalar_t *mine = sm + wave * (SMALL_TILE * SMALL_PITCH);
 #pragma unroll
 		for (int i = 0; i < 4; i++)
 #pragma unroll
 			for (int j = 0; j < 4; j++)
-				sm[(8 * i + 4 * (lane >> 5) + j) * SMALL_PITCH + r] = acc[4 * i + j];
+				mine[(8 * i + 4 * (lane >> 5) + j) * SMALL_PITCH + r] = acc[4 * i + j];
 		__syncthreads();
 #pragma unroll
-		for (int it = 0; it < 4; it++)
+		for (int it = 0; it < 4 / KW; it++)
 		{
-			const int row = (lane >> 3) + 8 * it;
-			const Pack<typename Epi::scalar_t, 4> v = *reinterpret_cast<const Pack<typename Epi::scalar_t, 4>*>(sm + row * SMALL_PITCH + (lane & 7) * 4);
+			const int row = (static_cast<int>(threadIdx.x) >> 3) + 8 * KW * it;
+			typedef Pack<typename Epi::scalar_t, 4> P4;
+			P4 v = *reinterpret_cast<const P4*>(sm + row * SMALL_PITCH + (threadIdx.x & 7) * 4);
+#pragma unroll
+			for (int part = 1; part < KW; part++)
+			{
+				const P4 o = *reinterpret_cast<const P4*>(sm + part * (SMALL_TILE * SMALL_PITCH) + row * SMALL_PITCH + (threadIdx.x & 7) * 4);
+#pragma unroll
+				for (int q = 0; q < 4; q++)
+					v.v[q] += o.v[q];
+			}
 			if (p0 + row < g.pixels && kcol < g.K)
 				epi.template store<ACT_SIMPLE, true>(p0 + row, kcol, v.v, columns);
 		}
@@ -195,8 +214,12 @@ namespace avhip
 		g.slabs_per_tap = (s.C * static_cast<int>(sizeof(TE)) + 31) / 32;
 		g.pixels = static_cast<int>(pixels);
 		g.images = s.N;
-		hipLaunchKernelGGL((k_conv_small<TE, Epi>), dim3(static_cast<unsigned int>(tiles), static_cast<unsigned int>(filter_tiles)), dim3(64), 0, stream,
-				static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
+		const dim3 grid(static_cast<unsigned int>(tiles), static_cast<unsigned int>(filter_tiles));
+		/* fewer tiles than half the 1024 SIMDs of the chip, and enough k to share: four wavefronts per tile */
+		if (tiles * filter_tiles < 512 && static_cast<int64_t>(s.R) * s.S * g.slabs_per_tap >= 4 * GROUP)
+			hipLaunchKernelGGL((k_conv_small<TE, Epi, 4>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
+		else
+			hipLaunchKernelGGL((k_conv_small<TE, Epi, 1>), grid, dim3(64), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
 		return true;
 	}
 
