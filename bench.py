@@ -33,7 +33,7 @@ SEED = 0xA70CAD0
 # HBM bytes per launch of the body convolution kernel (read + written, average over the residual and non-residual launches of a
 # pass), from the FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/conv_tile_bf16_cfg2_hbm_traffic.md.  Counters
 # cannot be read from inside this process, so the figure is carried here; it is only reported for the dtype it was taken on.
-COUNTED_TRAFFIC_BYTES = {"bf16": 39.50e6}
+COUNTED_TRAFFIC_BYTES = {"bf16": 39.52e6}
 
 
 class Hip:
