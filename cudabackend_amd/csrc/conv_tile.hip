@@ -19,7 +19,12 @@
  * position q (halo rows are HW = TW + S - 1 pixels long), so S - 1 rows at the end of every tile row compute values that
  * nobody stores.  In exchange the A operand of tap (i, j) for row q is halo pixel q + i * HW + j: the 32 rows of an MFMA
  * tile always read 32 CONSECUTIVE halo pixels, whatever the tap, and with the 144-byte pixel pitch that is free of LDS
- * bank conflicts.  Raster order would break the run at every tile-row end and serialise most reads two-fold.
+ * bank conflicts (raster order breaks the run at every tile-row end), and no per-row division is needed for the addresses.
+ *
+ * Epilogue: the accumulators leave through LDS so that a work-item stores 16 bytes of consecutive filters of one pixel with a
+ * streaming store; a table in LDS maps GEMM rows to output pixels; the residual z of the rows a work-item will store is fetched
+ * during the last channel slice, not between the stores (where possible aliasing of y and z would serialise the loads).
+ * Workgroups are numbered so that the tiles of an image, which share halo pixels, run on one XCD.
  */
 #include "conv_tile.hpp"
 #include "mfma_core.hpp"
@@ -34,7 +39,7 @@ namespace
 	constexpr int HALO_MAX = 300; /* halo pixels that fit */
 	constexpr int HALO_BYTES = HALO_MAX * PIXEL_PITCH;
 	constexpr int FILTER_TILE = TILE_N * LDS_ROW;
-	constexpr int ROW_TABLE = HALO_BYTES + 2 * FILTER_TILE; /* offset of the table: tile row -> (y << 16 | x) inside the tile, -1 past it */
+	constexpr int ROW_TABLE = HALO_BYTES + 2 * FILTER_TILE; /* offset of the table: GEMM row -> offset of its output pixel in the image, -1 if not stored */
 	constexpr int TILE_LDS = ROW_TABLE + TILE_M * 4;
 	constexpr int HALO_FETCHES = (HALO_MAX * STEP_CHUNKS + 255) / 256; /* 16-byte chunks of the halo per work-item */
 	constexpr int FILTER_FETCHES = TILE_N * STEP_CHUNKS / 256;
