@@ -227,6 +227,14 @@ namespace
 						Mma<TE>::run(a[slab & 1][tm], bq[slab & 1][tn], acc[tm][tn]);
 				__builtin_amdgcn_s_setprio(0);
 			}
+			/* instruction order within the step: after the first slab's reads, one LDS read behind every MFMA, so that reads
+			 * of the next slab trickle out under the matrix pipeline instead of in a burst between two groups of MFMAs */
+#pragma unroll
+			for (int i = 0; i < 4 * (SLABS - 1); i++)
+			{
+				__builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* one MFMA */
+				__builtin_amdgcn_sched_group_barrier(0x100, 1, 0); /* one LDS read */
+			}
 		};
 
 #pragma unroll
