@@ -15,8 +15,9 @@
 namespace avhip
 {
 	/* How a kernel instance treats the activation.  ACT_SIMPLE instances are launched only for LINEAR and RELU and pay one
-	 * compare and one select per element; ACT_ANY instances switch over all nine functions.  The split is made on the host,
-	 * per launch: a per-element switch in one kernel would make the compiler evaluate every transcendental and select. */
+	 * v_max_f32 per element behind a wavefront-uniform branch; ACT_ANY instances switch over all nine functions.  The split is
+	 * made on the host, per launch: a per-element switch in one kernel would make the compiler evaluate every transcendental
+	 * and select. */
 	constexpr int ACT_SIMPLE = -2;
 	constexpr int ACT_ANY = -1;
 	__host__ inline bool is_simple_activation(int activation)
@@ -30,7 +31,6 @@ namespace avhip
 			return (activation == ACT_RELU && x < static_cast<CT>(0)) ? static_cast<CT>(0) : x;
 		return activation_forward<CT>(activation, x);
 	}
-
 	__device__ inline int round_saturate(float v, float lo, float hi)
 	{
 		if (!(v == v))
@@ -94,6 +94,19 @@ namespace avhip
 			if (z != nullptr)
 				r.raw = *reinterpret_cast<const Pack<TE, W>*>(z + idx); /* whole, aligned runs only (VEC callers) */
 		}
+		/* t = [max(0, .)] (alpha1 * v + bias [+ alpha2 * zv]); max(0, x) as the reference writes ReLU (src/activations.cuh:274-293) */
+		template<bool RELU, bool HAS_Z, int W>
+		__device__ __forceinline__ void combine(float (&t)[W], const float (&v)[W], const ColumnsT<W> &c, const float (&zv)[W]) const
+		{
+#pragma unroll
+			for (int q = 0; q < W; q++)
+			{
+				float r = alpha1 * v[q] + c.bias[q];
+				if (HAS_Z)
+					r += alpha2 * zv[q];
+				t[q] = RELU ? __builtin_fmaxf(r, 0.0f) : r;
+			}
+		}
 		/* idx: element index of (pixel, filter k) in y and z, for callers that keep it cheaper than p * K + k */
 		template<int ACT, bool VEC = false, int W = 4>
 		__device__ __forceinline__ void store_at(int64_t idx, int k, const float (&v)[W], const ColumnsT<W> &c, const Residual<W> *fetched = nullptr) const
@@ -102,9 +115,9 @@ namespace avhip
 			const bool vec = VEC || this->vec;
 			const int valid = VEC ? W : K - k;
 			float t[W];
-#pragma unroll
-			for (int q = 0; q < W; q++)
-				t[q] = alpha1 * v[q] + c.bias[q];
+			/* ReLU sits in the same straight-line block as the multiply-add that feeds it: the compiler then knows the
+			 * operand is an arithmetic result (never a signalling NaN) and emits one bare v_max_f32 per element */
+			const bool relu = ACT == ACT_SIMPLE && activation == ACT_RELU;
 			if (z != nullptr)
 			{
 				float zv[W];
@@ -116,13 +129,24 @@ namespace avhip
 				}
 				else
 					load_vec<TE, W, float>(z + idx, valid, zv, vec);
+				if (relu)
+					combine<true, true, W>(t, v, c, zv);
+				else
+					combine<false, true, W>(t, v, c, zv);
+			}
+			else
+			{
+				if (relu)
+					combine<true, false, W>(t, v, c, v);
+				else
+					combine<false, false, W>(t, v, c, v);
+			}
+			if (ACT != ACT_SIMPLE)
+			{
 #pragma unroll
 				for (int q = 0; q < W; q++)
-					t[q] += alpha2 * zv[q];
+					t[q] = activation_forward<float>(activation, t[q]);
 			}
-#pragma unroll
-			for (int q = 0; q < W; q++)
-				t[q] = activate<ACT, float>(activation, t[q]);
 			if (beta != 0.0f)
 			{
 				float yv[W];
