@@ -299,19 +299,21 @@ def copy_bandwidth(hip, ctx, iters=10):
 
 def mfma_rates(hip, ctx):
     """What the matrix cores sustain with register-resident operands and no memory traffic (avhip_mfma_rate_probe), per
-    dtype, in T(FL)OP/s: the clock under sustained MFMA load is below the boost clock the datasheet peak assumes."""
+    dtype, in T(FL)OP/s: with nearly all-zero operand bits (clock near boost) and with random finite operands, whose
+    switching activity lowers the clock the power management allows; the datasheet peak assumes the boost clock."""
     lib = cb.load_library()
     lib.avhip_mfma_rate_probe.restype = C.c_int
-    lib.avhip_mfma_rate_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    lib.avhip_mfma_rate_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
     workgroups, iterations = 256 * 8, 4096
     sink = cb.DeviceTensor((workgroups * 256,), cb.DTYPE_FLOAT32)
-    out = {}
-    for name, k, per_call in (("bf16", 16, 1), ("f16", 16, 1), ("i8", 32, 1), ("f32", 2, 4)):
-        def call():
-            assert lib.avhip_mfma_rate_probe(ctx.stream(), DT[name], workgroups, iterations, sink.pointer()) == 0
-        ms = time_calls(hip, ctx, call, 4, warmup=1)
-        ops = workgroups * 4.0 * iterations * 8 * per_call * 2 * 32 * 32 * k
-        out[name] = ops / (ms * 1e-3) / 1e12
+    out = {"quiet_operands": {}, "random_operands": {}}
+    for operands, key in ((0, "quiet_operands"), (1, "random_operands")):
+        for name, k, per_call in (("bf16", 16, 1), ("f16", 16, 1), ("i8", 32, 1), ("f32", 2, 4)):
+            def call():
+                assert lib.avhip_mfma_rate_probe(ctx.stream(), DT[name], workgroups, iterations, operands, sink.pointer()) == 0
+            ms = time_calls(hip, ctx, call, 4, warmup=1)
+            ops = workgroups * 4.0 * iterations * 8 * per_call * 2 * 32 * 32 * k
+            out[key][name] = ops / (ms * 1e-3) / 1e12
     sink.close()
     return out
 
@@ -435,6 +437,11 @@ def main():
         "cpu_baseline": cpu,
         "detail": detail,
     }
+    rates = detail.get("mfma_rate_measured")
+    if rates is not None:
+        # the same fraction against what the matrix cores of THIS box sustain on random operands with nothing else running
+        key = {"bf16": "bf16", "f16": "f16", "f32": "f32"}[args.dtype]
+        line["roofline"]["frac_of_measured_mfma_rate"] = head["body_conv_tflops"] / rates["random_operands"][key]
     print(json.dumps(line))
 
 

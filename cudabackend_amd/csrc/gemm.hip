@@ -231,8 +231,24 @@ namespace
 namespace
 {
 	/* Eight independent accumulators per wavefront: enough MFMAs in flight to cover the pipeline depth without any memory
-	 * access in the loop.  The operands are arbitrary register contents derived from the lane number. */
-	template<typename TE>
+	 * access in the loop.  QUIET operands are almost all zero bits (the matrix cores toggle little and the clock stays near
+	 * boost); otherwise every MFMA reads one of four A and two B register sets filled with hashed bits shaped into finite
+	 * numbers of magnitude 0.5 .. 2, which is what the clock under a real workload's switching activity looks like. */
+	template<typename TE> __device__ inline unsigned finite_bits(unsigned r);
+	template<> __device__ inline unsigned finite_bits<f16_t>(unsigned r) { return (r & 0x83ff83ffu) | 0x38003800u; }
+	template<> __device__ inline unsigned finite_bits<bf16_t>(unsigned r) { return (r & 0x80ff80ffu) | 0x3f003f00u; }
+	template<> __device__ inline unsigned finite_bits<int8_t>(unsigned r) { return r; }
+	template<> __device__ inline unsigned finite_bits<float>(unsigned r) { return (r & 0x80ffffffu) | 0x3f000000u; }
+	__device__ inline unsigned hash_bits(unsigned v)
+	{
+		v ^= v >> 16;
+		v *= 0x7feb352du;
+		v ^= v >> 15;
+		v *= 0x846ca68bu;
+		v ^= v >> 16;
+		return v;
+	}
+	template<typename TE, bool QUIET>
 	__global__ __launch_bounds__(256) void k_mfma_rate_probe(int iterations, typename Mma<TE>::scalar_t *sink)
 	{
 		typename Mma<TE>::acc_t acc[8];
@@ -241,14 +257,36 @@ namespace
 #pragma unroll
 			for (int v = 0; v < 16; v++)
 				acc[i][v] = 0;
-		Chunk a, b;
-		a.u = make_uint4(threadIdx.x, 0u, 0u, 0u);
-		b.u = make_uint4(0u, threadIdx.x & 1u, 0u, 0u);
+		Chunk a[4], b[2];
+#pragma unroll
+		for (int i = 0; i < 4; i++)
+		{
+			if (QUIET)
+				a[i].u = make_uint4(threadIdx.x, 0u, 0u, 0u);
+			else
+			{
+				const unsigned seed = (blockIdx.x * 256u + threadIdx.x) * 32u + i * 4u;
+				a[i].u = make_uint4(finite_bits<TE>(hash_bits(seed)), finite_bits<TE>(hash_bits(seed + 1)), finite_bits<TE>(hash_bits(seed + 2)),
+						finite_bits<TE>(hash_bits(seed + 3)));
+			}
+		}
+#pragma unroll
+		for (int i = 0; i < 2; i++)
+		{
+			if (QUIET)
+				b[i].u = make_uint4(0u, threadIdx.x & 1u, 0u, 0u);
+			else
+			{
+				const unsigned seed = (blockIdx.x * 256u + threadIdx.x) * 32u + 16u + i * 4u;
+				b[i].u = make_uint4(finite_bits<TE>(hash_bits(seed)), finite_bits<TE>(hash_bits(seed + 1)), finite_bits<TE>(hash_bits(seed + 2)),
+						finite_bits<TE>(hash_bits(seed + 3)));
+			}
+		}
 		for (int it = 0; it < iterations; it++)
 		{
 #pragma unroll
 			for (int i = 0; i < 8; i++)
-				Mma<TE>::run(a, b, acc[i]);
+				Mma<TE>::run(a[i & 3], b[i >> 2], acc[i]);
 		}
 		typename Mma<TE>::scalar_t total = 0;
 #pragma unroll
@@ -258,27 +296,36 @@ namespace
 				total += acc[i][v];
 		sink[static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x] = total;
 	}
+	template<typename TE>
+	void launch_rate_probe(hipStream_t st, int workgroups, int iterations, int operands, void *sink)
+	{
+		typedef typename Mma<TE>::scalar_t scalar_t;
+		if (operands == 0)
+			hipLaunchKernelGGL((k_mfma_rate_probe<TE, true>), dim3(workgroups), dim3(256), 0, st, iterations, static_cast<scalar_t*>(sink));
+		else
+			hipLaunchKernelGGL((k_mfma_rate_probe<TE, false>), dim3(workgroups), dim3(256), 0, st, iterations, static_cast<scalar_t*>(sink));
+	}
 }
 
-extern "C" int avhip_mfma_rate_probe(void *stream, int dtype, int workgroups, int iterations, void *sink)
+extern "C" int avhip_mfma_rate_probe(void *stream, int dtype, int workgroups, int iterations, int operands, void *sink)
 {
-	if (workgroups <= 0 || iterations <= 0 || sink == nullptr)
+	if (workgroups <= 0 || iterations <= 0 || sink == nullptr || operands < 0 || operands > 1)
 		return AVHIP_BAD_PARAM;
 	hipStream_t st = static_cast<hipStream_t>(stream);
 	switch (dtype)
 	{
 		case DT_FLOAT16:
-			hipLaunchKernelGGL((k_mfma_rate_probe<f16_t>), dim3(workgroups), dim3(256), 0, st, iterations, static_cast<float*>(sink));
+			launch_rate_probe<f16_t>(st, workgroups, iterations, operands, sink);
 			return 0;
 		case DT_BFLOAT16:
-			hipLaunchKernelGGL((k_mfma_rate_probe<bf16_t>), dim3(workgroups), dim3(256), 0, st, iterations, static_cast<float*>(sink));
+			launch_rate_probe<bf16_t>(st, workgroups, iterations, operands, sink);
 			return 0;
 		case DT_INT8:
-			hipLaunchKernelGGL((k_mfma_rate_probe<int8_t>), dim3(workgroups), dim3(256), 0, st, iterations, static_cast<int*>(sink));
+			launch_rate_probe<int8_t>(st, workgroups, iterations, operands, sink);
 			return 0;
 		case DT_FLOAT32:
 			/* Mma<float>::run issues four 32x32x2 MFMAs per call */
-			hipLaunchKernelGGL((k_mfma_rate_probe<float>), dim3(workgroups), dim3(256), 0, st, iterations, static_cast<float*>(sink));
+			launch_rate_probe<float>(st, workgroups, iterations, operands, sink);
 			return 0;
 		default:
 			return AVHIP_UNSUPPORTED_DATATYPE;

@@ -116,11 +116,13 @@ extern "C"
 
 	/* Measurement aid without a counterpart in the reference: keeps every matrix core busy with register-resident
 	 * 32x32 MFMAs of `dtype` (FLOAT16, BFLOAT16, INT8 or FLOAT32) and nothing else, so that a harness can time the rate the
-	 * matrix cores sustain on this machine (clock under load included) next to the datasheet peak.  Launches `workgroups`
-	 * workgroups of 256 work-items, each wavefront issuing iterations * 8 MFMAs; sink receives one value per work-item
-	 * (workgroups * 256 * 4 bytes).  Operations performed = workgroups * 4 * iterations * 8 * 2*32*32*k, k = 16 / 32 / 2 for
-	 * 16-bit / int8 / fp32. */
-	AVHIP_API int avhip_mfma_rate_probe(void *stream, int dtype, int workgroups, int iterations, void *sink);
+	 * matrix cores sustain on this machine (clock under load included) next to the datasheet peak.  operands = 0: nearly
+	 * all-zero operand bits (least switching activity, clock near boost); operands = 1: hashed bits shaped into finite
+	 * numbers, several register sets in rotation (the switching activity, and so the clock, of real data).  Launches
+	 * `workgroups` workgroups of 256 work-items, each wavefront issuing iterations * 8 MFMAs; sink receives one value per
+	 * work-item (workgroups * 256 * 4 bytes).  Operations performed = workgroups * 4 * iterations * 8 * 2*32*32*k,
+	 * k = 16 / 32 / 2 for 16-bit / int8 / fp32. */
+	AVHIP_API int avhip_mfma_rate_probe(void *stream, int dtype, int workgroups, int iterations, int operands, void *sink);
 
 #ifdef __cplusplus
 }
