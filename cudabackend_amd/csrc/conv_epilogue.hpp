@@ -250,12 +250,15 @@ namespace avhip
 			if (MODE == I8_EXACT || MODE == I8_REQUANT)
 			{
 				int t[W];
+				/* one v_max_i32 against a scalar either way (hidden from the optimiser, which would otherwise turn it back
+				 * into a maximum and a select per element) */
+				int floor = activation == ACT_RELU ? 0 : -2147483647 - 1;
+				keep_in_sgpr(floor);
 #pragma unroll
 				for (int q = 0; q < W; q++)
 				{
 					t[q] = v[q] + c.ibias[q];
-					if (activation == ACT_RELU && t[q] < 0)
-						t[q] = 0;
+					t[q] = t[q] < floor ? floor : t[q];
 				}
 				/* whole runs leave as streaming vector stores: the kernel never reads y back, so the caches may drain it while
 				 * the kernel runs */
@@ -283,14 +286,31 @@ namespace avhip
 				}
 				else
 				{
+					/* Clamping to the integers -128 and 127 commutes with rounding to an integer, so the product is clamped
+					 * first; adding 1.5 * 2^23 then rounds it to nearest even in the adder (the sum's unit in the last place is 1)
+					 * and leaves the two's-complement byte in the low 8 bits of the sum: no rint, no conversion.  Three byte
+					 * permutes gather four such bytes into a word. */
 					union
 					{
 						int8_t b[W];
+						unsigned int u[W / 4];
 						words_t w;
 					} o;
 #pragma unroll
-					for (int q = 0; q < W; q++)
-						o.b[q] = static_cast<int8_t>(static_cast<int>(__builtin_amdgcn_fmed3f(rintf(static_cast<float>(t[q]) * c.scale[q]), -128.0f, 127.0f)));
+					for (int part = 0; part < W / 4; part++)
+					{
+						unsigned int bits[4];
+#pragma unroll
+						for (int q = 0; q < 4; q++)
+						{
+							const float product = static_cast<float>(t[4 * part + q]) * c.scale[4 * part + q];
+							const float rounded = __builtin_amdgcn_fmed3f(product, -128.0f, 127.0f) + 12582912.0f;
+							bits[q] = __builtin_bit_cast(unsigned int, rounded);
+						}
+						const unsigned int lo = __builtin_amdgcn_perm(bits[1], bits[0], 0x0c0c0400u);
+						const unsigned int hi = __builtin_amdgcn_perm(bits[3], bits[2], 0x0c0c0400u);
+						o.u[part] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+					}
 					int8_t *dst = static_cast<int8_t*>(y) + idx;
 					if (vec && valid >= W)
 						__builtin_nontemporal_store(o.w, reinterpret_cast<words_t*>(dst));
