@@ -73,6 +73,8 @@ PROTOTYPES = {
     "cudaWinogradWeightTransform": (i32, [i64, i64, i32, i64, i64, i64, i64]),
     "cudaWinogradInputTransform": (i32, [i64, i64, i32, i64, i64, i64, i64, i64]),
     "cudaWinogradOutputTransform": (i32, [i64, i64, i32, i64, vp, i64, i64, i64, i64, i64, i64, vp, i64, i64, vp, i32]),
+    "cudaWinogradGradientTransform": (i32, [i64, i64, i32, i64, i64, i64, i64, i64]),
+    "cudaWinogradUpdateTransform": (i32, [i64, i64, i32, vp, i64, i64, vp, i64, i64]),
     "cudaGetConvolutionWorkspaceSize": (i32, [i64, i64, i64, i64, i64, C.POINTER(i64)]),
     "cudaConvolutionBiasActivationForward": (i32, [i64, i64, vp, i64, i64, i64, i64, i64, i64, vp, i64, i64, vp, i64, i64, i32, i64]),
     "cudaConvolutionForward": (i32, [i64, i64, vp, i64, i64, i64, i64, vp, i64, i64, i64]),
@@ -82,7 +84,8 @@ PROTOTYPES = {
     "avhipInvalidateCaches": (i32, []),
 }
 # the thin kernel layer of include/avocado_hip_kernels.h (exported, bound only for the symbol check)
-KERNEL_LAYER_SYMBOLS = ["avhip_winograd_weight_transform", "avhip_winograd_input_transform", "avhip_winograd_output_transform", "avhip_gemm_batched",
+KERNEL_LAYER_SYMBOLS = ["avhip_winograd_weight_transform", "avhip_winograd_input_transform", "avhip_winograd_output_transform",
+                        "avhip_winograd_gradient_transform", "avhip_winograd_update_transform", "avhip_gemm_batched",
                         "avhip_conv2d_implicit_gemm", "avhip_conv2d_winograd_fused", "avhip_add_bias", "avhip_im2row", "avhip_change_type",
                         "avhip_set_memory", "avhip_mfma_rate_probe", "avhip_set_small_problem_threshold",
                         "avhip_affine_forward", "avhip_batchnorm_inference"]

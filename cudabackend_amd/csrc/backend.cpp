@@ -1462,6 +1462,71 @@ namespace avocado
 					y->dim[2], y->dim[3], scalar_or(alpha1, y->dtype, 1.0), scalar_or(alpha2, y->dtype, 1.0), scalar_or(beta, y->dtype, 0.0), activation));
 		}
 
+		avStatus_t cudaWinogradGradientTransform(avContextDescriptor_t context, const avConvolutionDescriptor_t config, int transformSize,
+				const avTensorDescriptor_t wDesc, const avTensorDescriptor_t dyDesc, const avMemoryDescriptor_t dyMem, const avTensorDescriptor_t matricesDesc,
+				avMemoryDescriptor_t matricesMem)
+		{
+			Context ctx;
+			if (!get_context(context, ctx))
+				return AVOCADO_STATUS_BAD_PARAM;
+			const Tensor *w = get_tensor(wDesc), *dy = get_tensor(dyDesc), *mx = get_tensor(matricesDesc);
+			if (get_convolution(config) == nullptr || w == nullptr || dy == nullptr || mx == nullptr)
+				return AVOCADO_STATUS_BAD_PARAM;
+			if (!is_floating(dy->dtype))
+				return AVOCADO_STATUS_UNSUPPORTED_DATATYPE;
+			if (w->nb_dims != 4 || dy->nb_dims != 4 || mx->nb_dims != 3)
+				return AVOCADO_STATUS_NOT_SUPPORTED;
+			const int r = w->dim[1];
+			if (!is_conv(r, *w) || !winograd_supported(r, transformSize))
+				return AVOCADO_STATUS_NOT_SUPPORTED;
+			if (!matrix_dtype_ok(dy->dtype, mx->dtype))
+				return AVOCADO_STATUS_UNSUPPORTED_DATATYPE;
+			const int m = transformSize, t = m + r - 1;
+			const av_int64 tiles = static_cast<av_int64>(dy->dim[0]) * ((dy->dim[1] + m - 1) / m) * ((dy->dim[2] + m - 1) / m);
+			if (mx->dim[0] != t * t || mx->dim[1] != tiles || mx->dim[2] != dy->dim[3])
+				return AVOCADO_STATUS_BAD_PARAM;
+			Memory *dm = get_memory(dyMem), *mm = get_memory(matricesMem);
+			if (!fits(dm, dy->volume() * size_of(dy->dtype)) || !fits(mm, mx->volume() * size_of(mx->dtype)))
+				return AVOCADO_STATUS_BAD_PARAM;
+			if (hipSetDevice(ctx.device) != hipSuccess)
+				return AVOCADO_STATUS_EXECUTION_FAILED;
+			touch(matricesMem);
+			return from_launcher(avhip_winograd_gradient_transform(ctx.stream, dy->dtype, mx->dtype, m, r, dm->data, mm->data, dy->dim[0], dy->dim[1],
+					dy->dim[2], dy->dim[3]));
+		}
+
+		avStatus_t cudaWinogradUpdateTransform(avContextDescriptor_t context, const avConvolutionDescriptor_t config, int transformSize, const void *alpha,
+				const avTensorDescriptor_t matricesDesc, const avMemoryDescriptor_t matricesMem, const void *beta, const avTensorDescriptor_t dwDesc,
+				avMemoryDescriptor_t dwMem)
+		{
+			Context ctx;
+			if (!get_context(context, ctx))
+				return AVOCADO_STATUS_BAD_PARAM;
+			const Tensor *dw = get_tensor(dwDesc), *mx = get_tensor(matricesDesc);
+			if (get_convolution(config) == nullptr || dw == nullptr || mx == nullptr)
+				return AVOCADO_STATUS_BAD_PARAM;
+			if (!is_floating(dw->dtype))
+				return AVOCADO_STATUS_UNSUPPORTED_DATATYPE;
+			if (dw->nb_dims != 4 || mx->nb_dims != 3)
+				return AVOCADO_STATUS_NOT_SUPPORTED;
+			const int r = dw->dim[1];
+			if (!is_conv(r, *dw) || !winograd_supported(r, transformSize))
+				return AVOCADO_STATUS_NOT_SUPPORTED;
+			if (!matrix_dtype_ok(dw->dtype, mx->dtype))
+				return AVOCADO_STATUS_UNSUPPORTED_DATATYPE;
+			const int t = transformSize + r - 1;
+			if (mx->dim[0] != t * t || mx->dim[1] != dw->dim[0] || mx->dim[2] != dw->dim[3])
+				return AVOCADO_STATUS_BAD_PARAM;
+			Memory *wm = get_memory(dwMem), *mm = get_memory(matricesMem);
+			if (!fits(wm, dw->volume() * size_of(dw->dtype)) || !fits(mm, mx->volume() * size_of(mx->dtype)))
+				return AVOCADO_STATUS_BAD_PARAM;
+			if (hipSetDevice(ctx.device) != hipSuccess)
+				return AVOCADO_STATUS_EXECUTION_FAILED;
+			touch(dwMem);
+			return from_launcher(avhip_winograd_update_transform(ctx.stream, dw->dtype, mx->dtype, transformSize, r, mm->data, wm->data, dw->dim[0],
+					dw->dim[3], scalar_or(alpha, dw->dtype, 1.0), scalar_or(beta, dw->dtype, 0.0)));
+		}
+
 		avStatus_t cudaGetConvolutionWorkspaceSize(avContextDescriptor_t context, const avConvolutionDescriptor_t config, const avTensorDescriptor_t xDesc,
 				const avTensorDescriptor_t wDesc, const avTensorDescriptor_t bDesc, av_int64 *result)
 		{

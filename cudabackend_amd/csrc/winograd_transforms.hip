@@ -1,8 +1,9 @@
 /*
- * winograd_transforms.hip -- the three non-fused Winograd transforms for F(2x2,3x3), F(4x4,3x3) and F(2x2,5x5).
+ * winograd_transforms.hip -- the non-fused Winograd transforms for F(2x2,3x3), F(4x4,3x3) and F(2x2,5x5): weight, input and
+ * output for the forward pass, gradient and update for the weight gradient.
  *
- * Replaces kernel_winograd_{weight,input,output}_transform and their launchers of the reference
- * (src/winograd_nonfused.cu:257-423, 609-777).  The mathematics is the same sandwich product M * tile * M^T with the
+ * Replaces kernel_winograd_{weight,input,output,gradient,update}_transform and their launchers of the reference
+ * (src/winograd_nonfused.cu:257-519, 609-877).  The mathematics is the same sandwich product M * tile * M^T with the
  * same coefficient tables (src/winograd_nonfused.cu:534-575); the mapping to the machine is not:
  *
  *  - these kernels are HBM-bound, so one work-item owns one tile x one 16-byte (or 8-byte) vector of channels, issues
@@ -22,7 +23,8 @@ namespace
 {
 	using namespace avhip;
 
-	/* Coefficient tables (row-major).  which: 0 = G [t x r], 1 = B^T [t x t], 2 = A^T [m x t]. */
+	/* Coefficient tables (row-major).  which: 0 = G [t x r], 1 = B^T [t x t], 2 = A^T [m x t], 3 = gradient [t x m],
+	 * 4 = update [r x t]. */
 	template<int M, int R> struct Tab;
 	template<> struct Tab<2, 3>
 	{
@@ -31,7 +33,9 @@ namespace
 			constexpr double G[4 * 3] = { 1, 0, 0, 1, 1, 1, 1, -1, 1, 0, 0, 1 };
 			constexpr double BT[4 * 4] = { 1, 0, -1, 0, 0, 1, 1, 0, 0, -1, 1, 0, 0, -1, 0, 1 };
 			constexpr double AT[2 * 4] = { 1, 0.5, 0.5, 0, 0, 0.5, -0.5, 1 };
-			return which == 0 ? G[i * 3 + j] : which == 1 ? BT[i * 4 + j] : AT[i * 4 + j];
+			constexpr double GR[4 * 2] = { 1, 0, 1, 1, 1, -1, 0, 1 };
+			constexpr double UP[3 * 4] = { 1, 0.5, 0.5, 0, 0, 0.5, -0.5, 0, 0, 0.5, 0.5, 1 };
+			return which == 0 ? G[i * 3 + j] : which == 1 ? BT[i * 4 + j] : which == 2 ? AT[i * 4 + j] : which == 3 ? GR[i * 2 + j] : UP[i * 4 + j];
 		}
 	};
 	template<> struct Tab<4, 3>
@@ -43,7 +47,10 @@ namespace
 			constexpr double BT[6 * 6] = { 1, 0, -1.25, 0, 0.25, 0, 0, 1, 1, -0.25, -0.25, 0, 0, -1, 1, 0.25, -0.25, 0, 0, -1, -0.5, 1, 0.5, 0, 0, 1, -0.5,
 					-1, 0.5, 0, 0, 1, 0, -1.25, 0, 0.25 };
 			constexpr double AT[4 * 6] = { 1, 1, 1, 0.25, 0.25, 0, 0, 1, -1, 0.5, -0.5, 0, 0, 1, 1, 1, 1, 0, 0, 1, -1, 2, -2, 2 };
-			return which == 0 ? G[i * 3 + j] : which == 1 ? BT[i * 6 + j] : AT[i * 6 + j];
+			constexpr double GR[6 * 4] = { 1, 0, 0, 0, 2 * a, 2 * a, 2 * a, 2 * a, 2 * a, -2 * a, 2 * a, -2 * a, a, 2 * a, 4 * a, 8 * a, a, -2 * a, 4 * a, -8 * a, 0,
+					0, 0, 2 };
+			constexpr double UP[3 * 6] = { 1, 1, 1, 0.25, 0.25, 0, 0, 1, -1, 0.5, -0.5, 0, 0, 1, 1, 1, 1, 2 };
+			return which == 0 ? G[i * 3 + j] : which == 1 ? BT[i * 6 + j] : which == 2 ? AT[i * 6 + j] : which == 3 ? GR[i * 4 + j] : UP[i * 6 + j];
 		}
 	};
 	template<> struct Tab<2, 5>
@@ -56,7 +63,9 @@ namespace
 			constexpr double BT[6 * 6] = { 1, 0, -1.25, 0, 0.25, 0, 0, 1, 1, -0.25, -0.25, 0, 0, -1, 1, 0.25, -0.25, 0, 0, -1, -0.5, 1, 0.5, 0, 0, 1, -0.5,
 					-1, 0.5, 0, 0, 1, 0, -1.25, 0, 0.25 };
 			constexpr double AT[2 * 6] = { 1, 1, 1, 0.5, 0.5, 0, 0, 1, -1, 1, -1, 2 };
-			return which == 0 ? G[i * 5 + j] : which == 1 ? BT[i * 6 + j] : AT[i * 6 + j];
+			constexpr double GR[6 * 2] = { 1, 0, 2 * a, 2 * a, 2 * a, -2 * a, a, 2 * a, a, -2 * a, 0, 1 };
+			constexpr double UP[5 * 6] = { 1, 1, 1, 0.25, 0.25, 0, 0, 1, -1, 0.5, -0.5, 0, 0, 1, 1, 1, 1, 0, 0, 1, -1, 2, -2, 0, 0, 1, 1, 4, 4, 4 };
+			return which == 0 ? G[i * 5 + j] : which == 1 ? BT[i * 6 + j] : which == 2 ? AT[i * 6 + j] : which == 3 ? GR[i * 2 + j] : UP[i * 6 + j];
 		}
 	};
 
@@ -296,6 +305,97 @@ namespace
 			}
 	}
 
+	/* Weight-gradient side, first transform: one M x M tile of dy (tiles do not overlap, positions past the border are zero)
+	 * becomes G' dy G'^T, a t x t tile of the matrices [t*t, tiles, K] (src/winograd_nonfused.cu:425-474). */
+	template<int M, int R, typename T, typename TM, int V>
+	__global__ __launch_bounds__(256) void k_gradient_transform(const T *__restrict__ dy, TM *__restrict__ Mx, int N, int H, int W, int K, int Th, int Tw)
+	{
+		typedef typename Traits<T>::compute CT;
+		constexpr int t = M + R - 1;
+		const size_t KV = static_cast<size_t>((K + V - 1) / V);
+		const size_t tiles = static_cast<size_t>(N) * Th * Tw;
+		const size_t gid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+		const size_t tile = gid / KV;
+		if (tile >= tiles)
+			return;
+		const int k = static_cast<int>(gid - tile * KV) * V;
+		const int valid = K - k;
+		const size_t row = tile / Tw;
+		const int tw = static_cast<int>(tile - row * Tw);
+		const size_t n = row / Th;
+		const int th = static_cast<int>(row - n * Th);
+
+		CT d[M * M][V];
+#pragma unroll
+		for (int a = 0; a < M; a++)
+#pragma unroll
+			for (int b = 0; b < M; b++)
+			{
+				const int h = th * M + a, w = tw * M + b;
+				if (h < H && w < W)
+					load_vec<T, V, CT>(dy + ((n * H + h) * W + w) * K + k, valid, d[a * M + b]);
+				else
+				{
+#pragma unroll
+					for (int v = 0; v < V; v++)
+						d[a * M + b][v] = static_cast<CT>(0);
+				}
+			}
+		CT out[t * t][V];
+		sandwich<M, R, 3, t, M, CT, V>(d, out);
+#pragma unroll
+		for (int i = 0; i < t * t; i++)
+		{
+			typename Traits<TM>::compute o[V];
+#pragma unroll
+			for (int v = 0; v < V; v++)
+				o[v] = static_cast<typename Traits<TM>::compute>(out[i][v]);
+			store_vec<TM, V>(Mx + (static_cast<size_t>(i) * tiles + tile) * K + k, valid, o);
+		}
+	}
+
+	/* Weight-gradient side, last transform: dw[k, :, :, c] = alpha * U' m U'^T + beta * dw, m = the t x t tile of the matrices
+	 * [t*t, K, C] at (k, c) (src/winograd_nonfused.cu:475-519). */
+	template<int M, int R, typename T, typename TM, int V>
+	__global__ __launch_bounds__(256) void k_update_transform(const TM *__restrict__ Mx, T *dw, int K, int C, typename Traits<T>::compute alpha,
+			typename Traits<T>::compute beta)
+	{
+		typedef typename Traits<T>::compute CT;
+		constexpr int t = M + R - 1;
+		const int CV = (C + V - 1) / V;
+		const size_t gid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+		const int c = static_cast<int>(gid % CV) * V;
+		const size_t k = gid / CV;
+		if (k >= static_cast<size_t>(K))
+			return;
+		const int valid = C - c;
+
+		CT m[t * t][V];
+#pragma unroll
+		for (int i = 0; i < t * t; i++)
+			load_vec<TM, V, CT>(Mx + (static_cast<size_t>(i) * K + k) * C + c, valid, m[i]);
+		CT out[R * R][V];
+		sandwich<M, R, 4, R, t, CT, V>(m, out);
+#pragma unroll
+		for (int i = 0; i < R * R; i++)
+		{
+			T *dst = dw + (k * R * R + i) * C + c;
+			CT o[V];
+#pragma unroll
+			for (int v = 0; v < V; v++)
+				o[v] = alpha * out[i][v];
+			if (beta != static_cast<CT>(0))
+			{
+				CT old[V];
+				load_vec<T, V, CT>(dst, valid, old);
+#pragma unroll
+				for (int v = 0; v < V; v++)
+					o[v] += beta * old[v];
+			}
+			store_vec<T, V>(dst, valid, o);
+		}
+	}
+
 	/* Channels per work-item: as many as 16 bytes of the wider of the two types hold, but never so many that the t x t tile
 	 * (t*t values per channel, twice during the products) pushes the kernel to one or two wavefronts per SIMD: these kernels
 	 * live on many loads and stores in flight from many wavefronts. */
@@ -394,6 +494,37 @@ namespace
 		return 0;
 	}
 
+	template<int M, int R, typename T, typename TM>
+	int launch_gradient(hipStream_t s, const void *dy, void *Mx, int N, int H, int W, int K)
+	{
+		const int Th = (H + M - 1) / M, Tw = (W + M - 1) / M;
+		const int V = pick_vec<M, R, T, TM>(K, dy, Mx);
+		const size_t items = static_cast<size_t>(N) * Th * Tw * ((K + V - 1) / V);
+		const dim3 grid(ceil_div(items, 256));
+		if (V > 1)
+			hipLaunchKernelGGL((k_gradient_transform<M, R, T, TM, VecOf<M, R, T, TM>::value>), grid, dim3(256), 0, s, static_cast<const T*>(dy),
+					static_cast<TM*>(Mx), N, H, W, K, Th, Tw);
+		else
+			hipLaunchKernelGGL((k_gradient_transform<M, R, T, TM, 1>), grid, dim3(256), 0, s, static_cast<const T*>(dy), static_cast<TM*>(Mx), N, H, W, K, Th,
+					Tw);
+		return 0;
+	}
+	template<int M, int R, typename T, typename TM>
+	int launch_update(hipStream_t s, const void *Mx, void *dw, int K, int C, double alpha, double beta)
+	{
+		typedef typename Traits<T>::compute CT;
+		const int V = pick_vec<M, R, T, TM>(C, Mx, dw);
+		const size_t items = static_cast<size_t>(K) * ((C + V - 1) / V);
+		const dim3 grid(ceil_div(items, 256));
+		if (V > 1)
+			hipLaunchKernelGGL((k_update_transform<M, R, T, TM, VecOf<M, R, T, TM>::value>), grid, dim3(256), 0, s, static_cast<const TM*>(Mx),
+					static_cast<T*>(dw), K, C, static_cast<CT>(alpha), static_cast<CT>(beta));
+		else
+			hipLaunchKernelGGL((k_update_transform<M, R, T, TM, 1>), grid, dim3(256), 0, s, static_cast<const TM*>(Mx), static_cast<T*>(dw), K, C,
+					static_cast<CT>(alpha), static_cast<CT>(beta));
+		return 0;
+	}
+
 	/* Supported (tensor dtype, matrix dtype) pairs: equal types (the reference's behaviour), and fp16 or fp32 matrices
 	 * for 16-bit tensors.  CALL is instantiated with <T, TM>. */
 #define AVHIP_DISPATCH_PAIR(dtype, mat_dtype, CALL)                                              \
@@ -455,6 +586,27 @@ extern "C"
 			return AVHIP_BAD_PARAM;
 		hipStream_t s = static_cast<hipStream_t>(stream);
 #define CALL(T, TM) AVHIP_DISPATCH_MR(m, r, launch_output, T, TM, s, M, y, bias, z, N, H, W, K, alpha1, alpha2, beta, activation)
+		AVHIP_DISPATCH_PAIR(dtype, mat_dtype, CALL)
+#undef CALL
+	}
+
+	int avhip_winograd_gradient_transform(void *stream, int dtype, int mat_dtype, int m, int r, const void *dy, void *M, int N, int H, int W, int K)
+	{
+		if (dy == nullptr || M == nullptr || N <= 0 || H <= 0 || W <= 0 || K <= 0)
+			return AVHIP_BAD_PARAM;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+#define CALL(T, TM) AVHIP_DISPATCH_MR(m, r, launch_gradient, T, TM, s, dy, M, N, H, W, K)
+		AVHIP_DISPATCH_PAIR(dtype, mat_dtype, CALL)
+#undef CALL
+	}
+
+	int avhip_winograd_update_transform(void *stream, int dtype, int mat_dtype, int m, int r, const void *M, void *dw, int K, int C, double alpha,
+			double beta)
+	{
+		if (M == nullptr || dw == nullptr || K <= 0 || C <= 0)
+			return AVHIP_BAD_PARAM;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+#define CALL(T, TM) AVHIP_DISPATCH_MR(m, r, launch_update, T, TM, s, M, dw, K, C, alpha, beta)
 		AVHIP_DISPATCH_PAIR(dtype, mat_dtype, CALL)
 #undef CALL
 	}

@@ -176,6 +176,16 @@ namespace avocado
 					const avTensorDescriptor_t yDesc, avMemoryDescriptor_t yMem, const avTensorDescriptor_t bDesc, const avMemoryDescriptor_t bMem,
 					const void *alpha2, const avTensorDescriptor_t zDesc, const avMemoryDescriptor_t zMem, const void *beta, avActivationType_t activation);
 
+			/* cuda_backend.h:911.  Weight-gradient side: matrices[t*t, tiles, K] = G' dy-tile G'^T over non-overlapping
+			 * transformSize x transformSize tiles of dy (src/winograd_nonfused.cu:963). */
+			DLL_PUBLIC avStatus_t cudaWinogradGradientTransform(avContextDescriptor_t context, const avConvolutionDescriptor_t config, int transformSize,
+					const avTensorDescriptor_t wDesc, const avTensorDescriptor_t dyDesc, const avMemoryDescriptor_t dyMem,
+					const avTensorDescriptor_t matricesDesc, avMemoryDescriptor_t matricesMem);
+			/* cuda_backend.h:927.  dw[K, r, r, C] = alpha * U' matrices[t*t, K, C] U'^T + beta * dw (src/winograd_nonfused.cu:983). */
+			DLL_PUBLIC avStatus_t cudaWinogradUpdateTransform(avContextDescriptor_t context, const avConvolutionDescriptor_t config, int transformSize,
+					const void *alpha, const avTensorDescriptor_t matricesDesc, const avMemoryDescriptor_t matricesMem, const void *beta,
+					const avTensorDescriptor_t dwDesc, avMemoryDescriptor_t dwMem);
+
 			/* Not in the reference header; NOT_SUPPORTED stubs at src/convolution.cu:30-99 of the reference.  Here they are the
 			 * dispatcher a front-end calls per layer: it picks fused Winograd, non-fused Winograd (needs the workspace) or
 			 * implicit GEMM from shape and dtype.  The workspace may be an invalid descriptor when the size query returned 0. */

@@ -60,6 +60,16 @@ extern "C"
 	AVHIP_API int avhip_winograd_output_transform(void *stream, int dtype, int mat_dtype, int m, int r, const void *M, void *y, const void *bias, const void *z,
 			int N, int H, int W, int K, double alpha1, double alpha2, double beta, int activation);
 
+	/* M = G' dy G'^T over non-overlapping m x m tiles of dy [N, H, W, K] (zeros past the border), M [t*t, tiles, K].
+	 * Replaces launch_gradient_transform / kernel_winograd_gradient_transform, src/winograd_nonfused.cu:780,425. */
+	AVHIP_API int avhip_winograd_gradient_transform(void *stream, int dtype, int mat_dtype, int m, int r, const void *dy, void *M, int N, int H, int W,
+			int K);
+
+	/* dw [K, r, r, C] = alpha * U' M U'^T + beta * dw, M [t*t, K, C].  Replaces launch_update_transform /
+	 * kernel_winograd_update_transform, src/winograd_nonfused.cu:828,475. */
+	AVHIP_API int avhip_winograd_update_transform(void *stream, int dtype, int mat_dtype, int m, int r, const void *M, void *dw, int K, int C, double alpha,
+			double beta);
+
 	/* C[b] = alpha * op(A[b]) op(B[b]) + beta * C[b], row-major.  Replaces the cuBLAS calls of cudaGemm and
 	 * cudaGemmBatched, src/gemm.cpp:25-124,126-209.  ab_dtype: FLOAT16 / BFLOAT16 / FLOAT32 / FLOAT64 / INT8;
 	 * c_dtype: same as ab_dtype, FLOAT32 for 16-bit inputs, INT32 for INT8.  Strides are in elements. */

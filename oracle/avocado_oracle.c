@@ -20,6 +20,10 @@
  *                             reference has no requantisation step: parity unpinned.
  *   orc_winograd_*_transform  pinned: A^T[(G g G^T) .* (B^T d B)]A == direct correlation to 1e-12
  *                             for every (m, r) table, partial tiles and offsets included.
+ *   orc_winograd_gradient_transform, orc_winograd_update_transform
+ *                             pinned: U'[(G' dy G'^T) .* (B^T d B)]U'^T == the r x r correlation of the input tile d
+ *                             with the m x m tile dy to 1e-12 for every (m, r); a whole weight gradient assembled from
+ *                             them equals torch's fp64 autograd weight gradient of conv2d.
  *   orc_gemm_batched          pinned: numpy matmul / einsum on all four (N|T, N|T) combinations.
  *                             (The reference delegates to cuBLAS, whose source is not part of it.)
  *   orc_add_bias              pinned: numpy restatement of the documented formula in two algebraic
@@ -36,6 +40,7 @@
  *   include/Avocado/cuda_backend.h:796,822,877  y = act(alpha1*conv + alpha2*z + b) + beta*y
  *   src/winograd_nonfused.cu:220-254         M * tile * M^T algebra of first/second transform
  *   src/winograd_nonfused.cu:303-423         tiling, padding, clipping, epilogue order
+ *   src/winograd_nonfused.cu:425-519         gradient and update transforms of the weight gradient
  *   src/winograd_nonfused.cu:534-575         transform coefficient tables
  *   src/activations.cuh:30-121               NHWC offsets, tile index, [t*t, tiles, C] matrices
  *   src/activations.cuh:202-456              activation functions
@@ -266,6 +271,38 @@ static const double G_2_5[6 * 5] = { 1, 0, 0, 0, 0, 2 * T3, 2 * T3, 2 * T3, 2 * 
 		4 * T3, 8 * T3, T3 / 2, -T3, 2 * T3, -4 * T3, 8 * T3, 0, 0, 0, 0, 2 };
 static const double AT_2_5[2 * 6] = { 1, 1, 1, 0.5, 0.5, 0, 0, 1, -1, 1, -1, 2 };
 
+/* Weight-gradient side (src/winograd_nonfused.cu:538-539,558-562,571-574): gradient G' [t x m], update U' [r x t]. */
+static const double GR_2_3[4 * 2] = { 1, 0, 1, 1, 1, -1, 0, 1 };
+static const double UP_2_3[3 * 4] = { 1, 0.5, 0.5, 0, 0, 0.5, -0.5, 0, 0, 0.5, 0.5, 1 };
+static const double GR_4_3[6 * 4] = { 1, 0, 0, 0, 2 * T3, 2 * T3, 2 * T3, 2 * T3, 2 * T3, -2 * T3, 2 * T3, -2 * T3, T3, 2 * T3, 4 * T3, 8 * T3, T3, -2 * T3,
+	4 * T3, -8 * T3, 0, 0, 0, 2 };
+static const double UP_4_3[3 * 6] = { 1, 1, 1, 0.25, 0.25, 0, 0, 1, -1, 0.5, -0.5, 0, 0, 1, 1, 1, 1, 2 };
+static const double GR_2_5[6 * 2] = { 1, 0, 2 * T3, 2 * T3, 2 * T3, -2 * T3, T3, 2 * T3, T3, -2 * T3, 0, 1 };
+static const double UP_2_5[5 * 6] = { 1, 1, 1, 0.25, 0.25, 0, 0, 1, -1, 0.5, -0.5, 0, 0, 1, 1, 1, 1, 0, 0, 1, -1, 2, -2, 0, 0, 1, 1, 4, 4, 4 };
+
+static int get_training_tables(int m, int r, const double **GR, const double **UP)
+{
+	if (m == 2 && r == 3)
+	{
+		*GR = GR_2_3;
+		*UP = UP_2_3;
+		return 0;
+	}
+	if (m == 4 && r == 3)
+	{
+		*GR = GR_4_3;
+		*UP = UP_4_3;
+		return 0;
+	}
+	if (m == 2 && r == 5)
+	{
+		*GR = GR_2_5;
+		*UP = UP_2_5;
+		return 0;
+	}
+	return -1;
+}
+
 /* Returns 0 when (m, r) is one of the three supported pairs, src/winograd_nonfused.cu:626-650. */
 static int get_tables(int m, int r, const double **G, const double **BT, const double **AT)
 {
@@ -293,15 +330,15 @@ static int get_tables(int m, int r, const double **G, const double **BT, const d
 	return -1;
 }
 
-/* Copies a table out (which: 0 = G, 1 = B^T, 2 = A^T); returns the number of coefficients or -1. */
+/* Copies a table out (which: 0 = G, 1 = B^T, 2 = A^T, 3 = gradient, 4 = update); returns the number of coefficients or -1. */
 int orc_winograd_table(int m, int r, int which, double *out)
 {
-	const double *G, *BT, *AT;
-	if (get_tables(m, r, &G, &BT, &AT) != 0)
+	const double *G, *BT, *AT, *GR, *UP;
+	if (get_tables(m, r, &G, &BT, &AT) != 0 || get_training_tables(m, r, &GR, &UP) != 0 || which < 0 || which > 4)
 		return -1;
 	const int t = m + r - 1;
-	const double *src = which == 0 ? G : which == 1 ? BT : AT;
-	const int n = which == 0 ? t * r : which == 1 ? t * t : m * t;
+	const double *src = which == 0 ? G : which == 1 ? BT : which == 2 ? AT : which == 3 ? GR : UP;
+	const int n = which == 0 ? t * r : which == 1 ? t * t : which == 2 ? m * t : which == 3 ? t * m : r * t;
 	memcpy(out, src, sizeof(double) * n);
 	return n;
 }
@@ -446,6 +483,67 @@ int orc_winograd_output_transform(const double *Mx, double *y, const double *bia
 							y[idx] = v;
 						}
 				}
+	return 0;
+}
+
+/*
+ * Mx[(i*t+j), tile, k] = (G' d G'^T)[i,j], d[a,b] = dy[n, th*m + a, tw*m + b, k] or 0 past the border; tiles do not overlap,
+ * tile = (n*Th + th)*Tw + tw (src/winograd_nonfused.cu:425-474).  dy is [N, H, W, K], Mx is [t*t, tiles, K].
+ */
+int orc_winograd_gradient_transform(const double *dy, double *Mx, int N, int H, int W, int K, int m, int r)
+{
+	const double *GR, *UP;
+	if (get_training_tables(m, r, &GR, &UP) != 0)
+		return -1;
+	const int t = m + r - 1;
+	const int Th = (H + m - 1) / m, Tw = (W + m - 1) / m;
+	const size_t tiles = (size_t) N * Th * Tw;
+	for (int n = 0; n < N; n++)
+		for (int th = 0; th < Th; th++)
+			for (int tw = 0; tw < Tw; tw++)
+				for (int k = 0; k < K; k++)
+				{
+					double d[8 * 8], out[8 * 8];
+					for (int a = 0; a < m; a++)
+						for (int b = 0; b < m; b++)
+						{
+							const int h = th * m + a, w = tw * m + b;
+							d[a * m + b] = (h < H && w < W) ? dy[(((size_t) n * H + h) * W + w) * K + k] : 0.0;
+						}
+					sandwich(GR, t, m, d, out);
+					const size_t tile = ((size_t) n * Th + th) * Tw + tw;
+					for (int i = 0; i < t * t; i++)
+						Mx[((size_t) i * tiles + tile) * K + k] = out[i];
+				}
+	return 0;
+}
+
+/*
+ * dw[k, i, j, c] = alpha * (U' d U'^T)[i,j] + beta * dw_old, d = the t x t tile Mx[:, k, c]
+ * (src/winograd_nonfused.cu:475-519).  Mx is [t*t, K, C], dw is [K, r, r, C].
+ */
+int orc_winograd_update_transform(const double *Mx, double *dw, int K, int C, int m, int r, double alpha, double beta)
+{
+	const double *GR, *UP;
+	if (get_training_tables(m, r, &GR, &UP) != 0)
+		return -1;
+	const int t = m + r - 1;
+	for (int k = 0; k < K; k++)
+		for (int c = 0; c < C; c++)
+		{
+			double d[8 * 8], out[8 * 8];
+			for (int i = 0; i < t * t; i++)
+				d[i] = Mx[((size_t) i * K + k) * C + c];
+			sandwich(UP, r, t, d, out);
+			for (int i = 0; i < r * r; i++)
+			{
+				const size_t idx = ((size_t) k * r * r + i) * C + c;
+				double v = alpha * out[i];
+				if (beta != 0.0)
+					v += beta * dw[idx];
+				dw[idx] = v;
+			}
+		}
 	return 0;
 }
 

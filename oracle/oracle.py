@@ -157,7 +157,7 @@ def conv2d_i8_float_epilogue(acc, bias, z, y, alpha1, alpha2, beta, activation):
 
 def winograd_table(m, r, which):
     t = m + r - 1
-    shape = {0: (t, r), 1: (t, t), 2: (m, t)}[which]
+    shape = {0: (t, r), 1: (t, t), 2: (m, t), 3: (t, m), 4: (r, t)}[which]
     out = np.zeros(shape, dtype=np.float64)
     n = lib().orc_winograd_table(m, r, which, _p(out))
     if n != out.size:
@@ -194,6 +194,28 @@ def winograd_output_transform(M, shape, m, r, bias=None, z=None, y=None, alpha1=
                                            C.c_double(beta), activation) != 0:
         raise ValueError("unsupported transform")
     return y
+
+
+def winograd_gradient_transform(dy, m, r):
+    dy = _f64(dy)
+    N, H, W, K = dy.shape
+    t = m + r - 1
+    tiles = N * ((H + m - 1) // m) * ((W + m - 1) // m)
+    M = np.zeros((t * t, tiles, K), dtype=np.float64)
+    if lib().orc_winograd_gradient_transform(_p(dy), _p(M), N, H, W, K, m, r) != 0:
+        raise ValueError("unsupported transform")
+    return M
+
+
+def winograd_update_transform(M, m, r, dw=None, alpha=1.0, beta=0.0):
+    M = _f64(M)
+    t = m + r - 1
+    assert M.shape[0] == t * t
+    _, K, Cin = M.shape
+    dw = np.zeros((K, r, r, Cin), dtype=np.float64) if dw is None else np.array(dw, dtype=np.float64).reshape(K, r, r, Cin)
+    if lib().orc_winograd_update_transform(_p(M), _p(dw), K, Cin, m, r, C.c_double(alpha), C.c_double(beta)) != 0:
+        raise ValueError("unsupported transform")
+    return dw
 
 
 def gemm_batched(A, B, Cm=None, opA=False, opB=False, alpha=1.0, beta=0.0):

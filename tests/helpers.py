@@ -118,6 +118,36 @@ def winograd_output_transform(M, yshape, wshape, dtype, m, bias=None, z=None, y0
         return y.download() if st == cb.STATUS_SUCCESS else None
 
 
+def winograd_gradient_transform(dy, wshape, dtype, m, mat_dtype=None, expect=cb.STATUS_SUCCESS):
+    mat_dtype = mat_dtype or dtype
+    N, H, W, K = dy.shape
+    r = wshape[1]
+    t = m + r - 1
+    tiles = N * ((H + m - 1) // m) * ((W + m - 1) // m)
+    with Call() as c:
+        conv = cb.ConvolutionDescriptor()
+        dyt = c.tensor(dy, dtype)
+        wt = c.empty(wshape, dtype)
+        M = c.empty((t * t, tiles, K), mat_dtype)
+        st = c.lib.cudaWinogradGradientTransform(c.ctx.handle, conv.handle, m, wt.desc, dyt.desc, dyt.mem, M.desc, M.mem)
+        assert st == expect, cb.STATUS_NAMES[st]
+        c.finish()
+        return M.download() if st == cb.STATUS_SUCCESS else None
+
+
+def winograd_update_transform(M, wshape, dtype, m, dw0=None, alpha=None, beta=None, mat_dtype=None, expect=cb.STATUS_SUCCESS):
+    mat_dtype = mat_dtype or dtype
+    with Call() as c:
+        conv = cb.ConvolutionDescriptor()
+        Mt = c.tensor(M, mat_dtype)
+        dw = c.tensor(dw0, dtype) if dw0 is not None else c.empty(wshape, dtype)
+        d = DT[dtype]
+        st = c.lib.cudaWinogradUpdateTransform(c.ctx.handle, conv.handle, m, cb.scalar(alpha, d), Mt.desc, Mt.mem, cb.scalar(beta, d), dw.desc, dw.mem)
+        assert st == expect, cb.STATUS_NAMES[st]
+        c.finish()
+        return dw.download() if st == cb.STATUS_SUCCESS else None
+
+
 def gemm(A, B, C0, dtype, opA=False, opB=False, alpha=None, beta=None, c_dtype=None, batched=False, expect=cb.STATUS_SUCCESS):
     c_dtype = c_dtype or dtype
     with Call() as c:

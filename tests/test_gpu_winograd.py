@@ -1,4 +1,5 @@
-"""GPU parity of the three non-fused Winograd transforms and of the whole non-fused pipeline, through the C API,
+"""GPU parity of the non-fused Winograd transforms (forward: weight, input, output; weight gradient: gradient, update) and of
+the whole non-fused pipelines, through the C API,
 against the CPU oracle on identical seeded inputs.  Shapes follow the reference's own tests
 (test/test_winograd.cpp:28,32-38,174: x {12,13,14,135}, w {21,3,3,135} / {21,5,5,135}, alpha1 1.1, alpha2 1.2, beta 0.1,
 all four bias / residual combinations) plus channel counts that take the vectorised code path."""
@@ -76,6 +77,70 @@ def test_output_transform_vector_path_and_activations(oracle):
         got = h.winograd_output_transform(M * 0.2, (N, H, W, K), (K, 3, 3, 8), "f32", 4, bias, activation=act)
         want = oracle.winograd_output_transform(M * 0.2, (N, H, W, K), 4, 3, bias, activation=act)
         assert oracle.rel_l2(got, want) < 5e-6, act
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32", "f64"])
+@pytest.mark.parametrize("m,r", CASES)
+@pytest.mark.parametrize("shape", [(12, 13, 14, 21), (3, 15, 15, 64)])
+def test_gradient_transform(oracle, dtype, m, r, shape):
+    """reference shapes test/test_winograd.cpp:101 (dy {12,13,14,21}) plus a vector-path channel count"""
+    g = h.rng(7)
+    dy = h.rounded(oracle, g.standard_normal(shape), dtype)
+    got = h.winograd_gradient_transform(dy, (shape[3], r, r, 8), dtype, m)
+    want = oracle.winograd_gradient_transform(dy, m, r)
+    assert got.shape == want.shape
+    assert oracle.rel_l2(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32", "f64"])
+@pytest.mark.parametrize("m,r", CASES)
+@pytest.mark.parametrize("C", [135, 64])
+def test_update_transform(oracle, dtype, m, r, C):
+    g = h.rng(8)
+    K, t = 21, m + r - 1
+    M = h.rounded(oracle, g.standard_normal((t * t, K, C)), dtype)
+    got = h.winograd_update_transform(M, (K, r, r, C), dtype, m)
+    want = oracle.winograd_update_transform(M, m, r)
+    assert oracle.rel_l2(got, want) < TOL[dtype]
+    dw0 = h.rounded(oracle, g.standard_normal((K, r, r, C)), dtype)
+    a, b = (1.1, 0.1) if dtype == "f64" else (float(np.float32(1.1)), float(np.float32(0.1)))
+    got = h.winograd_update_transform(M, (K, r, r, C), dtype, m, dw0, a, b)
+    want = oracle.winograd_update_transform(M, m, r, dw0, a, b)
+    assert oracle.rel_l2(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("m,r", CASES)
+def test_weight_gradient_pipeline_matches_direct_correlation(oracle, m, r):
+    """dw through the Winograd domain (input transform of x, gradient transform of dy, batched GEMM (T, N) over the tiles,
+    update transform) against the direct sum dw[k,i,j,c] = sum dy[n,h,w,k] * x[n,h+i-p,w+j-p,c] in fp64, fp32 tensors."""
+    import cudabackend_amd as cb
+    g = h.rng(9)
+    N, H, W, Cin, K = 4, 15, 15, 32, 24
+    x = h.rounded(oracle, g.standard_normal((N, H, W, Cin)), "f32")
+    dy = h.rounded(oracle, g.standard_normal((N, H, W, K)), "f32")
+    t, p = m + r - 1, r // 2
+    tiles = N * ((H + m - 1) // m) * ((W + m - 1) // m)
+    with h.Call() as c:
+        conv = cb.ConvolutionDescriptor(padding=(-p, -p))
+        xt, dyt = c.tensor(x, "f32"), c.tensor(dy, "f32")
+        wt = c.empty((K, r, r, Cin), "f32")
+        V, Mg, dU = c.empty((t * t, tiles, Cin), "f32"), c.empty((t * t, tiles, K), "f32"), c.empty((t * t, K, Cin), "f32")
+        dw = c.empty((K, r, r, Cin), "f32")
+        lib, ctx = c.lib, c.ctx.handle
+        cb.check(lib.cudaWinogradInputTransform(ctx, conv.handle, m, wt.desc, xt.desc, xt.mem, V.desc, V.mem), "input")
+        cb.check(lib.cudaWinogradGradientTransform(ctx, conv.handle, m, wt.desc, dyt.desc, dyt.mem, Mg.desc, Mg.mem), "gradient")
+        cb.check(lib.cudaGemmBatched(ctx, cb.GEMM_OPERATION_T, cb.GEMM_OPERATION_N, None, Mg.desc, Mg.mem, V.desc, V.mem, None, dU.desc, dU.mem), "gemm")
+        cb.check(lib.cudaWinogradUpdateTransform(ctx, conv.handle, m, None, dU.desc, dU.mem, None, dw.desc, dw.mem), "update")
+        c.finish()
+        got = dw.download()
+    xp = np.pad(x, ((0, 0), (p, p), (p, p), (0, 0)))
+    want = np.zeros((K, r, r, Cin))
+    for i in range(r):
+        for j in range(r):
+            want[:, i, j, :] = np.einsum("nhwk,nhwc->kc", dy, xp[:, i:i + H, j:j + W, :])
+    err = oracle.rel_l2(got, want)
+    print("weight gradient F(%d,%d) rel-L2 = %.3e" % (m, r, err))
+    assert err < 1e-4  # the fp32 Winograd bar
 
 
 def test_unsupported_combinations_return_status(oracle):

@@ -210,6 +210,59 @@ def test_winograd_layouts(oracle):
     np.testing.assert_allclose(Ui[:, 2, 1].reshape(4, 4), G @ w[2, ::-1, ::-1, 1] @ G.T, atol=1e-13)
 
 
+@pytest.mark.parametrize("m,r", [(2, 3), (4, 3), (2, 5)])
+def test_winograd_training_tables_reproduce_weight_gradient(oracle, m, r):
+    """U'[(G' dy G'^T) .* (B^T d B)]U'^T equals the r x r correlation of a t x t input patch with an m x m tile of dy."""
+    BT, GR, UP = (oracle.winograd_table(m, r, i) for i in (1, 3, 4))
+    t = m + r - 1
+    assert GR.shape == (t, m) and UP.shape == (r, t)
+    d = RNG.standard_normal((t, t))
+    dy = RNG.standard_normal((m, m))
+    dw = UP @ ((GR @ dy @ GR.T) * (BT @ d @ BT.T)) @ UP.T
+    want = np.array([[np.sum(d[i:i + m, j:j + m] * dy) for j in range(r)] for i in range(r)])
+    np.testing.assert_allclose(dw, want, atol=1e-12)
+
+
+@pytest.mark.parametrize("m,r", [(2, 3), (4, 3), (2, 5)])
+def test_winograd_weight_gradient_pipeline_matches_torch(oracle, m, r):
+    """input transform (x) and gradient transform (dy) -> batched GEMM (T, N) -> update transform == the weight gradient
+    torch's fp64 autograd gives for conv2d, on odd sizes (partial tiles); alpha and beta of the update transform applied."""
+    N, H, W, Cin, K = 2, 7, 9, 3, 4
+    x = RNG.standard_normal((N, H, W, Cin))
+    dy = RNG.standard_normal((N, H, W, K))
+    xt = torch.tensor(x.transpose(0, 3, 1, 2).copy(), dtype=torch.float64)
+    wt = torch.zeros((K, Cin, r, r), dtype=torch.float64, requires_grad=True)
+    y = torch.nn.functional.conv2d(xt, wt, padding=r // 2)
+    y.backward(torch.tensor(dy.transpose(0, 3, 1, 2).copy(), dtype=torch.float64))
+    want = wt.grad.numpy().transpose(0, 2, 3, 1)  # [K, r, r, C]
+    V = oracle.winograd_input_transform(x, m, r, (-(r // 2), -(r // 2)))
+    Mg = oracle.winograd_gradient_transform(dy, m, r)
+    dU = oracle.gemm_batched(Mg, V, opA=True, opB=False)
+    got = oracle.winograd_update_transform(dU, m, r)
+    np.testing.assert_allclose(got, want, atol=1e-10)
+    dw0 = RNG.standard_normal((K, r, r, Cin))
+    got = oracle.winograd_update_transform(dU, m, r, dw=dw0, alpha=0.5, beta=-2.0)
+    np.testing.assert_allclose(got, 0.5 * want - 2.0 * dw0, atol=1e-10)
+
+
+def test_winograd_training_layouts(oracle):
+    """gradient transform: non-overlapping tiles, zeros past the border, [t*t, tiles, K]; update transform: [t*t, K, C] -> [K, r, r, C]."""
+    m, r = 2, 3
+    dy = RNG.standard_normal((2, 3, 5, 2))
+    Mg = oracle.winograd_gradient_transform(dy, m, r)
+    GR, UP = oracle.winograd_table(m, r, 3), oracle.winograd_table(m, r, 4)
+    Th, Tw = 2, 3
+    assert Mg.shape == (16, 2 * Th * Tw, 2)
+    n, th, tw, k = 1, 1, 2, 1
+    d = np.zeros((2, 2))
+    d[0, 0] = dy[n, 2, 4, k]  # rows 2..3, columns 4..5 of a 3 x 5 map: only (2, 4) exists
+    np.testing.assert_allclose(Mg[:, (n * Th + th) * Tw + tw, k].reshape(4, 4), GR @ d @ GR.T, atol=1e-13)
+    Mx = RNG.standard_normal((16, 3, 2))
+    dw = oracle.winograd_update_transform(Mx, m, r)
+    assert dw.shape == (3, 3, 3, 2)
+    np.testing.assert_allclose(dw[2, :, :, 1], UP @ Mx[:, 2, 1].reshape(4, 4) @ UP.T, atol=1e-13)
+
+
 @pytest.mark.parametrize("opA", [False, True])
 @pytest.mark.parametrize("opB", [False, True])
 def test_gemm_batched_matches_numpy(oracle, opA, opB):
