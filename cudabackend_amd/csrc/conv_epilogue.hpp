@@ -76,6 +76,15 @@ namespace avhip
 			for (int q = 0; q < W; q++)
 				c.bias[q] = (bias != nullptr && k + q < K) ? bias[k + q] : 0.0f;
 		}
+		/* the same constants out of a table of one-filter records (a kernel that walks several filter blocks stages
+		 * load_columns(k, table[k]) for every k in LDS once) */
+		template<int W>
+		__device__ static __forceinline__ void pick_columns(const ColumnsT<1> *table, int k, ColumnsT<W> &c)
+		{
+#pragma unroll
+			for (int q = 0; q < W; q++)
+				c.bias[q] = table[k + q].bias[0];
+		}
 		/* p: index of the output pixel (row of y), k: first of the W filters.  VEC instances require whole, aligned vectors. */
 		template<int ACT, bool VEC = false>
 		__device__ __forceinline__ void store(int64_t p, int k, const float (&v)[4], const Columns &c) const
@@ -224,6 +233,17 @@ namespace avhip
 				sc = (sc == sc) ? sc : 0.0f;
 				sc = sc > 3.0e38f ? 3.0e38f : (sc < -3.0e38f ? -3.0e38f : sc);
 				c.scale[q] = sc;
+			}
+		}
+		template<int W>
+		__device__ static __forceinline__ void pick_columns(const ColumnsT<1> *table, int k, ColumnsT<W> &c)
+		{
+#pragma unroll
+			for (int q = 0; q < W; q++)
+			{
+				c.ibias[q] = table[k + q].ibias[0];
+				c.fbias[q] = table[k + q].fbias[0];
+				c.scale[q] = table[k + q].scale[0];
 			}
 		}
 		template<int ACT, bool VEC = false>

@@ -20,6 +20,7 @@
 #include <cstring>
 
 #include "conv_epilogue.hpp"
+#include "conv_pointwise.hpp"
 #include "conv_small.hpp"
 #include "conv_tile.hpp"
 #include "mfma_core.hpp"
@@ -546,6 +547,9 @@ namespace
 		}
 		/* a problem of a few big tiles goes to the kernel with one 32 x 32 tile per wavefront */
 		if (fast && conv_small_launch<TE, Epi>(st, s, x, w, epi, static_cast<int64_t>(grid.x) * grid.y))
+			return 0;
+		/* one-tap filters are plain matrix products with a short k: a persistent kernel pipelines across tiles */
+		if (fast && s.R * s.S == 1 && conv_pointwise_launch<TE, Epi>(st, s, x, w, epi))
 			return 0;
 		/* stride-1 filters with more than one tap first try the kernel that keeps an image tile resident in LDS */
 		if (fast && s.R * s.S > 1 && conv_tile_launch<TE, Epi>(st, s, x, w, epi))
