@@ -9,7 +9,10 @@
  * Unlike the reference there is a bf16 case, fp16 always accumulates in fp32, and the result of a 16-bit product may be
  * kept in fp32.
  */
+#include <type_traits>
+
 #include "mfma_core.hpp"
+#include "persistent_gemm.hpp"
 
 namespace
 {
@@ -140,6 +143,55 @@ namespace
 		});
 	}
 
+	/* C = alpha * acc + beta * C as the epilogue of the persistent short-k product (floating types). */
+	template<typename TC>
+	struct GemmEpilogue
+	{
+		typedef float scalar_t;
+		static constexpr int wide = sizeof(TC) >= 4 ? 4 : 8; /* one 16-byte store */
+		template<int W> struct ColumnsT
+		{
+		};
+		TC *c;
+		float alpha, beta;
+		__device__ __forceinline__ void pin()
+		{
+			keep_in_sgpr(alpha);
+			keep_in_sgpr(beta);
+		}
+		__device__ __forceinline__ void load_columns(int, ColumnsT<1>&) const
+		{
+		}
+		template<int W>
+		__device__ static __forceinline__ void pick_columns(const ColumnsT<1>*, int, ColumnsT<W>&)
+		{
+		}
+		template<int ACT, bool VEC, int W>
+		__device__ __forceinline__ void store_at(int64_t idx, int, const float (&v)[W], const ColumnsT<W>&) const
+		{
+			float t[W];
+#pragma unroll
+			for (int q = 0; q < W; q++)
+				t[q] = alpha * v[q];
+			if (beta != 0.0f)
+			{
+				float old[W];
+				load_vec<TC, W, float>(c + idx, W, old, true);
+#pragma unroll
+				for (int q = 0; q < W; q++)
+					t[q] += beta * old[q];
+			}
+			store_vec<TC, W, float, true>(c + idx, W, t, true); /* streaming: C is not read back by this kernel */
+		}
+	};
+
+	template<typename TE, typename TC, int STEPS>
+	__global__ __launch_bounds__(256, 2) void k_gemm_nt_persistent(const TE *__restrict__ A, const TE *__restrict__ B, PersistentGeom g, GemmEpilogue<TC> epi)
+	{
+		__shared__ __attribute__((aligned(16))) char lds[PERSISTENT_LDS_BYTES];
+		persistent_nt_gemm<TE, GemmEpilogue<TC>, STEPS>(lds, A, B, g, epi);
+	}
+
 	/* Any operand form, any supported type: 16 x 16 outputs per workgroup, k in slices of 16 through LDS. */
 	template<typename TA, typename TC, typename CT>
 	__global__ __launch_bounds__(256) void k_gemm_generic(const TA *__restrict__ A, const TA *__restrict__ B, TC *C, int M, int N, int K, int opA, int opB,
@@ -196,6 +248,57 @@ namespace
 	};
 
 	template<typename TE, typename TC>
+	bool launch_persistent(hipStream_t s, const void *A, const void *B, void *C, int batch, int M, int N, int K, int lda, int ldb, int ldc, int64_t sA,
+			int64_t sB, int64_t sC, double alpha, double beta, bool fast)
+	{
+		if constexpr (std::is_same<typename Mma<TE>::scalar_t, float>::value)
+		{
+			typedef GemmEpilogue<TC> Epi;
+			const int64_t row_bytes = static_cast<int64_t>(K) * sizeof(TE);
+			const int steps = static_cast<int>((row_bytes + STEP_BYTES - 1) / STEP_BYTES);
+			/* fp32 products are bound by the matrix cores (sixteen-pass MFMAs): for the Winograd shapes measured (1152 tiles
+			 * on 512 resident workgroups) the one-tile kernel, whose workgroups the hardware hands out as slots free up, beats
+			 * a static split of 2.25 rounds of tiles into 2 and 3 (61 against 65 us) */
+			if (!fast || steps > PERSISTENT_MAX_STEPS || sizeof(TE) >= 4)
+				return false;
+			/* whole 16-byte runs of C, rows of C a multiple of them apart */
+			if (N % Epi::wide != 0 || ldc % Epi::wide != 0 || sC % Epi::wide != 0 || !aligned_to(C, 16) || ldc >= (1 << 24))
+				return false;
+			const int64_t a_bytes = ((batch - 1) * sA + static_cast<int64_t>(M - 1) * lda + K) * static_cast<int64_t>(sizeof(TE));
+			const int64_t b_bytes = ((batch - 1) * sB + static_cast<int64_t>(N - 1) * ldb + K) * static_cast<int64_t>(sizeof(TE));
+			const int64_t row_blocks = ceil_div(M, BLOCK_M), col_blocks = ceil_div(N, BLOCK_N);
+			const int64_t tiles = row_blocks * col_blocks * batch;
+			if (sA < 0 || sB < 0 || a_bytes >= (1ll << 31) || b_bytes >= (1ll << 31) || tiles >= (1ll << 31) - 1024)
+				return false;
+			PersistentGeom g;
+			g.rows = M;
+			g.cols = N;
+			g.row_bytes = static_cast<unsigned int>(row_bytes);
+			g.a_pitch = static_cast<unsigned int>(lda * sizeof(TE));
+			g.b_pitch = static_cast<unsigned int>(ldb * sizeof(TE));
+			g.a_batch = static_cast<unsigned int>(sA * sizeof(TE));
+			g.b_batch = static_cast<unsigned int>(sB * sizeof(TE));
+			g.a_bytes = static_cast<unsigned int>(a_bytes);
+			g.b_bytes = static_cast<unsigned int>(b_bytes);
+			g.c_batch = sC;
+			g.c_pitch = ldc;
+			g.row_blocks = static_cast<int>(row_blocks);
+			g.col_blocks = static_cast<int>(col_blocks);
+			g.tiles = static_cast<int>(tiles);
+			g.table_columns = 0;
+			const Epi epi { static_cast<TC*>(C), static_cast<float>(alpha), static_cast<float>(beta) };
+			const dim3 grid(persistent_workgroups(tiles));
+			if (steps <= 2)
+				hipLaunchKernelGGL((k_gemm_nt_persistent<TE, TC, 2>), grid, dim3(256), 0, s, static_cast<const TE*>(A), static_cast<const TE*>(B), g, epi);
+			else
+				hipLaunchKernelGGL((k_gemm_nt_persistent<TE, TC, 4>), grid, dim3(256), 0, s, static_cast<const TE*>(A), static_cast<const TE*>(B), g, epi);
+			return true;
+		}
+		else
+			return false;
+	}
+
+	template<typename TE, typename TC>
 	int launch_mfma(hipStream_t s, const void *A, const void *B, void *C, int batch, int M, int N, int K, int lda, int ldb, int ldc, int64_t sA, int64_t sB,
 			int64_t sC, double alpha, double beta)
 	{
@@ -208,6 +311,9 @@ namespace
 		const bool small = (static_cast<int64_t>(M) * lda + K) * static_cast<int64_t>(sizeof(TE)) < (1ll << 31)
 				&& (static_cast<int64_t>(N) * ldb + K) * static_cast<int64_t>(sizeof(TE)) < (1ll << 31);
 		const bool fast = vec_ok && small && K % (16 / static_cast<int>(sizeof(TE))) == 0;
+		/* a short k (the channel count of a Winograd layer): workgroups stay resident and pipeline across tiles */
+		if (launch_persistent<TE, TC>(s, A, B, C, batch, M, N, K, lda, ldb, ldc, sA, sB, sC, alpha, beta, fast))
+			return 0;
 #define AVHIP_GEMM_ARGS static_cast<const TE*>(A), static_cast<const TE*>(B), static_cast<TC*>(C), M, N, K, lda, ldb, ldc, sA, sB, sC, static_cast<S>(alpha), \
 		static_cast<S>(beta), flags
 		if (fast)
