@@ -332,4 +332,6 @@ def test_convolution_argument_errors(oracle):
     h.conv_forward("implicit_gemm", x, w, (2, 6, 6, 4), "f32", groups=2, expect=cb.STATUS_NOT_SUPPORTED)
     h.conv_forward("implicit_gemm", x, w, (2, 6, 6, 4), "f64", expect=cb.STATUS_UNSUPPORTED_DATATYPE)
     h.conv_forward("implicit_gemm", x, w, (2, 20, 20, 4), "f32", expect=cb.STATUS_BAD_PARAM)            # output larger than any window grid
+    # an empty batch is refused, not skipped (the reference's launch with a zero-sized grid fails as well)
+    h.conv_forward("implicit_gemm", np.zeros((0, 6, 6, 8)), w, (0, 6, 6, 4), "f32", expect=cb.STATUS_BAD_PARAM)
     h.conv_forward("winograd_fused", x, np.zeros((4, 5, 5, 8)), (2, 6, 6, 4), "f32", pad=(-2, -2), expect=cb.STATUS_NOT_SUPPORTED)
