@@ -297,6 +297,25 @@ def copy_bandwidth(hip, ctx, iters=10):
     return 2.0 * nbytes / (ms * 1e-3) / 1e9
 
 
+def stream_rates(hip, ctx, iters=10):
+    """Read-only, write-only and copy rates of streaming kernels with 16-byte accesses (avhip_stream_probe) over 1 GiB, GB/s:
+    the ceilings an HBM-bound kernel of this library can reach on this box, next to the nominal 8 TB/s."""
+    lib = cb.load_library()
+    lib.avhip_stream_probe.restype = C.c_int
+    lib.avhip_stream_probe.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int64]
+    nbytes = 1 << 30
+    a, b = cb.DeviceTensor((nbytes,), cb.DTYPE_UINT8), cb.DeviceTensor((nbytes,), cb.DTYPE_UINT8)
+    out = {}
+    for kind, name, moved in ((0, "read", 1.0), (1, "write", 1.0), (2, "copy", 2.0)):
+        def call():
+            assert lib.avhip_stream_probe(ctx.stream(), kind, a.pointer(), b.pointer(), nbytes) == 0
+        ms = time_calls(hip, ctx, call, iters)
+        out[name] = moved * nbytes / (ms * 1e-3) / 1e9
+    a.close()
+    b.close()
+    return out
+
+
 def mfma_rates(hip, ctx):
     """What the matrix cores sustain with register-resident operands and no memory traffic (avhip_mfma_rate_probe), per
     dtype, in T(FL)OP/s: with nearly all-zero operand bits (clock near boost) and with random finite operands, whose
@@ -421,6 +440,7 @@ def main():
         detail["nonfused_winograd_f32_F4"] = nonfused_stages(hip, ctx, "f32", "f32", 4, it)
         detail["nonfused_winograd_bf16_F2_fp16mat"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it)
         detail["copy_GBs_measured"] = copy_bandwidth(hip, ctx)
+        detail["stream_GBs_measured"] = stream_rates(hip, ctx)
         detail["mfma_rate_measured"] = mfma_rates(hip, ctx)
         detail["other_configs"] = other_configs(hip, ctx, it)
         cpu = None if args.no_cpu else cpu_baseline()

@@ -298,6 +298,50 @@ namespace
 	}
 }
 
+namespace
+{
+	/* Streaming kernels of known traffic for a harness that wants this machine's HBM ceilings next to the datasheet figure:
+	 * every work-item moves four 16-byte vectors per trip, a wavefront 1 KiB contiguous per instruction. */
+	typedef unsigned int probe_vec_t __attribute__((ext_vector_type(4)));
+	__global__ __launch_bounds__(256) void k_stream_read(const probe_vec_t *__restrict__ p, size_t vectors, unsigned int *sink)
+	{
+		unsigned int acc = 0;
+		const size_t stride = static_cast<size_t>(gridDim.x) * 1024;
+		for (size_t i = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x; i + 768 < vectors; i += stride)
+		{
+			const probe_vec_t a = __builtin_nontemporal_load(p + i), b = __builtin_nontemporal_load(p + i + 256);
+			const probe_vec_t c = __builtin_nontemporal_load(p + i + 512), d = __builtin_nontemporal_load(p + i + 768);
+			acc ^= a.x ^ b.y ^ c.z ^ d.w;
+		}
+		if (acc == 0x9E3779B9u) /* keeps the loads alive; practically never true */
+			sink[0] = acc;
+	}
+	__global__ __launch_bounds__(256) void k_stream_write(probe_vec_t *__restrict__ p, size_t vectors)
+	{
+		const size_t stride = static_cast<size_t>(gridDim.x) * 1024;
+		const probe_vec_t value = { blockIdx.x, threadIdx.x, 2u, 3u };
+		for (size_t i = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x; i + 768 < vectors; i += stride)
+		{
+			__builtin_nontemporal_store(value, p + i);
+			__builtin_nontemporal_store(value, p + i + 256);
+			__builtin_nontemporal_store(value, p + i + 512);
+			__builtin_nontemporal_store(value, p + i + 768);
+		}
+	}
+	__global__ __launch_bounds__(256) void k_stream_copy(const probe_vec_t *__restrict__ src, probe_vec_t *__restrict__ dst, size_t vectors)
+	{
+		const size_t stride = static_cast<size_t>(gridDim.x) * 1024;
+		for (size_t i = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x; i + 768 < vectors; i += stride)
+		{
+			const probe_vec_t a = src[i], b = src[i + 256], c = src[i + 512], d = src[i + 768];
+			__builtin_nontemporal_store(a, dst + i);
+			__builtin_nontemporal_store(b, dst + i + 256);
+			__builtin_nontemporal_store(c, dst + i + 512);
+			__builtin_nontemporal_store(d, dst + i + 768);
+		}
+	}
+}
+
 extern "C"
 {
 	int avhip_add_bias(void *stream, int dtype, const void *x, const void *b, const void *z, void *y, int64_t first, int last, double alpha1,
@@ -410,5 +454,22 @@ extern "C"
 			default:
 				return AVHIP_BAD_PARAM;
 		}
+	}
+	int avhip_stream_probe(void *stream, int kind, const void *src, void *dst, int64_t bytes)
+	{
+		if (kind < 0 || kind > 2 || bytes < 16384 || dst == nullptr || (kind != 1 && src == nullptr))
+			return AVHIP_BAD_PARAM; /* the read kernel, too, needs one word it may write */
+		if (!aligned_to(src, 16) || !aligned_to(dst, 16))
+			return AVHIP_BAD_PARAM;
+		hipStream_t s = static_cast<hipStream_t>(stream);
+		const size_t vectors = static_cast<size_t>(bytes) / 16;
+		const dim3 grid(8192);
+		if (kind == 0)
+			hipLaunchKernelGGL(k_stream_read, grid, dim3(256), 0, s, static_cast<const probe_vec_t*>(src), vectors, static_cast<unsigned int*>(dst));
+		else if (kind == 1)
+			hipLaunchKernelGGL(k_stream_write, grid, dim3(256), 0, s, static_cast<probe_vec_t*>(dst), vectors);
+		else
+			hipLaunchKernelGGL(k_stream_copy, grid, dim3(256), 0, s, static_cast<const probe_vec_t*>(src), static_cast<probe_vec_t*>(dst), vectors);
+		return 0;
 	}
 }

@@ -134,6 +134,12 @@ extern "C"
 	 * k = 16 / 32 / 2 for 16-bit / int8 / fp32. */
 	AVHIP_API int avhip_mfma_rate_probe(void *stream, int dtype, int workgroups, int iterations, int operands, void *sink);
 
+	/* Measurement aid without a counterpart in the reference: a streaming kernel of known HBM traffic, so that a harness can
+	 * put this machine's read, write and copy ceilings next to the datasheet bandwidth.  kind 0 reads `bytes` from src (dst
+	 * must point to at least 4 writable bytes), kind 1 writes `bytes` to dst, kind 2 copies src to dst (2 * bytes of
+	 * traffic).  16-byte aligned buffers; the last up to 16 KiB of a buffer may stay untouched. */
+	AVHIP_API int avhip_stream_probe(void *stream, int kind, const void *src, void *dst, int64_t bytes);
+
 #ifdef __cplusplus
 }
 #endif
