@@ -185,11 +185,11 @@ namespace
 		}
 	};
 
-	template<typename TE, typename TC, int STEPS>
+	template<typename TE, typename TC, int STEPS, int TM>
 	__global__ __launch_bounds__(256, 2) void k_gemm_nt_persistent(const TE *__restrict__ A, const TE *__restrict__ B, PersistentGeom g, GemmEpilogue<TC> epi)
 	{
 		__shared__ __attribute__((aligned(16))) char lds[PERSISTENT_LDS_BYTES];
-		persistent_nt_gemm<TE, GemmEpilogue<TC>, STEPS>(lds, A, B, g, epi);
+		persistent_nt_gemm<TE, GemmEpilogue<TC>, STEPS, TM>(lds, A, B, g, epi);
 	}
 
 	/* Any operand form, any supported type: 16 x 16 outputs per workgroup, k in slices of 16 through LDS. */
@@ -256,17 +256,19 @@ namespace
 			typedef GemmEpilogue<TC> Epi;
 			const int64_t row_bytes = static_cast<int64_t>(K) * sizeof(TE);
 			const int steps = static_cast<int>((row_bytes + STEP_BYTES - 1) / STEP_BYTES);
-			/* fp32 products are bound by the matrix cores (sixteen-pass MFMAs): for the Winograd shapes measured (1152 tiles
-			 * on 512 resident workgroups) the one-tile kernel, whose workgroups the hardware hands out as slots free up, beats
-			 * a static split of 2.25 rounds of tiles into 2 and 3 (61 against 65 us) */
-			if (!fast || steps > PERSISTENT_MAX_STEPS || sizeof(TE) >= 4)
+			if (!fast || steps > PERSISTENT_MAX_STEPS)
 				return false;
+			/* fp32 products are bound by the matrix cores (sixteen-pass MFMAs), not by operand traffic: half-height tiles cost
+			 * them nothing and split the work into rounds more evenly (the Winograd layer measured: 1152 tiles of 128 rows are
+			 * 2.25 rounds of the 512 resident workgroups, 2304 of 64 rows are 4.5) */
+			constexpr int TM = sizeof(TE) >= 4 ? 1 : 2;
+			constexpr int ROWS = 64 * TM;
 			/* whole 16-byte runs of C, rows of C a multiple of them apart */
 			if (N % Epi::wide != 0 || ldc % Epi::wide != 0 || sC % Epi::wide != 0 || !aligned_to(C, 16) || ldc >= (1 << 24))
 				return false;
 			const int64_t a_bytes = ((batch - 1) * sA + static_cast<int64_t>(M - 1) * lda + K) * static_cast<int64_t>(sizeof(TE));
 			const int64_t b_bytes = ((batch - 1) * sB + static_cast<int64_t>(N - 1) * ldb + K) * static_cast<int64_t>(sizeof(TE));
-			const int64_t row_blocks = ceil_div(M, BLOCK_M), col_blocks = ceil_div(N, BLOCK_N);
+			const int64_t row_blocks = ceil_div(M, ROWS), col_blocks = ceil_div(N, BLOCK_N);
 			const int64_t tiles = row_blocks * col_blocks * batch;
 			if (sA < 0 || sB < 0 || a_bytes >= (1ll << 31) || b_bytes >= (1ll << 31) || tiles >= (1ll << 31) - 1024)
 				return false;
@@ -289,9 +291,9 @@ namespace
 			const Epi epi { static_cast<TC*>(C), static_cast<float>(alpha), static_cast<float>(beta) };
 			const dim3 grid(persistent_workgroups(tiles));
 			if (steps <= 2)
-				hipLaunchKernelGGL((k_gemm_nt_persistent<TE, TC, 2>), grid, dim3(256), 0, s, static_cast<const TE*>(A), static_cast<const TE*>(B), g, epi);
+				hipLaunchKernelGGL((k_gemm_nt_persistent<TE, TC, 2, TM>), grid, dim3(256), 0, s, static_cast<const TE*>(A), static_cast<const TE*>(B), g, epi);
 			else
-				hipLaunchKernelGGL((k_gemm_nt_persistent<TE, TC, 4>), grid, dim3(256), 0, s, static_cast<const TE*>(A), static_cast<const TE*>(B), g, epi);
+				hipLaunchKernelGGL((k_gemm_nt_persistent<TE, TC, 4, TM>), grid, dim3(256), 0, s, static_cast<const TE*>(A), static_cast<const TE*>(B), g, epi);
 			return true;
 		}
 		else

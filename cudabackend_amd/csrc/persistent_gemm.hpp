@@ -41,7 +41,7 @@ namespace avhip
 		unsigned int a_bytes, b_bytes; /* extent of all of A and of B (below 2 GiB) */
 		int64_t c_batch; /* elements between batch members of C */
 		int c_pitch; /* elements between rows of C (below 2^24: 128 rows of it are a 32-bit product) */
-		int row_blocks, col_blocks; /* ceil(rows / 128), ceil(cols / 128) */
+		int row_blocks, col_blocks; /* ceil(rows / tile rows), ceil(cols / 128) */
 		int tiles; /* batch * row_blocks * col_blocks */
 		int table_columns; /* columns whose constants are staged in LDS (cols, or 0 when the epilogue has none) */
 	};
@@ -62,12 +62,18 @@ namespace avhip
 		return r;
 	}
 
-	/* STEPS: k-steps per tile, even (an odd count is rounded up and the extra step reads zeros).  Called by all 256 work-items
-	 * of a workgroup with PERSISTENT_LDS_BYTES of LDS; gridDim.x workgroups share the tiles. */
-	template<typename TE, typename Epi, int STEPS>
+	/* STEPS: k-steps per tile, even (an odd count is rounded up and the extra step reads zeros).  TM: the tile has 64 * TM rows
+	 * (each of the 2 x 2 wavefronts takes TM 32-row MFMA tiles by two 32-column ones); g.row_blocks counts blocks of that
+	 * height.  TM = 1 halves the tile for products so slow per tile (fp32) that evening out the rounds matters more than
+	 * operand reuse.  Called by all 256 work-items of a workgroup with PERSISTENT_LDS_BYTES of LDS; gridDim.x workgroups share
+	 * the tiles. */
+	template<typename TE, typename Epi, int STEPS, int TM = 2>
 	__device__ __forceinline__ void persistent_nt_gemm(char *lds, const TE *__restrict__ A, const TE *__restrict__ B, const PersistentGeom &g, Epi &epi)
 	{
 		static_assert(STEPS % 2 == 0 && STEPS <= PERSISTENT_MAX_STEPS, "register sets and LDS buffers alternate with the step parity");
+		static_assert(TM == 1 || TM == 2, "64 or 128 rows");
+		constexpr int ROWS = 64 * TM;
+		constexpr int A_PASSES = ROWS / FETCH_ROWS;
 		constexpr int W = Epi::wide;
 		static_assert(DrainShape<2, W>::bytes <= 2 * LDS_TILE, "the accumulators leave through one operand buffer");
 		typedef typename Epi::template ColumnsT<1> Record;
@@ -80,32 +86,37 @@ namespace avhip
 		const int fpart = tid & (STEP_CHUNKS - 1);
 		const int frow = tid / STEP_CHUNKS;
 		const int st_off = frow * LDS_ROW + fpart * 16;
-		const int rd_a = (wm * 64 + (lane & 31)) * LDS_ROW + (lane >> 5) * 16;
+		const int rd_a = (wm * 32 * TM + (lane & 31)) * LDS_ROW + (lane >> 5) * 16;
 		const int rd_b = (wn * 64 + (lane & 31)) * LDS_ROW + (lane >> 5) * 16;
 		const __amdgpu_buffer_rsrc_t ra_rsrc = make_buffer(A, g.a_bytes);
 		const __amdgpu_buffer_rsrc_t rb_rsrc = make_buffer(B, g.b_bytes);
 
-		/* tile sequence of this workgroup: round j takes tile j * gridDim.x + (its number within the round, XCD-contiguous) */
-		const int first = xcd_block(blockIdx.x, gridDim.x);
-		const int stride = gridDim.x;
+		/* tile sequence of this workgroup: in round j it takes tile j * gridDim.x + (its number within the round).  In full
+		 * rounds that number is XCD-contiguous (neighbouring tiles share rows of A behind one L2); the last, partial round hands
+		 * its tiles out by plain workgroup number, which spreads them over all XCDs instead of filling the first ones. */
+		const int in_full_round = xcd_block(blockIdx.x, gridDim.x);
+		const int full_rounds = g.tiles / static_cast<int>(gridDim.x);
+		auto tile_of = [&](int round) { return round * static_cast<int>(gridDim.x) + (round < full_rounds ? in_full_round : static_cast<int>(blockIdx.x)); };
 
 		/* the two fetch cursors: A one tile ahead of the MFMAs, B two steps ahead */
-		int a_tile = first, a_step = 0, b_tile = first, b_step = 0;
-		unsigned int a_base[FETCH_PASSES], b_base[FETCH_PASSES];
+		int a_round = 0, a_step = 0, b_round = 0, b_step = 0;
+		unsigned int a_base[A_PASSES], b_base[FETCH_PASSES];
 		auto aim_a = [&]()
 		{
+			const int a_tile = tile_of(a_round);
 			const bool live = a_tile < g.tiles;
 			const PersistentTile t = persistent_tile(g, live ? a_tile : 0);
 #pragma unroll
-			for (int q = 0; q < FETCH_PASSES; q++)
+			for (int q = 0; q < A_PASSES; q++)
 			{
-				const int r = t.row_block * BLOCK_M + frow + FETCH_ROWS * q;
+				const int r = t.row_block * ROWS + frow + FETCH_ROWS * q;
 				a_base[q] = (live && r < g.rows) ? static_cast<unsigned int>(t.batch) * g.a_batch + static_cast<unsigned int>(r) * g.a_pitch + fpart * 16 :
 						OUT_OF_RANGE;
 			}
 		};
 		auto aim_b = [&]()
 		{
+			const int b_tile = tile_of(b_round);
 			const bool live = b_tile < g.tiles;
 			const PersistentTile t = persistent_tile(g, live ? b_tile : 0);
 #pragma unroll
@@ -116,17 +127,17 @@ namespace avhip
 						OUT_OF_RANGE;
 			}
 		};
-		auto fetch_a = [&](uint4 (&a)[FETCH_PASSES]) __attribute__((always_inline))
+		auto fetch_a = [&](uint4 (&a)[A_PASSES]) __attribute__((always_inline))
 		{
 			const unsigned int k_byte = static_cast<unsigned int>(a_step) * STEP_BYTES;
 			const bool in_row = k_byte + fpart * 16 < g.row_bytes;
 #pragma unroll
-			for (int q = 0; q < FETCH_PASSES; q++)
+			for (int q = 0; q < A_PASSES; q++)
 				a[q] = buffer_fetch(ra_rsrc, (in_row && a_base[q] < OUT_OF_RANGE) ? a_base[q] + k_byte : OUT_OF_RANGE);
 			if (++a_step == STEPS)
 			{
 				a_step = 0;
-				a_tile += stride;
+				a_round++;
 				aim_a();
 			}
 		};
@@ -140,37 +151,37 @@ namespace avhip
 			if (++b_step == STEPS)
 			{
 				b_step = 0;
-				b_tile += stride;
+				b_round++;
 				aim_b();
 			}
 		};
-		auto stash = [&](int buffer, const uint4 (&a)[FETCH_PASSES], const uint4 (&b)[FETCH_PASSES]) __attribute__((always_inline))
+		auto stash = [&](int buffer, const uint4 (&a)[A_PASSES], const uint4 (&b)[FETCH_PASSES]) __attribute__((always_inline))
 		{
 			char *sa = lds + buffer * 2 * LDS_TILE;
 			char *sb = sa + LDS_TILE;
 #pragma unroll
-			for (int q = 0; q < FETCH_PASSES; q++)
-			{
+			for (int q = 0; q < A_PASSES; q++)
 				*reinterpret_cast<uint4*>(sa + st_off + q * FETCH_ROWS * LDS_ROW) = a[q];
+#pragma unroll
+			for (int q = 0; q < FETCH_PASSES; q++)
 				*reinterpret_cast<uint4*>(sb + st_off + q * FETCH_ROWS * LDS_ROW) = b[q];
-			}
 		};
 
-		typename Mma<TE>::acc_t acc[2][2];
+		typename Mma<TE>::acc_t acc[TM][2];
 		auto multiply = [&](int buffer) __attribute__((always_inline))
 		{
 			const char *sa = lds + buffer * 2 * LDS_TILE;
 			const char *sb = sa + LDS_TILE;
 			constexpr int SLABS = STEP_BYTES / 32;
-			Chunk a[2][2], b[2][2]; /* LDS reads run one 32-byte slab ahead of the MFMAs */
-			auto read = [&](int slab, Chunk (&ra_)[2], Chunk (&rb_)[2]) __attribute__((always_inline))
+			Chunk a[2][TM], b[2][2]; /* LDS reads run one 32-byte slab ahead of the MFMAs */
+			auto read = [&](int slab, Chunk (&ra_)[TM], Chunk (&rb_)[2]) __attribute__((always_inline))
 			{
 #pragma unroll
-				for (int i = 0; i < 2; i++)
-				{
+				for (int i = 0; i < TM; i++)
 					ra_[i].u = *reinterpret_cast<const uint4*>(sa + rd_a + i * 32 * LDS_ROW + slab * 32);
+#pragma unroll
+				for (int i = 0; i < 2; i++)
 					rb_[i].u = *reinterpret_cast<const uint4*>(sb + rd_b + i * 32 * LDS_ROW + slab * 32);
-				}
 			};
 			read(0, a[0], b[0]);
 #pragma unroll
@@ -181,7 +192,7 @@ namespace avhip
 				if (sizeof(TE) < 4)
 					__builtin_amdgcn_s_setprio(1);
 #pragma unroll
-				for (int i = 0; i < 2; i++)
+				for (int i = 0; i < TM; i++)
 #pragma unroll
 					for (int j = 0; j < 2; j++)
 						Mma<TE>::run(a[slab & 1][i], b[slab & 1][j], acc[i][j]);
@@ -191,7 +202,7 @@ namespace avhip
 		};
 
 		/* prologue: all of the first tile's A, two steps of B, step 0 into LDS, and set 0 of A goes on to the second tile */
-		uint4 ra[STEPS][FETCH_PASSES], rb[2][FETCH_PASSES];
+		uint4 ra[STEPS][A_PASSES], rb[2][FETCH_PASSES];
 		aim_a();
 		aim_b();
 #pragma unroll
@@ -205,12 +216,12 @@ namespace avhip
 		fetch_a(ra[0]);
 
 		const int col_in_tile = drain_column<2, W>();
-		for (int tile = first; tile < g.tiles; tile += stride)
+		for (int round = 0; tile_of(round) < g.tiles; round++)
 		{
-			const PersistentTile t = persistent_tile(g, tile);
+			const PersistentTile t = persistent_tile(g, tile_of(round));
 			const int col = t.col_block * BLOCK_N + col_in_tile;
 #pragma unroll
-			for (int i = 0; i < 2; i++)
+			for (int i = 0; i < TM; i++)
 #pragma unroll
 				for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -229,12 +240,12 @@ namespace avhip
 			}
 			/* buffer 1 was multiplied last and is refilled only after the next barrier of the loop above: the accumulators
 			 * leave through it while buffer 0 already holds step 0 of the next tile */
-			const int64_t c0 = static_cast<int64_t>(t.batch) * g.c_batch + static_cast<int64_t>(t.row_block * BLOCK_M) * g.c_pitch + col;
-			const int row0 = t.row_block * BLOCK_M;
+			const int64_t c0 = static_cast<int64_t>(t.batch) * g.c_batch + static_cast<int64_t>(t.row_block * ROWS) * g.c_pitch + col;
+			const int row0 = t.row_block * ROWS;
 			typename Epi::template ColumnsT<W> columns;
 			if (col < g.table_columns)
 				Epi::pick_columns(table, col, columns);
-			drain_tile<TE, 2, 2, W>(lds + 2 * LDS_TILE, acc, [&](int r, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
+			drain_tile<TE, TM, 2, W>(lds + 2 * LDS_TILE, acc, [&](int r, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
 			{
 				if (row0 + r < g.rows && col < g.cols)
 					epi.template store_at<ACT_SIMPLE, true, W>(c0 + r * g.c_pitch, col, v, columns);
