@@ -395,10 +395,10 @@ namespace
 		uint64_t uid;
 		uint64_t version;
 		av_int64 offset;
-		int K, C, dtype, mode;
+		int K, C, dtype, mode, m; /* m: Winograd output tile, 2 = F(2x2,3x3) for the fused kernel, 4 = F(4x4,3x3) for the non-fused plan */
 		bool operator<(const WeightKey &o) const
 		{
-			return std::tie(uid, version, offset, K, C, dtype, mode) < std::tie(o.uid, o.version, o.offset, o.K, o.C, o.dtype, o.mode);
+			return std::tie(uid, version, offset, K, C, dtype, mode, m) < std::tie(o.uid, o.version, o.offset, o.K, o.C, o.dtype, o.mode, o.m);
 		}
 	};
 	struct WeightCache
@@ -438,17 +438,16 @@ namespace
 		return ++uid;
 	}
 
-	/* Returns the [16, K, C] F(2x2,3x3) weight matrices for the fused kernel (fp16 for 16-bit tensors, fp32 for fp32),
-	 * transforming on `stream` when the weight block changed since the cached copy was made. */
-	avStatus_t fused_weights(const Context &ctx, const ConvProblem &p, avMemoryDescriptor_t wMem, const void **U)
+	/* Returns the [t*t, K, C] Winograd weight matrices F(m x m, 3x3) of a weight tensor in `mat_dtype`, transforming on the
+	 * context's stream when the weight block changed since the cached copy was made. */
+	avStatus_t cached_winograd_weights(const Context &ctx, const ConvProblem &p, avMemoryDescriptor_t wMem, int m, avDataType_t mat_dtype, const void **U)
 	{
 		Memory *wm = get_memory(wMem);
 		Memory *owner = owner_of(wm);
 		if (wm == nullptr || owner == nullptr)
 			return AVOCADO_STATUS_BAD_PARAM;
-		const avDataType_t mat_dtype = (p.w_dtype == AVOCADO_DTYPE_FLOAT32) ? AVOCADO_DTYPE_FLOAT32 : AVOCADO_DTYPE_FLOAT16;
 		const WeightKey key { owner->uid, owner->version, static_cast<av_int64>(wm->data - owner->data), p.shape.K, p.shape.C,
-				static_cast<int>(p.w_dtype), p.shape.mode };
+				static_cast<int>(p.w_dtype), p.shape.mode, m };
 		WeightCache &cache = weight_cache();
 		std::lock_guard<std::mutex> lock(cache.mutex);
 		auto it = cache.entries.find(key);
@@ -457,9 +456,9 @@ namespace
 			*U = it->second;
 			return AVOCADO_STATUS_SUCCESS;
 		}
-		/* stale copies of the same tensor are of no further use */
+		/* copies of older versions of the same tensor are of no further use */
 		for (auto e = cache.entries.begin(); e != cache.entries.end();)
-			if (e->first.uid == key.uid && e->first.offset == key.offset)
+			if (e->first.uid == key.uid && e->first.offset == key.offset && e->first.version != key.version)
 			{
 				/* the kernel that last read it may still be running on another stream: order the free behind all work */
 				(void) hipDeviceSynchronize();
@@ -469,13 +468,14 @@ namespace
 			else
 				++e;
 		void *buf = nullptr;
-		const size_t bytes = static_cast<size_t>(16) * p.shape.K * p.shape.C * size_of(mat_dtype);
+		const int t = m + 2;
+		const size_t bytes = static_cast<size_t>(t * t) * p.shape.K * p.shape.C * size_of(mat_dtype);
 		if (hipMalloc(&buf, bytes) != hipSuccess)
 		{
 			(void) hipGetLastError();
 			return AVOCADO_STATUS_ALLOC_FAILED;
 		}
-		const int rc = avhip_winograd_weight_transform(ctx.stream, p.w_dtype, mat_dtype, 2, 3, p.shape.mode, wm->data, buf, p.shape.K, p.shape.C);
+		const int rc = avhip_winograd_weight_transform(ctx.stream, p.w_dtype, mat_dtype, m, 3, p.shape.mode, wm->data, buf, p.shape.K, p.shape.C);
 		const avStatus_t st = from_launcher(rc);
 		if (st != AVOCADO_STATUS_SUCCESS)
 		{
@@ -485,6 +485,12 @@ namespace
 		cache.entries[key] = buf;
 		*U = buf;
 		return AVOCADO_STATUS_SUCCESS;
+	}
+	/* [16, K, C] for the fused kernel: fp16 matrices for 16-bit tensors, fp32 for fp32 */
+	avStatus_t fused_weights(const Context &ctx, const ConvProblem &p, avMemoryDescriptor_t wMem, const void **U)
+	{
+		const avDataType_t mat_dtype = (p.w_dtype == AVOCADO_DTYPE_FLOAT32) ? AVOCADO_DTYPE_FLOAT32 : AVOCADO_DTYPE_FLOAT16;
+		return cached_winograd_weights(ctx, p, wMem, 2, mat_dtype, U);
 	}
 
 	bool winograd_supported(int r, int m)
@@ -654,10 +660,11 @@ namespace
 		return from_launcher(rc);
 	}
 
-	/* Non-fused Winograd F(4x4,3x3) through a caller workspace laid out as [U | V | M], each part 256-byte aligned. */
+	/* Non-fused Winograd F(4x4,3x3) through a caller workspace laid out as [V | M], each part 256-byte aligned; the transformed
+	 * weights come from the library's cache (one transform per weight tensor and version). */
 	struct NonFusedPlan
 	{
-		av_int64 u_bytes, v_bytes, m_bytes, total;
+		av_int64 v_bytes, m_bytes, total;
 		int tiles;
 		avDataType_t mat_dtype;
 	};
@@ -673,20 +680,29 @@ namespace
 			return false;
 		plan.mat_dtype = AVOCADO_DTYPE_FLOAT32;
 		plan.tiles = s.N * ((s.H + 3) / 4) * ((s.W + 3) / 4);
-		plan.u_bytes = align256(static_cast<av_int64>(36) * s.K * s.C * 4);
 		plan.v_bytes = align256(static_cast<av_int64>(36) * plan.tiles * s.C * 4);
 		plan.m_bytes = align256(static_cast<av_int64>(36) * plan.tiles * s.K * 4);
-		plan.total = plan.u_bytes + plan.v_bytes + plan.m_bytes;
+		plan.total = plan.v_bytes + plan.m_bytes;
 		return true;
 	}
-	avStatus_t run_nonfused_winograd(const ConvCall &c, const NonFusedPlan &plan, Memory *ws, avMemoryDescriptor_t yMem, avActivationType_t activation)
+	/* Large fp32 layers: three HBM-bound passes around a batched GEMM that needs a quarter of the direct multiplications
+	 * beat the fused kernel, which needs 4/9 of them and forms its operands in registers (measured on 256 x 15 x 15 x 128 ->
+	 * 128: 16 + 56 + 18 us against 105 us; the weights are transformed once and cached).  Small ones do not fill the four launches. */
+	bool nonfused_preferred(const ConvProblem &p, const NonFusedPlan &plan)
+	{
+		return plan.tiles >= 2048 && p.shape.C >= 64 && p.shape.K >= 64;
+	}
+	avStatus_t run_nonfused_winograd(const ConvCall &c, const NonFusedPlan &plan, Memory *ws, avMemoryDescriptor_t wMem, avMemoryDescriptor_t yMem,
+			avActivationType_t activation)
 	{
 		const avhipConvShape &s = c.problem.shape;
-		char *U = ws->data, *V = U + plan.u_bytes, *Mx = V + plan.v_bytes;
+		char *V = ws->data, *Mx = V + plan.v_bytes;
 		void *st = c.ctx.stream;
-		int rc = avhip_winograd_weight_transform(st, AVOCADO_DTYPE_FLOAT32, plan.mat_dtype, 4, 3, s.mode, c.w->data, U, s.K, s.C);
-		if (rc == 0)
-			rc = avhip_winograd_input_transform(st, AVOCADO_DTYPE_FLOAT32, plan.mat_dtype, 4, 3, c.x->data, V, s.N, s.H, s.W, s.C, s.pad_h, s.pad_w,
+		const void *U = nullptr;
+		const avStatus_t ws_status = cached_winograd_weights(c.ctx, c.problem, wMem, 4, plan.mat_dtype, &U);
+		if (ws_status != AVOCADO_STATUS_SUCCESS)
+			return ws_status;
+		int rc = avhip_winograd_input_transform(st, AVOCADO_DTYPE_FLOAT32, plan.mat_dtype, 4, 3, c.x->data, V, s.N, s.H, s.W, s.C, s.pad_h, s.pad_w,
 					padding_value_or_null(c.problem.conv));
 		if (rc == 0)
 			rc = avhip_gemm_batched(st, plan.mat_dtype, plan.mat_dtype, 0, 1, V, U, Mx, 36, plan.tiles, s.K, s.C, s.C, s.C, s.K,
@@ -1553,7 +1569,7 @@ namespace avocado
 			if (st != AVOCADO_STATUS_SUCCESS)
 				return st;
 			NonFusedPlan plan;
-			result[0] = (!fused_winograd_applicable(p) && nonfused_plan(p, plan)) ? plan.total : 0;
+			result[0] = (nonfused_plan(p, plan) && (nonfused_preferred(p, plan) || !fused_winograd_applicable(p))) ? plan.total : 0;
 			return AVOCADO_STATUS_SUCCESS;
 		}
 
@@ -1577,6 +1593,15 @@ namespace avocado
 			 * kernels, which can cut it finer */
 			const av_int64 fused_workgroups = static_cast<av_int64>(p.shape.N) * ((p.shape.Ho + 15) / 16) * ((p.shape.Wo + 15) / 16)
 					* ((p.shape.K + 127) / 128);
+			NonFusedPlan plan;
+			Memory *ws = get_memory(workspaceMem);
+			const bool nonfused_ready = nonfused_plan(p, plan) && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32 && ws != nullptr && ws->data != nullptr
+					&& ws->size >= plan.total && reinterpret_cast<uintptr_t>(ws->data) % 256 == 0;
+			if (nonfused_ready && nonfused_preferred(p, plan))
+			{
+				touch(workspaceMem);
+				return run_nonfused_winograd(call, plan, ws, wMem, yMem, activation);
+			}
 			if (fused_winograd_applicable(p) && p.x_dtype == AVOCADO_DTYPE_FLOAT32 && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32
 					&& p.shape.Ho == p.shape.H && p.shape.Wo == p.shape.W && fused_workgroups >= 128)
 			{
@@ -1584,13 +1609,10 @@ namespace avocado
 				if (fs != AVOCADO_STATUS_NOT_SUPPORTED)
 					return fs;
 			}
-			NonFusedPlan plan;
-			Memory *ws = get_memory(workspaceMem);
-			if (nonfused_plan(p, plan) && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32 && ws != nullptr && ws->data != nullptr && ws->size >= plan.total
-					&& reinterpret_cast<uintptr_t>(ws->data) % 256 == 0)
+			if (nonfused_ready)
 			{
 				touch(workspaceMem);
-				return run_nonfused_winograd(call, plan, ws, yMem, activation);
+				return run_nonfused_winograd(call, plan, ws, wMem, yMem, activation);
 			}
 			return run_implicit_gemm(call, yMem, activation, nullptr);
 		}

@@ -324,6 +324,45 @@ def test_dispatcher_without_workspace_falls_back(oracle):
     np.testing.assert_array_equal(got, oracle.conv2d_i8(xi, wi, None))
 
 
+def test_dispatcher_large_fp32_layer_takes_workspace_and_sees_rewritten_weights(oracle):
+    """A large fp32 3x3 layer asks for a workspace ([V | M] of non-fused F(4x4,3x3)) and, given it, runs the three-pass plan
+    with weights transformed once and cached per memory block and version: overwriting the weights through the API must show
+    in the next call; without the workspace the same call still succeeds (fused kernel)."""
+    g = h.rng(33)
+    N, H, W, Cin, K = 40, 15, 15, 64, 64       # 40 x 4 x 4 = 640 tiles of 4 x 4 ... below the threshold
+    x = h.rounded(oracle, g.standard_normal((N, H, W, Cin)), "f32")
+    w1, w2 = he(g, (K, 3, 3, Cin), "f32", oracle), he(g, (K, 3, 3, Cin), "f32", oracle)
+    b = g.uniform(-0.1, 0.1, K).astype(np.float32).astype(np.float64)
+    got = h.conv_forward("dispatch", x, w1, (N, H, W, K), "f32", bias=b, activation=cb.ACTIVATION_RELU)
+    assert oracle.rel_l2(got, oracle.conv2d(x, w1, b, activation=oracle.RELU)) < 1e-4
+    N = 136                                    # 136 x 16 = 2176 tiles: the non-fused plan is preferred
+    x = h.rounded(oracle, g.standard_normal((N, H, W, Cin)), "f32")
+    z = h.rounded(oracle, g.standard_normal((N, H, W, K)), "f32")
+    with h.Call() as c:
+        conv = cb.ConvolutionDescriptor(padding=(-1, -1), dtype=cb.DTYPE_FLOAT32)
+        xt, wt, bt, zt, y = c.tensor(x, "f32"), c.tensor(w1, "f32"), c.tensor(b, "f32"), c.tensor(z, "f32"), c.empty((N, H, W, K), "f32")
+        need = h.C.c_int64(0)
+        cb.check(c.lib.cudaGetConvolutionWorkspaceSize(c.ctx.handle, conv.handle, xt.desc, wt.desc, bt.desc, h.C.byref(need)), "workspace size")
+        tiles = N * 4 * 4
+        assert need.value >= 36 * tiles * (Cin + K) * 4
+        ws = c.empty((need.value,), cb.DTYPE_UINT8)
+
+        def run(workspace):
+            st = c.lib.cudaConvolutionBiasActivationForward(c.ctx.handle, conv.handle, None, xt.desc, xt.mem, wt.desc, wt.mem, bt.desc, bt.mem, None,
+                                                            zt.desc, zt.mem, None, y.desc, y.mem, cb.ACTIVATION_RELU, workspace)
+            assert st == cb.STATUS_SUCCESS
+            c.finish()
+            return y.download()
+        first = run(ws.mem)
+        wt.upload(w2)
+        second = run(ws.mem)
+        third = run(0)
+    want2 = oracle.conv2d(x, w2, b, z, activation=oracle.RELU)
+    assert oracle.rel_l2(first, oracle.conv2d(x, w1, b, z, activation=oracle.RELU)) < 1e-4
+    assert oracle.rel_l2(second, want2) < 1e-4
+    assert oracle.rel_l2(third, want2) < 1e-4
+
+
 def test_convolution_argument_errors(oracle):
     x = np.zeros((2, 6, 6, 8))
     w = np.zeros((4, 3, 3, 8))
