@@ -42,6 +42,32 @@ def test_gemm_batched_nt(oracle, dtype, c_dtype, shape):
     assert oracle.rel_l2(got, want) < tol
 
 
+@pytest.mark.parametrize("dtype,c_dtype", [("f32", "f32"), ("f16", "f32"), ("bf16", "bf16"), ("bf16", "f32")])
+def test_gemm_batched_nt_random_shapes(oracle, dtype, c_dtype):
+    """Seeded random batched (N, T) products with alpha and beta: short k (the persistent kernel: one to four 128-byte steps,
+    several rounds of tiles per workgroup, ragged last row block) and k, n that send the call to the one-tile kernel (k beyond
+    four steps, n not a multiple of the 16-byte run)."""
+    g = h.rng(13)
+    esz = 4 if dtype == "f32" else 2
+    for case in range(10):
+        if case == 0:
+            batch, M, N, K = 9, 64 * 130 + 7, 128, 96 // esz * 2     # more tiles than resident workgroups
+        else:
+            batch = int(g.integers(1, 6))
+            M = int(g.integers(1, 700))
+            N = int(g.choice([8, 24, 64, 128, 136, 200, 45]))
+            K = int(g.choice([8, 16, 32, 64, 96, 128, 256, 67])) if case < 8 else int(g.choice([512, 384]))
+        A = h.rounded(oracle, g.standard_normal((batch, M, K)), dtype)
+        B = h.rounded(oracle, g.standard_normal((batch, N, K)), dtype)
+        C0 = h.rounded(oracle, g.standard_normal((batch, M, N)), c_dtype)
+        a, b = (float(np.float32(0.7)), float(np.float32(0.3))) if case % 2 else (None, None)
+        print("gemm", dtype, c_dtype, batch, M, N, K, a, b, flush=True)
+        got = h.gemm(A, B, C0, dtype, False, True, a, b, c_dtype=c_dtype, batched=True)
+        want = oracle.gemm_batched(A, B, C0, False, True, a if a is not None else 1.0, b if b is not None else 0.0)
+        tol = TOL[c_dtype] if c_dtype != "f32" else 2e-6
+        assert oracle.rel_l2(got, want) < tol, (batch, M, N, K)
+
+
 @pytest.mark.parametrize("opA,opB", [(False, False), (True, False), (True, True)])
 def test_gemm_batched_other_forms(oracle, opA, opB):
     g = h.rng(12)
