@@ -248,15 +248,20 @@ namespace
 		 * loop only. */
 		typedef DrainRows<2, 1, W> Rows;
 		const int64_t image_base = static_cast<int64_t>(n) * g.Ho * g.Wo * g.K + kcol; /* element index of (image n, pixel 0, filter kcol); one image of y is below 2^31 elements (checked by the launcher) */
-		typename Epi::template Residual<W> residual[Rows::slots];
+		/* (16-bit and int8 tensors only: sixteen rows of four fp32 values are 64 registers, which the fp32 instance does not
+		 * have; it loads its residual row by row in the epilogue) */
+		constexpr bool RESIDUAL_AHEAD = sizeof(TE) < 4;
+		typename Epi::template Residual<W> residual[RESIDUAL_AHEAD ? Rows::slots : 1];
 		auto fetch_residual = [&]() __attribute__((always_inline))
 		{
+			if (!RESIDUAL_AHEAD)
+				return;
 #pragma unroll
 			for (int slot = 0; slot < Rows::slots; slot++)
 			{
 				const int e = row_table[Rows::row(slot)];
 				if (e >= 0 && kcol < g.K)
-					epi.load_residual(image_base + e * g.K, residual[slot]);
+					epi.load_residual(image_base + e * g.K, residual[RESIDUAL_AHEAD ? slot : 0]);
 			}
 		};
 
@@ -308,7 +313,7 @@ namespace
 		{
 			const int e = row_table[row];
 			if (e >= 0 && kcol < g.K)
-				epi.template store_at<ACT_SIMPLE, true, W>(image_base + e * g.K, kcol, v, columns, &residual[slot]);
+				epi.template store_at<ACT_SIMPLE, true, W>(image_base + e * g.K, kcol, v, columns, RESIDUAL_AHEAD ? &residual[slot] : nullptr);
 		});
 	}
 
