@@ -23,6 +23,8 @@
 #ifndef AVHIP_PERSISTENT_GEMM_HPP_
 #define AVHIP_PERSISTENT_GEMM_HPP_
 
+#include <atomic>
+
 #include "conv_epilogue.hpp"
 #include "mfma_core.hpp"
 
@@ -256,10 +258,20 @@ namespace avhip
 	/* How many workgroups to launch: two per compute unit stay resident; with fewer tiles every workgroup has one. */
 	inline unsigned int persistent_workgroups(int64_t tiles)
 	{
-		int device = 0, units = 256;
-		if (hipGetDevice(&device) == hipSuccess)
-			(void) hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device);
-		const int64_t resident = 2 * static_cast<int64_t>(units > 0 ? units : 256);
+		static std::atomic<int> known_units[64]; /* per device, 0 = not asked yet; the answer never changes */
+		int device = 0, units = 0;
+		if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64)
+			device = -1;
+		if (device >= 0)
+			units = known_units[device].load(std::memory_order_relaxed);
+		if (units <= 0)
+		{
+			if (device < 0 || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || units <= 0)
+				units = 256;
+			else
+				known_units[device].store(units, std::memory_order_relaxed);
+		}
+		const int64_t resident = 2 * static_cast<int64_t>(units);
 		return static_cast<unsigned int>(tiles < resident ? tiles : resident);
 	}
 }
