@@ -1,6 +1,6 @@
 /*
  * persistent_gemm.hpp -- a batched NT product  C[b][rows, cols] = A[b][rows, k] * B[b][cols, k]^T  with a SHORT k, run by
- * workgroups that stay on their compute unit and walk a sequence of 128 x 128 tiles as one software pipeline.
+ * workgroups that stay on their compute unit and walk a sequence of 128 x 128 (or 64 x 128) tiles as one software pipeline.
  *
  * Used where k is so short (at most four 128-byte steps) that a workgroup computing a single tile spends most of its life
  * waiting for its first operands and draining its accumulators: 1x1 convolutions (conv_pointwise.hip) and the batched GEMM
