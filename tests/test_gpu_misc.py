@@ -152,3 +152,38 @@ def test_affine_forward_and_batchnorm_inference(oracle, dtype, tol):
     x = np.zeros((2, 4, 8))
     h.affine_forward(x, np.zeros(5), np.zeros(5), "f32", expect=cb.STATUS_BAD_PARAM)  # 5 does not divide 64
     h.affine_forward(x.astype(np.int32), np.zeros(8), np.zeros(8), "i32", expect=cb.STATUS_UNSUPPORTED_DATATYPE)
+
+
+def test_measurement_probes_run_and_validate_arguments():
+    """The two measurement aids of the kernel layer: they launch, leave the device healthy and refuse nonsense."""
+    import ctypes as C
+    lib = cb.load_library()
+    lib.avhip_mfma_rate_probe.restype = C.c_int
+    lib.avhip_mfma_rate_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    lib.avhip_stream_probe.restype = C.c_int
+    lib.avhip_stream_probe.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int64]
+    ctx = cb.Context(0)
+    sink = cb.DeviceTensor((64 * 256,), cb.DTYPE_FLOAT32)
+    for dtype in (cb.DTYPE_BFLOAT16, cb.DTYPE_FLOAT16, cb.DTYPE_INT8, cb.DTYPE_FLOAT32):
+        for operands in (0, 1):
+            assert lib.avhip_mfma_rate_probe(ctx.stream(), dtype, 64, 16, operands, sink.pointer()) == 0
+    assert lib.avhip_mfma_rate_probe(ctx.stream(), cb.DTYPE_FLOAT64, 64, 16, 0, sink.pointer()) != 0
+    assert lib.avhip_mfma_rate_probe(ctx.stream(), cb.DTYPE_BFLOAT16, 0, 16, 0, sink.pointer()) != 0
+    assert lib.avhip_mfma_rate_probe(ctx.stream(), cb.DTYPE_BFLOAT16, 64, 16, 2, sink.pointer()) != 0
+    n = 1 << 20
+    a = cb.DeviceTensor.from_numpy(np.arange(n, dtype=np.int32), cb.DTYPE_INT32)
+    b = cb.DeviceTensor((n,), cb.DTYPE_INT32)
+    assert lib.avhip_stream_probe(ctx.stream(), 2, a.pointer(), b.pointer(), 4 * n) == 0
+    assert lib.avhip_stream_probe(ctx.stream(), 0, a.pointer(), sink.pointer(), 4 * n) == 0
+    assert lib.avhip_stream_probe(ctx.stream(), 1, None, sink.pointer(), 4 * 64 * 256) == 0
+    assert lib.avhip_stream_probe(ctx.stream(), 3, a.pointer(), b.pointer(), 4 * n) != 0
+    assert lib.avhip_stream_probe(ctx.stream(), 2, None, b.pointer(), 4 * n) != 0
+    assert lib.avhip_stream_probe(ctx.stream(), 2, a.pointer(), b.pointer(), 64) != 0
+    ctx.synchronize()
+    got = b.download()
+    # the copy moves everything but at most the last 16 KiB
+    np.testing.assert_array_equal(got[:n - 4096], np.arange(n - 4096, dtype=np.int32))
+    for t in (a, b, sink):
+        t.close()
+    ctx.close()
+
