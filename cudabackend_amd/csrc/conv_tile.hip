@@ -43,7 +43,7 @@ namespace
 	constexpr int TILE_LDS = ROW_TABLE + TILE_M * 4;
 	constexpr int HALO_FETCHES = (HALO_MAX * STEP_CHUNKS + 255) / 256; /* 16-byte chunks of the halo per work-item */
 	constexpr int FILTER_FETCHES = TILE_N * STEP_CHUNKS / 256;
-	static_assert(DrainShape<1>::bytes <= ROW_TABLE, "the drain buffer reuses the operand buffers");
+	static_assert(4 * PrivateDrainRows<2, 4>::bytes <= ROW_TABLE, "the drain buffers of the four wavefronts reuse the operand buffers");
 
 	struct TileGeom
 	{
@@ -246,7 +246,7 @@ namespace
 		/* The residual of every row this work-item will store is requested during the last channel slice: its latency and its
 		 * HBM traffic run under the MFMAs of that slice instead of in the epilogue, and the registers are held for half the
 		 * loop only. */
-		typedef DrainRows<2, 1, W> Rows;
+		typedef PrivateDrainRows<2, W> Rows;
 		const int64_t image_base = static_cast<int64_t>(n) * g.Ho * g.Wo * g.K + kcol; /* element index of (image n, pixel 0, filter kcol); one image of y is below 2^31 elements (checked by the launcher) */
 		/* (16-bit and int8 tensors only: sixteen rows of four fp32 values are 64 registers, which the fp32 instance does not
 		 * have; it loads its residual row by row in the epilogue) */
@@ -309,7 +309,7 @@ namespace
 			step(s + 5, 1, fr[2], fr[0]);
 		}
 
-		drain_tile<TE, 2, 1, W>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[W], int slot) __attribute__((always_inline))
+		drain_tile_private<TE, 2, W>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[W], int slot) __attribute__((always_inline))
 		{
 			const int e = row_table[row];
 			if (e >= 0 && kcol < g.K)

@@ -347,6 +347,72 @@ namespace avhip
 			}
 		}
 	}
+
+	/*
+	 * The same hand-over for workgroups whose four wavefronts are stacked (each owns TM 32-row tiles by 64 columns, the
+	 * workgroup (4 * TM * 32) rows by 64 columns), without workgroup barriers after the first: a wavefront passes its own
+	 * accumulators through its own 8.5 KB of LDS, where its writes and reads stay in program order, so nobody waits for the
+	 * slowest wavefront between the passes.  A work-item gets CPL consecutive columns (drain_column<1, CPL>()) of rows of its
+	 * own wavefront; PrivateDrainRows<...>::row(slot) names the row of call `slot`.  `lds` needs 4 * PrivateDrainRows::bytes.
+	 */
+	template<int TM, int CPL> struct PrivateDrainRows
+	{
+		static constexpr int pitch = 64 + 4; /* words per LDS row: keeps rows 16-byte aligned and staggers banks */
+		static constexpr int threads_per_row = 64 / CPL;
+		static constexpr int rows_per_sweep = 64 / threads_per_row; /* rows one wavefront covers per instruction */
+		static constexpr int iterations = 32 / rows_per_sweep; /* sweeps per 32-row MFMA tile */
+		static constexpr int slots = TM * iterations;
+		static constexpr int bytes = 32 * pitch * 4; /* per wavefront */
+		__device__ static inline int row(int slot)
+		{
+			const int tm = slot / iterations, it = slot - tm * iterations;
+			const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+			return wave * (TM * 32) + tm * 32 + lane / threads_per_row + it * rows_per_sweep;
+		}
+	};
+	template<typename TE, int TM, int CPL, typename F>
+	__device__ __forceinline__ void drain_tile_private(char *lds, const typename Mma<TE>::acc_t (&acc)[TM][2], const F &f)
+	{
+		typedef typename Mma<TE>::scalar_t S;
+		typedef PrivateDrainRows<TM, CPL> D;
+		static_assert(sizeof(S) == 4, "accumulators are 32-bit");
+		static_assert(CPL == 4 || CPL == 8 || CPL == 16, "a work-item takes 4, 8 or 16 consecutive columns");
+		const int lane = threadIdx.x & 63;
+		const int wave = threadIdx.x >> 6;
+		S *sm = reinterpret_cast<S*>(lds + wave * D::bytes);
+		const int col = (lane % D::threads_per_row) * CPL;
+		__syncthreads(); /* the last LDS reads of the k loop, by any wavefront, are over */
+#pragma unroll
+		for (int tm = 0; tm < TM; tm++)
+		{
+#pragma unroll
+			for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+				for (int i = 0; i < 4; i++)
+#pragma unroll
+					for (int j = 0; j < 4; j++)
+						sm[(8 * i + 4 * (lane >> 5) + j) * D::pitch + tn * 32 + (lane & 31)] = acc[tm][tn][4 * i + j];
+			/* what other lanes of this wavefront wrote is read next: LDS serves a wavefront's accesses in order, the fence keeps
+			 * the compiler from reordering them */
+			__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+			Pack<S, 4> vals[D::iterations][CPL / 4];
+#pragma unroll
+			for (int it = 0; it < D::iterations; it++)
+#pragma unroll
+				for (int part = 0; part < CPL / 4; part++)
+					vals[it][part] = *reinterpret_cast<const Pack<S, 4>*>(sm + (lane / D::threads_per_row + it * D::rows_per_sweep) * D::pitch + col + 4 * part);
+			__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront"); /* the next pass overwrites what was just read */
+#pragma unroll
+			for (int it = 0; it < D::iterations; it++)
+			{
+				S v[CPL];
+#pragma unroll
+				for (int q = 0; q < CPL; q++)
+					v[q] = vals[it][q / 4].v[q % 4];
+				f(D::row(tm * D::iterations + it), v, tm * D::iterations + it);
+			}
+		}
+	}
 }
 
 #endif /* AVHIP_MFMA_CORE_HPP_ */
