@@ -159,6 +159,21 @@ namespace avhip
 		asm volatile("" : "+s"(v));
 	}
 
+	/* Issue priority of a wavefront inside the MFMA burst of one k-step, by how far the burst has come (slab = 32-byte part of
+	 * the step).  Two wavefronts of different workgroups share a SIMD and its one matrix pipeline; at equal priority their
+	 * bursts interleave, both finish late and both then wait for LDS together.  A wavefront that is further into its burst
+	 * wins, so bursts run one after the other and each wavefront's loads and barrier fall under the other's MFMAs (measured
+	 * on the 3x3 tile kernel: 3 % on the whole kernel against one fixed raised priority).  s_setprio takes an immediate. */
+	__device__ __forceinline__ void burst_priority(int slab)
+	{
+		if (slab == 0)
+			__builtin_amdgcn_s_setprio(1);
+		else if (slab == 1)
+			__builtin_amdgcn_s_setprio(2);
+		else
+			__builtin_amdgcn_s_setprio(3);
+	}
+
 	/* Workgroups of a grid are handed to the eight XCDs of the chip round-robin (workgroup b runs on XCD b % 8) and every
 	 * XCD has its own L2.  Kernels whose neighbouring blocks of work share input (tiles with halos, pixel blocks whose filter
 	 * windows overlap) renumber their workgroups so that each XCD owns a contiguous eighth of the blocks: workgroup b of nb

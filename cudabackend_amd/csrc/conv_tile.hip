@@ -219,13 +219,14 @@ namespace
 				if (slab + 1 < SLABS)
 					read(slab + 1, a[(slab + 1) & 1], bq[(slab + 1) & 1]);
 				/* a wavefront with operands in hand goes ahead of one that is still issuing loads */
-				__builtin_amdgcn_s_setprio(1);
+				burst_priority(slab);
 #pragma unroll
 				for (int tm = 0; tm < 2; tm++)
 #pragma unroll
 					for (int tn = 0; tn < 2; tn++)
 						Mma<TE>::run(a[slab & 1][tm], bq[slab & 1][tn], acc[tm][tn]);
-				__builtin_amdgcn_s_setprio(0);
+				if (slab + 1 == SLABS)
+					__builtin_amdgcn_s_setprio(0);
 			}
 			/* instruction order within the step: after the first slab's reads, one LDS read behind every MFMA, so that reads
 			 * of the next slab trickle out under the matrix pipeline instead of in a burst between two groups of MFMAs */

@@ -233,13 +233,13 @@ namespace avhip
 				/* a wavefront with operands in hand goes ahead of one that is still issuing loads (measured: helps the short 16-bit
 				 * and int8 MFMAs, hurts the sixteen-pass fp32 ones, whose loaders then starve) */
 				if (sizeof(TE) < 4)
-					__builtin_amdgcn_s_setprio(1);
+					burst_priority(slab);
 #pragma unroll
 				for (int i = 0; i < 2; i++)
 #pragma unroll
 					for (int j = 0; j < 2; j++)
 						Mma<TE>::run(a[slab & 1][i], b[slab & 1][j], acc[i][j]);
-				if (sizeof(TE) < 4)
+				if (sizeof(TE) < 4 && slab + 1 == SLABS)
 					__builtin_amdgcn_s_setprio(0);
 			}
 		};

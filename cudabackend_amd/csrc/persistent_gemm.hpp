@@ -192,13 +192,13 @@ namespace avhip
 				if (slab + 1 < SLABS)
 					read(slab + 1, a[(slab + 1) & 1], b[(slab + 1) & 1]);
 				if (sizeof(TE) < 4)
-					__builtin_amdgcn_s_setprio(1);
+					burst_priority(slab);
 #pragma unroll
 				for (int i = 0; i < TM; i++)
 #pragma unroll
 					for (int j = 0; j < 2; j++)
 						Mma<TE>::run(a[slab & 1][i], b[slab & 1][j], acc[i][j]);
-				if (sizeof(TE) < 4)
+				if (sizeof(TE) < 4 && slab + 1 == SLABS)
 					__builtin_amdgcn_s_setprio(0);
 			}
 		};
