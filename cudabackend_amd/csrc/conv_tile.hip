@@ -28,6 +28,7 @@
  */
 #include "conv_tile.hpp"
 #include "mfma_core.hpp"
+#include <type_traits>
 
 namespace
 {
@@ -39,7 +40,8 @@ namespace
 	constexpr int HALO_MAX = 300; /* halo pixels that fit */
 	constexpr int HALO_BYTES = HALO_MAX * PIXEL_PITCH;
 	constexpr int FILTER_TILE = TILE_N * LDS_ROW;
-	constexpr int ROW_TABLE = HALO_BYTES + 2 * FILTER_TILE; /* offset of the table: GEMM row -> offset of its output pixel in the image, -1 if not stored */
+	constexpr int FILTER_RING = 3; /* filter tiles in LDS: two for the general k loop, a ring of three for the unrolled 3x3 one */
+	constexpr int ROW_TABLE = HALO_BYTES + FILTER_RING * FILTER_TILE; /* offset of the table: GEMM row -> offset of its output pixel in the image, -1 if not stored */
 	constexpr int TILE_LDS = ROW_TABLE + TILE_M * 4;
 	constexpr int HALO_FETCHES = (HALO_MAX * STEP_CHUNKS + 255) / 256; /* 16-byte chunks of the halo per work-item */
 	constexpr int FILTER_FETCHES = TILE_N * STEP_CHUNKS / 256;
@@ -55,7 +57,9 @@ namespace
 		int images;
 	};
 
-	template<typename TE, typename Epi>
+	/* FS = 3: the filter is 3 x 3 and the k loop is written out tap by tap (see the second half of the kernel); FS = 0: any
+	 * filter, general loop. */
+	template<typename TE, typename Epi, int FS>
 	__global__ __launch_bounds__(256, 2) void k_conv_tile(const TE *__restrict__ x, const TE *__restrict__ w, TileGeom g, Epi epi)
 	{
 		epi.pin();
@@ -300,6 +304,130 @@ namespace
 				}
 			}
 		};
+		if constexpr (FS > 0)
+		{
+			/*
+			 * 3 x 3 filters: the k loop written out, one channel slice = nine steps with nothing conditional inside.
+			 *
+			 * Why: loads return in order and the compiler counts them statically.  In the general loop below the halo and
+			 * residual prefetches sit behind run-time conditions, so every later wait for a filter load has to assume they
+			 * were not issued and ends up waiting for them as well: a whole HBM latency, twice per tile.  Written out, every
+			 * wait names exactly the loads it needs.  The filters go through a ring of three LDS tiles (tap % 3; nine taps
+			 * keep the phase) instead of two, which makes the tile of step t + 1 visible during step t: the operands of the
+			 * first 32-byte slab of the next step are read while the last MFMAs of the current one run, so the LDS latency
+			 * after each barrier is off the critical path too.
+			 *
+			 * Filters of step t: requested at the top of step t - 3 into register set t % 3, written to ring[t % 3] at the
+			 * end of step t - 2 (everyone has passed the barrier of step t - 2, so nobody reads step t - 3's tile any more),
+			 * visible from the barrier of step t - 1.
+			 */
+			constexpr int TAPS = FS * FS;
+			constexpr int SLABS = STEP_BYTES / 32;
+			constexpr int PREFETCH_TAP = 2;
+			static_assert(TAPS % FILTER_RING == 0, "the ring phase must be the same in every channel slice");
+			stash_filters(1, fr[1]);
+			const int row_pitch = g.HW * PIXEL_PITCH;
+			const int flip_base = g.flip ? (FS - 1) * (row_pitch + PIXEL_PITCH) : 0;
+			const int flip_sign = g.flip ? -1 : 1;
+			Chunk a[2][2], bq[2][2]; /* operands of two consecutive slabs; they live across steps */
+			auto read = [&](int tap, int slab, Chunk (&ra_)[2], Chunk (&rb_)[2]) __attribute__((always_inline))
+			{
+				const char *sa = halo + flip_base + flip_sign * ((tap / FS) * row_pitch + (tap % FS) * PIXEL_PITCH);
+				const char *sb = filt + (tap % FILTER_RING) * FILTER_TILE + b_off;
+#pragma unroll
+				for (int t = 0; t < 2; t++)
+				{
+					ra_[t].u = *reinterpret_cast<const uint4*>(sa + a_off[t] + slab * 32);
+					rb_[t].u = *reinterpret_cast<const uint4*>(sb + t * 32 * LDS_ROW + slab * 32);
+				}
+			};
+			auto fetch_filters_at = [&](int slice, int tap, uint4 (&r)[FILTER_FETCHES]) __attribute__((always_inline))
+			{
+				const int sl = tap >= TAPS ? slice + 1 : slice, tp = tap >= TAPS ? tap - TAPS : tap;
+				const unsigned int k_bytes = static_cast<unsigned int>(tp * g.C) * SZ + static_cast<unsigned int>(sl) * STEP_BYTES;
+				const bool exists = sl * KE + chunk_channel < g.C; /* false for every slice past the last */
+#pragma unroll
+				for (int f = 0; f < FILTER_FETCHES; f++)
+					r[f] = buffer_fetch(rw, exists ? filt_src[f] + k_bytes : OUT_OF_RANGE);
+			};
+			/* the residual through a buffer load: rows that are not stored ask for an out-of-range offset instead of being
+			 * skipped, so the number of loads in flight does not depend on the data */
+			constexpr bool RESIDUAL_BUFFER = RESIDUAL_AHEAD && sizeof(TE) == 2;
+			__amdgpu_buffer_rsrc_t rz = make_buffer(nullptr, 0);
+			if constexpr (RESIDUAL_BUFFER)
+				if (epi.z != nullptr)
+					rz = make_buffer(epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
+			auto fetch_residual_rows = [&]() __attribute__((always_inline))
+			{
+				if constexpr (RESIDUAL_BUFFER)
+				{
+#pragma unroll
+					for (int slot = 0; slot < Rows::slots; slot++)
+					{
+						const int e = row_table[Rows::row(slot)];
+						union
+						{
+							uint4 u;
+							decltype(residual[0].raw) p;
+						} cast;
+						cast.u = buffer_fetch(rz, (e >= 0 && kcol < g.K) ? static_cast<unsigned int>(e * g.K + kcol) * SZ : OUT_OF_RANGE);
+						residual[slot].raw = cast.p;
+					}
+				}
+			};
+			auto slice_steps = [&](int slice, auto is_last) __attribute__((always_inline))
+			{
+				constexpr bool LAST = decltype(is_last)::value;
+#pragma unroll
+				for (int tap = 0; tap < TAPS; tap++)
+				{
+					__syncthreads(); /* ring[(tap + 1) % 3] and, at tap 0, the halo are visible; everyone is done with the step before */
+					fetch_filters_at(slice, tap + 3, fr[tap % 3]);
+					if (tap == PREFETCH_TAP)
+					{
+						if constexpr (LAST)
+							fetch_residual_rows();
+						else
+							fetch_halo(slice + 1, hr);
+					}
+					if (tap == 0)
+						read(0, 0, a[0], bq[0]); /* the halo changed under the barrier above: nothing could be read ahead */
+#pragma unroll
+					for (int slab = 0; slab < SLABS; slab++)
+					{
+						if (slab + 1 < SLABS)
+							read(tap, slab + 1, a[(slab + 1) & 1], bq[(slab + 1) & 1]);
+						else if (tap + 1 < TAPS)
+							read(tap + 1, 0, a[0], bq[0]);
+						burst_priority(slab);
+#pragma unroll
+						for (int tm = 0; tm < 2; tm++)
+#pragma unroll
+							for (int tn = 0; tn < 2; tn++)
+								Mma<TE>::run(a[slab & 1][tm], bq[slab & 1][tn], acc[tm][tn]);
+						if (slab + 1 == SLABS)
+							__builtin_amdgcn_s_setprio(0);
+					}
+					/* one LDS read behind every MFMA */
+#pragma unroll
+					for (int i = 0; i < 4 * (SLABS - 1) + (tap + 1 < TAPS ? 4 : 0); i++)
+					{
+						__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+						__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+					}
+					stash_filters((tap + 2) % FILTER_RING, fr[(tap + 2) % FILTER_RING]);
+				}
+				if constexpr (!LAST)
+				{
+					__syncthreads(); /* nobody reads the old halo any more */
+					stash_halo(hr);
+				}
+			};
+			for (int slice = 0; slice + 1 < g.slices; slice++)
+				slice_steps(slice, std::false_type());
+			slice_steps(g.slices - 1, std::true_type());
+		}
+		else
 		for (int s = 0; s < total; s += 6)
 		{
 			step(s, 0, fr[0], fr[1]);
@@ -387,8 +515,11 @@ namespace avhip
 		const int64_t filter_blocks = (static_cast<int64_t>(s.K) + TILE_N - 1) / TILE_N;
 		if (blocks > 0x7FFFFFFFll || filter_blocks > 65535)
 			return false;
-		hipLaunchKernelGGL((k_conv_tile<TE, Epi>), dim3(static_cast<unsigned int>(blocks), static_cast<unsigned int>(filter_blocks)), dim3(256), 0, stream,
-				static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
+		const dim3 grid(static_cast<unsigned int>(blocks), static_cast<unsigned int>(filter_blocks));
+		if (s.R == 3 && s.S == 3)
+			hipLaunchKernelGGL((k_conv_tile<TE, Epi, 3>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
+		else
+			hipLaunchKernelGGL((k_conv_tile<TE, Epi, 0>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
 		return true;
 	}
 
