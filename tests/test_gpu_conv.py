@@ -147,6 +147,59 @@ def test_implicit_gemm_padding_value(oracle):
     assert oracle.rel_l2(got, want) < 1e-5
 
 
+# ---- the image-tile kernel: shapes that fill at least half of its 256-row tiles ----------------------------------------------
+TILE_CASES = [
+    dict(x=(3, 15, 15, 160), w=(72, 3, 3, 160), pad=(-1, -1)),            # several channel slices, the last partial; two filter blocks
+    dict(x=(2, 14, 13, 64), w=(64, 3, 3, 64), pad=(-1, -1), mode=1),      # flipped 3x3
+    dict(x=(2, 20, 21, 96), w=(40, 3, 3, 96), pad=(-1, -1)),              # several tiles per image, partial ones at the edges
+    dict(x=(2, 16, 15, 32), w=(16, 3, 3, 32), pad=(-2, -2)),              # full convolution: output larger than input
+    dict(x=(2, 15, 15, 64), w=(32, 5, 5, 64), pad=(-2, -2)),              # the general k loop (not 3x3)
+    dict(x=(2, 15, 14, 72), w=(24, 3, 1, 72), pad=(-1, 0), mode=1),       # three taps only, flipped
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", TILE_CASES, ids=[str(i) for i in range(len(TILE_CASES))])
+def test_tile_kernel_with_residual(oracle, dtype, case):
+    """Bias, residual (alpha2 != 1) and ReLU fused, and then the same with beta != 0 on top."""
+    g = h.rng(40)
+    x = h.rounded(oracle, g.standard_normal(case["x"]), dtype)
+    w = he(g, case["w"], dtype, oracle)
+    ys = out_shape(oracle, case)
+    b = g.uniform(-0.1, 0.1, ys[3]).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal(ys), dtype)
+    y0 = h.rounded(oracle, g.standard_normal(ys), dtype)
+    kw = dict(pad=case["pad"], mode=case.get("mode", 0))
+    a2 = float(np.float32(0.7))
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, bias=b, z=z, alpha2=a2, activation=cb.ACTIVATION_RELU, **kw)
+    want = oracle.conv2d(x, w, b, z, alpha2=a2, activation=oracle.RELU, **kw)
+    assert got.shape == want.shape
+    assert oracle.rel_l2(got, want) < BAR[dtype]
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, **kw)
+    assert oracle.rel_l2(got, oracle.conv2d(x, w, **kw)) < BAR[dtype]
+    be = float(np.float32(0.3))
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, bias=b, z=z, y0=y0, alpha2=a2, beta=be, activation=cb.ACTIVATION_RELU, **kw)
+    want = oracle.conv2d(x, w, b, z, y0, alpha2=a2, beta=be, activation=oracle.RELU, **kw)
+    assert oracle.rel_l2(got, want) < BAR[dtype]
+
+
+@pytest.mark.parametrize("case", TILE_CASES, ids=[str(i) for i in range(len(TILE_CASES))])
+def test_tile_kernel_int8_bit_exact(oracle, case):
+    g = h.rng(41)
+    x = g.integers(-127, 128, case["x"], dtype=np.int8)
+    w = g.integers(-127, 128, case["w"], dtype=np.int8)
+    K = case["w"][0]
+    b = g.integers(-2 ** 15, 2 ** 15, K).astype(np.int32)
+    kw = dict(pad=case["pad"], mode=case.get("mode", 0))
+    ys = out_shape(oracle, case)
+    got = h.conv_forward("implicit_gemm", x, w, ys, "i8", y_dtype="i32", bias=b, bias_dtype="i32", activation=cb.ACTIVATION_RELU, **kw)
+    np.testing.assert_array_equal(got, oracle.conv2d_i8(x, w, b, activation=cb.ACTIVATION_RELU, **kw))
+    if case.get("mode", 0) == 0:
+        scale = g.uniform(1e-4, 1e-3, K).astype(np.float32)
+        got = h.conv_forward("requant", x, w, ys, "i8", y_dtype="i8", bias=b, bias_dtype="i32", scale=scale, activation=cb.ACTIVATION_LINEAR, pad=case["pad"])
+        np.testing.assert_array_equal(got, oracle.requant_i8(oracle.conv2d_i8(x, w, b, pad=case["pad"]), scale))
+
+
 # ---- fused Winograd F(2x2, 3x3) ------------------------------------------------------------------------------------------
 WINOGRAD_BAR = {"f32": 1e-4, "f16": 2e-3, "bf16": 2e-3}
 
