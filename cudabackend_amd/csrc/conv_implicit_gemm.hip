@@ -22,6 +22,7 @@
 #include "conv_epilogue.hpp"
 #include "conv_pointwise.hpp"
 #include "conv_small.hpp"
+#include "conv_stem.hpp"
 #include "conv_tile.hpp"
 #include "mfma_core.hpp"
 
@@ -521,6 +522,9 @@ namespace
 		const int pixel_bytes = s.C * static_cast<int>(sizeof(TE));
 		if (pixel_bytes <= STEP_BYTES / 2 && s.R * s.S > 1 && fast_path_ok<TE>(s, 1, padding_value) && is_simple_activation(epi.activation) && (flags & 2) != 0)
 		{
+			/* a pixel of exactly 8 bytes and a small filter: operands straight into registers, no k loop */
+			if (conv_stem_launch<TE, Epi>(st, s, x, w, epi))
+				return 0;
 			int pb = 16;
 			while (pb > 1 && (pixel_bytes % pb != 0 || !aligned_to(x, pb) || !aligned_to(w, pb)))
 				pb /= 2;

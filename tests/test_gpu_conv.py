@@ -87,6 +87,12 @@ FEW_CHANNELS = [
     dict(x=(2, 8, 9, 12), w=(136, 3, 3, 12), pad=(-1, -1)),                                       # k spans several steps, two filter blocks
     dict(x=(1, 7, 7, 16), w=(16, 5, 5, 16), pad=(-2, -2)),
     dict(x=(1, 7, 7, 5), w=(16, 3, 3, 5), pad=(0, 0)),                                            # valid convolution, odd channel count
+    # 8-byte pixels (4 channels of a 16-bit type, 8 of int8) and at most 12 taps: the register-operand stem kernel
+    dict(x=(2, 13, 11, 4), w=(72, 3, 3, 4), pad=(-1, -1), mode=1),                                # flipped, second filter block partial
+    dict(x=(2, 14, 12, 4), w=(40, 2, 5, 4), pad=(0, -2), stride=(2, 1)),                          # ten taps, strided
+    dict(x=(2, 12, 12, 4), w=(16, 3, 4, 4), pad=(-2, -3), dilation=(2, 2)),                       # twelve taps, dilated
+    dict(x=(2, 13, 11, 8), w=(72, 3, 3, 8), pad=(-1, -1), mode=1),
+    dict(x=(3, 14, 12, 8), w=(48, 4, 3, 8), pad=(-1, -1), stride=(1, 2)),
 ]
 
 
