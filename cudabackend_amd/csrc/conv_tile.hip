@@ -90,7 +90,6 @@ namespace
 		constexpr int W = Epi::wide; /* filters per work-item in the epilogue: one 16-byte store each */
 		const int kcol = k0 + drain_column<1, W>();
 		typename Epi::template ColumnsT<W> columns;
-		epi.load_columns(kcol, columns);
 
 		const __amdgpu_buffer_rsrc_t rx = make_buffer(x, static_cast<unsigned int>(g.images) * g.H * g.W * g.C * SZ);
 		const __amdgpu_buffer_rsrc_t rw = make_buffer(w, static_cast<unsigned int>(g.K) * g.R * g.S * g.C * SZ);
@@ -153,29 +152,41 @@ namespace
 		fetch_filters(fr[1]);
 		fetch_filters(fr[2]);
 		/* where this work-item's halo chunks come from (slice 0).  Integer division by a run-time divisor costs about thirty
-		 * instructions: the work-item divides once and then walks. */
+		 * instructions and a 32-bit multiply four issue slots: the work-item divides once and then walks, position and byte
+		 * offset alike (the offset of a pixel outside the image is never used; inside the image it is below 2 GiB and the
+		 * additions are exact modulo 2^32). */
 		{
 			constexpr int STRIDE = 256 / STEP_CHUNKS; /* halo pixels between two fetches of a work-item */
 			const int dy = STRIDE / g.HW, dx = STRIDE - dy * g.HW;
+			const unsigned int pixel_bytes = static_cast<unsigned int>(g.C) * SZ, line_bytes = static_cast<unsigned int>(g.W) * pixel_bytes;
+			const unsigned int step_bytes = dy * line_bytes + dx * pixel_bytes, wrap_bytes = line_bytes - g.HW * pixel_bytes;
 			int h = tid / STEP_CHUNKS;
-			int hy = h / g.HW, hx = h - hy * g.HW;
+			const int hy = h / g.HW;
+			int hx = h - hy * g.HW;
+			int ih = oh0 + g.pad_h + hy, iw = ow0 + g.pad_w + hx;
+			unsigned int offset = static_cast<unsigned int>((n * g.H + ih) * g.W + iw) * pixel_bytes + static_cast<unsigned int>(chunk_channel) * SZ;
 #pragma unroll
 			for (int f = 0; f < HALO_FETCHES; f++)
 			{
-				const int ih = oh0 + g.pad_h + hy, iw = ow0 + g.pad_w + hx;
-				const bool inside = (h < halo_pixels) & (ih >= 0) & (ih < g.H) & (iw >= 0) & (iw < g.W);
-				halo_src[f] = inside ? static_cast<unsigned int>(((n * g.H + ih) * g.W + iw) * g.C + chunk_channel) * SZ : OUT_OF_RANGE;
+				const bool inside = (h < halo_pixels) & (static_cast<unsigned int>(ih) < static_cast<unsigned int>(g.H))
+						& (static_cast<unsigned int>(iw) < static_cast<unsigned int>(g.W));
+				halo_src[f] = inside ? offset : OUT_OF_RANGE;
 				h += STRIDE;
-				hy += dy;
+				ih += dy;
+				iw += dx;
 				hx += dx;
+				offset += step_bytes;
 				if (hx >= g.HW)
 				{
 					hx -= g.HW;
-					hy++;
+					iw -= g.HW;
+					ih++;
+					offset += wrap_bytes;
 				}
 			}
 		}
 		fetch_halo(0, hr);
+		epi.load_columns(kcol, columns); /* needed in the epilogue only: behind everything the first MFMA waits for */
 		int *row_table = reinterpret_cast<int*>(lds + ROW_TABLE);
 		{
 			/* GEMM row -> offset of its output pixel inside the image, in pixels; -1 for rows that are not stored */
