@@ -116,14 +116,14 @@ namespace avhip
 				t[q] = RELU ? __builtin_fmaxf(r, 0.0f) : r;
 			}
 		}
-		/* idx: element index of (pixel, filter k) in y and z, for callers that keep it cheaper than p * K + k */
-		template<int ACT, bool VEC = false, int W = 4>
-		__device__ __forceinline__ void store_at(int64_t idx, int k, const float (&v)[W], const ColumnsT<W> &c, const Residual<W> *fetched = nullptr) const
+		/* The arithmetic of store_at without its store.  `readable`: the run exists in y and z (callers that store
+		 * unconditionally compute rows past the end of the tensor on zeros). */
+		template<int ACT, bool VEC, int W>
+		__device__ __forceinline__ void values(float (&t)[W], bool readable, int64_t idx, int k, const float (&v)[W], const ColumnsT<W> &c,
+				const Residual<W> *fetched) const
 		{
-			static_assert(VEC || W == 4, "`vec` vouches for 4-element vectors only; wider runs are for callers that checked");
 			const bool vec = VEC || this->vec;
 			const int valid = VEC ? W : K - k;
-			float t[W];
 			/* ReLU sits in the same straight-line block as the multiply-add that feeds it: the compiler then knows the
 			 * operand is an arithmetic result (never a signalling NaN) and emits one bare v_max_f32 per element */
 			const bool relu = ACT == ACT_SIMPLE && activation == ACT_RELU;
@@ -136,8 +136,14 @@ namespace avhip
 					for (int q = 0; q < W; q++)
 						zv[q] = Traits<TE>::load(fetched->raw.v[q]);
 				}
-				else
+				else if (readable)
 					load_vec<TE, W, float>(z + idx, valid, zv, vec);
+				else
+				{
+#pragma unroll
+					for (int q = 0; q < W; q++)
+						zv[q] = 0.0f;
+				}
 				if (relu)
 					combine<true, true, W>(t, v, c, zv);
 				else
@@ -156,7 +162,7 @@ namespace avhip
 				for (int q = 0; q < W; q++)
 					t[q] = activation_forward<float>(activation, t[q]);
 			}
-			if (beta != 0.0f)
+			if (beta != 0.0f && readable)
 			{
 				float yv[W];
 				load_vec<TE, W, float>(y + idx, valid, yv, vec);
@@ -164,7 +170,39 @@ namespace avhip
 				for (int q = 0; q < W; q++)
 					t[q] += beta * yv[q];
 			}
-			store_vec<TE, W, float, VEC>(y + idx, valid, t, vec);
+		}
+		/* idx: element index of (pixel, filter k) in y and z, for callers that keep it cheaper than p * K + k */
+		template<int ACT, bool VEC = false, int W = 4>
+		__device__ __forceinline__ void store_at(int64_t idx, int k, const float (&v)[W], const ColumnsT<W> &c, const Residual<W> *fetched = nullptr) const
+		{
+			static_assert(VEC || W == 4, "`vec` vouches for 4-element vectors only; wider runs are for callers that checked");
+			float t[W];
+			values<ACT, VEC, W>(t, true, idx, k, v, c, fetched);
+			store_vec<TE, W, float, VEC>(y + idx, VEC ? W : K - k, t, VEC || this->vec);
+		}
+		/* For kernels that walk many tiles and must not have a store behind a condition (vector-memory operations complete in
+		 * order and are counted statically: after a conditional store every later wait for an older load also waits for the
+		 * store): the W results as 16 bytes handed to `sink` exactly once, whether or not the run exists; the caller's sink
+		 * drops runs that do not (a buffer store at an out-of-range offset).  LINEAR / RELU, whole aligned runs. */
+		static constexpr bool masked_stores = true;
+		static constexpr int out_bytes = sizeof(TE);
+		__device__ __forceinline__ char *out() const { return reinterpret_cast<char*>(y); }
+		template<int W, typename Sink>
+		__device__ __forceinline__ void store_masked(bool exists, int64_t idx, int k, const float (&v)[W], const ColumnsT<W> &c, const Sink &sink) const
+		{
+			static_assert(W * sizeof(TE) == 16, "one 16-byte run");
+			float t[W];
+			values<ACT_SIMPLE, true, W>(t, exists, idx, k, v, c, nullptr);
+			typedef unsigned int words_t __attribute__((ext_vector_type(4)));
+			union
+			{
+				Pack<TE, W> p;
+				words_t words;
+			} u;
+#pragma unroll
+			for (int q = 0; q < W; q++)
+				u.p.v[q] = Traits<TE>::store(t[q]);
+			sink(u.words);
 		}
 	};
 
@@ -258,6 +296,49 @@ namespace avhip
 		__device__ __forceinline__ void load_residual(int64_t, Residual<W>&) const
 		{
 		}
+		/* EXACT / REQUANT: act(sum + bias) in integer arithmetic */
+		template<int W>
+		__device__ __forceinline__ void integer_values(int (&t)[W], const int (&v)[W], const ColumnsT<W> &c) const
+		{
+			/* one v_max_i32 against a scalar either way (hidden from the optimiser, which would otherwise turn it back
+			 * into a maximum and a select per element) */
+			int floor = activation == ACT_RELU ? 0 : -2147483647 - 1;
+			keep_in_sgpr(floor);
+#pragma unroll
+			for (int q = 0; q < W; q++)
+			{
+				t[q] = v[q] + c.ibias[q];
+				t[q] = t[q] < floor ? floor : t[q];
+			}
+		}
+		/* REQUANT: sat_i8(rne(float(t) * scale)), four results per 32-bit word.
+		 * Clamping to the integers -128 and 127 commutes with rounding to an integer, so the product is clamped
+		 * first; adding 1.5 * 2^23 then rounds it to nearest even in the adder (the sum's unit in the last place is 1)
+		 * and leaves the two's-complement byte in the low 8 bits of the sum: no rint, no conversion.  Three byte
+		 * permutes gather four such bytes into a word. */
+		template<int W>
+		__device__ __forceinline__ void requantise(unsigned int (&words)[W / 4], const int (&t)[W], const ColumnsT<W> &c) const
+		{
+#pragma clang fp contract(off)
+#pragma unroll
+			for (int part = 0; part < W / 4; part++)
+			{
+				unsigned int bits[4];
+#pragma unroll
+				for (int q = 0; q < 4; q++)
+				{
+					const float product = static_cast<float>(t[4 * part + q]) * c.scale[4 * part + q];
+					const float rounded = __builtin_amdgcn_fmed3f(product, -128.0f, 127.0f) + 12582912.0f;
+					bits[q] = __builtin_bit_cast(unsigned int, rounded);
+				}
+				const unsigned int lo = __builtin_amdgcn_perm(bits[1], bits[0], 0x0c0c0400u);
+				const unsigned int hi = __builtin_amdgcn_perm(bits[3], bits[2], 0x0c0c0400u);
+				words[part] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+			}
+		}
+		/* no unconditional hand-over of runs (FloatEpilogue::store_masked) here: measured on the 1x1 layer of config 4 it
+		 * made the int32-output kernel 5 % slower and left the requantising one unchanged */
+		static constexpr bool masked_stores = false;
 		template<int ACT, bool VEC = false, int W = 4>
 		__device__ __forceinline__ void store_at(int64_t idx, int k, const int (&v)[W], const ColumnsT<W> &c, const Residual<W>* = nullptr) const
 		{
@@ -270,16 +351,7 @@ namespace avhip
 			if (MODE == I8_EXACT || MODE == I8_REQUANT)
 			{
 				int t[W];
-				/* one v_max_i32 against a scalar either way (hidden from the optimiser, which would otherwise turn it back
-				 * into a maximum and a select per element) */
-				int floor = activation == ACT_RELU ? 0 : -2147483647 - 1;
-				keep_in_sgpr(floor);
-#pragma unroll
-				for (int q = 0; q < W; q++)
-				{
-					t[q] = v[q] + c.ibias[q];
-					t[q] = t[q] < floor ? floor : t[q];
-				}
+				integer_values<W>(t, v, c);
 				/* whole runs leave as streaming vector stores: the kernel never reads y back, so the caches may drain it while
 				 * the kernel runs */
 				typedef typename Words<W / 4>::type words_t; /* W int8 values as 32-bit words */
@@ -306,31 +378,13 @@ namespace avhip
 				}
 				else
 				{
-					/* Clamping to the integers -128 and 127 commutes with rounding to an integer, so the product is clamped
-					 * first; adding 1.5 * 2^23 then rounds it to nearest even in the adder (the sum's unit in the last place is 1)
-					 * and leaves the two's-complement byte in the low 8 bits of the sum: no rint, no conversion.  Three byte
-					 * permutes gather four such bytes into a word. */
 					union
 					{
 						int8_t b[W];
 						unsigned int u[W / 4];
 						words_t w;
 					} o;
-#pragma unroll
-					for (int part = 0; part < W / 4; part++)
-					{
-						unsigned int bits[4];
-#pragma unroll
-						for (int q = 0; q < 4; q++)
-						{
-							const float product = static_cast<float>(t[4 * part + q]) * c.scale[4 * part + q];
-							const float rounded = __builtin_amdgcn_fmed3f(product, -128.0f, 127.0f) + 12582912.0f;
-							bits[q] = __builtin_bit_cast(unsigned int, rounded);
-						}
-						const unsigned int lo = __builtin_amdgcn_perm(bits[1], bits[0], 0x0c0c0400u);
-						const unsigned int hi = __builtin_amdgcn_perm(bits[3], bits[2], 0x0c0c0400u);
-						o.u[part] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-					}
+					requantise<W>(o.u, t, c);
 					int8_t *dst = static_cast<int8_t*>(y) + idx;
 					if (vec && valid >= W)
 						__builtin_nontemporal_store(o.w, reinterpret_cast<words_t*>(dst));

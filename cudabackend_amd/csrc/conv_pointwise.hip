@@ -36,7 +36,7 @@ namespace avhip
 		const int64_t pixels = static_cast<int64_t>(s.N) * s.H * s.W;
 		const int64_t row_blocks = (pixels + BLOCK_M - 1) / BLOCK_M, col_blocks = (static_cast<int64_t>(s.K) + BLOCK_N - 1) / BLOCK_N;
 		const int64_t tiles = row_blocks * col_blocks;
-		if (pixels >= (1ll << 31) - BLOCK_M || tiles >= (1ll << 31) - 1024 || s.K >= (1 << 24))
+		if (pixels >= (1ll << 31) - BLOCK_M || tiles >= (1ll << 31) - 1024 || s.K >= (1 << 22))
 			return false;
 		PersistentGeom g;
 		g.rows = static_cast<int>(pixels);

@@ -183,6 +183,36 @@ namespace
 			}
 			store_vec<TC, W, float, true>(c + idx, W, t, true); /* streaming: C is not read back by this kernel */
 		}
+		static constexpr bool masked_stores = true;
+		static constexpr int out_bytes = sizeof(TC);
+		__device__ __forceinline__ char *out() const { return reinterpret_cast<char*>(c); }
+		template<int W, typename Sink>
+		__device__ __forceinline__ void store_masked(bool exists, int64_t idx, int, const float (&v)[W], const ColumnsT<W>&, const Sink &sink) const
+		{
+			static_assert(W * sizeof(TC) == 16, "one 16-byte run");
+			float t[W];
+#pragma unroll
+			for (int q = 0; q < W; q++)
+				t[q] = alpha * v[q];
+			if (beta != 0.0f && exists)
+			{
+				float old[W];
+				load_vec<TC, W, float>(c + idx, W, old, true);
+#pragma unroll
+				for (int q = 0; q < W; q++)
+					t[q] += beta * old[q];
+			}
+			typedef unsigned int words_t __attribute__((ext_vector_type(4)));
+			union
+			{
+				Pack<TC, W> p;
+				words_t words;
+			} u;
+#pragma unroll
+			for (int q = 0; q < W; q++)
+				u.p.v[q] = Traits<TC>::store(t[q]);
+			sink(u.words);
+		}
 	};
 
 	template<typename TE, typename TC, int STEPS, int TM>
@@ -264,7 +294,7 @@ namespace
 			constexpr int TM = sizeof(TE) >= 4 ? 1 : 2;
 			constexpr int ROWS = 64 * TM;
 			/* whole 16-byte runs of C, rows of C a multiple of them apart */
-			if (N % Epi::wide != 0 || ldc % Epi::wide != 0 || sC % Epi::wide != 0 || !aligned_to(C, 16) || ldc >= (1 << 24))
+			if (N % Epi::wide != 0 || ldc % Epi::wide != 0 || sC % Epi::wide != 0 || !aligned_to(C, 16) || ldc >= (1 << 22))
 				return false;
 			const int64_t a_bytes = ((batch - 1) * sA + static_cast<int64_t>(M - 1) * lda + K) * static_cast<int64_t>(sizeof(TE));
 			const int64_t b_bytes = ((batch - 1) * sB + static_cast<int64_t>(N - 1) * ldb + K) * static_cast<int64_t>(sizeof(TE));

@@ -121,6 +121,19 @@ namespace avhip
 		const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(byte_offset), 0, 0);
 		return make_uint4(v[0], v[1], v[2], v[3]);
 	}
+	/* The store counterpart: 16 or 8 bytes at a 32-bit byte offset, non-temporal (the writing kernel never reads them back);
+	 * a store at OUT_OF_RANGE is dropped by the hardware, so "this row does not exist" needs no branch around the store. */
+	typedef __attribute__((__vector_size__(2 * sizeof(unsigned int)))) unsigned int u32x2_t;
+	__device__ inline void buffer_put(__amdgpu_buffer_rsrc_t rsrc, unsigned int byte_offset, unsigned int __attribute__((ext_vector_type(4))) words)
+	{
+		const u32x4_t v = { words.x, words.y, words.z, words.w };
+		__builtin_amdgcn_raw_buffer_store_b128(v, rsrc, static_cast<int>(byte_offset), 0, 2);
+	}
+	__device__ inline void buffer_put(__amdgpu_buffer_rsrc_t rsrc, unsigned int byte_offset, unsigned int __attribute__((ext_vector_type(2))) words)
+	{
+		const u32x2_t v = { words.x, words.y };
+		__builtin_amdgcn_raw_buffer_store_b64(v, rsrc, static_cast<int>(byte_offset), 0, 2);
+	}
 	template<typename TE>
 	__device__ inline uint4 splat_chunk(TE value, int valid)
 	{

@@ -18,7 +18,8 @@
  * them, so the workgroups that share a block of A rows run at the same time behind the same L2 and A comes from HBM once.
  *
  * The epilogue type provides: scalar_t, wide, ColumnsT<W>, pin(), load_columns(col, ColumnsT<1>&),
- * pick_columns(table, col, ColumnsT<W>&) and store_at<ACT_SIMPLE, true, W>(element index, col, values, columns).
+ * pick_columns(table, col, ColumnsT<W>&), store_at<ACT_SIMPLE, true, W>(element index, col, values, columns) and, when its
+ * masked_stores is set, store_masked<W>(exists, element index, col, values, columns, sink) with out_bytes and out().
  */
 #ifndef AVHIP_PERSISTENT_GEMM_HPP_
 #define AVHIP_PERSISTENT_GEMM_HPP_
@@ -42,7 +43,7 @@ namespace avhip
 		unsigned int a_batch, b_batch; /* bytes between consecutive batch members */
 		unsigned int a_bytes, b_bytes; /* extent of all of A and of B (below 2 GiB) */
 		int64_t c_batch; /* elements between batch members of C */
-		int c_pitch; /* elements between rows of C (below 2^24: 128 rows of it are a 32-bit product) */
+		int c_pitch; /* elements between rows of C (below 2^22: the byte offset of a tile's last row is a 32-bit product) */
 		int row_blocks, col_blocks; /* ceil(rows / tile rows), ceil(cols / 128) */
 		int tiles; /* batch * row_blocks * col_blocks */
 		int table_columns; /* columns whose constants are staged in LDS (cols, or 0 when the epilogue has none) */
@@ -216,6 +217,19 @@ namespace avhip
 			epi.load_columns(c, table[c]);
 		stash(0, ra[0], rb[0]);
 		fetch_a(ra[0]);
+		if constexpr (Epi::masked_stores)
+		{
+			/* The compiler counts the vector-memory operations in flight statically and, where two paths meet, assumes the
+			 * shorter queue.  The first tile is entered from here, every later one from behind the stores of the drain: as
+			 * many stores that go nowhere (empty buffer: dropped by the hardware) make the two queues equal, so the waits of
+			 * the tile loop allow the drain's stores to be in flight instead of waiting for them. */
+			const __amdgpu_buffer_rsrc_t nowhere = make_buffer(epi.out(), 0);
+			typedef unsigned int drain_words_t __attribute__((ext_vector_type(W * Epi::out_bytes / 4)));
+			const drain_words_t nothing = {};
+#pragma unroll
+			for (int i = 0; i < DrainRows<TM, 2, W>::slots; i++)
+				buffer_put(nowhere, OUT_OF_RANGE + 16u * i, nothing); /* distinct offsets, or the compiler keeps only the last */
+		}
 
 		const int col_in_tile = drain_column<2, W>();
 		for (int round = 0; tile_of(round) < g.tiles; round++)
@@ -242,16 +256,32 @@ namespace avhip
 			}
 			/* buffer 1 was multiplied last and is refilled only after the next barrier of the loop above: the accumulators
 			 * leave through it while buffer 0 already holds step 0 of the next tile */
-			const int64_t c0 = static_cast<int64_t>(t.batch) * g.c_batch + static_cast<int64_t>(t.row_block * ROWS) * g.c_pitch + col;
+			const int64_t c_tile = static_cast<int64_t>(t.batch) * g.c_batch + static_cast<int64_t>(t.row_block * ROWS) * g.c_pitch + t.col_block * BLOCK_N;
+			const int64_t c0 = c_tile + col_in_tile; /* element index of (first row of the tile, this work-item's first column) */
 			const int row0 = t.row_block * ROWS;
 			typename Epi::template ColumnsT<W> columns;
 			if (col < g.table_columns)
 				Epi::pick_columns(table, col, columns);
-			drain_tile<TE, TM, 2, W>(lds + 2 * LDS_TILE, acc, [&](int r, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
+			if constexpr (Epi::masked_stores)
 			{
-				if (row0 + r < g.rows && col < g.cols)
-					epi.template store_at<ACT_SIMPLE, true, W>(c0 + r * g.c_pitch, col, v, columns);
-			});
+				/* every work-item issues every store, rows and columns that do not exist at an out-of-range offset: a store
+				 * behind a condition would make each later wait for the next tile's operands wait for the stores as well */
+				const __amdgpu_buffer_rsrc_t rc = make_buffer(epi.out() + c_tile * Epi::out_bytes, 0x7FFFFFF0u);
+				drain_tile<TE, TM, 2, W>(lds + 2 * LDS_TILE, acc, [&](int r, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
+				{
+					const bool exists = row0 + r < g.rows && col < g.cols;
+					epi.template store_masked<W>(exists, c0 + r * g.c_pitch, col, v, columns, [&](auto words) __attribute__((always_inline))
+					{
+						buffer_put(rc, exists ? static_cast<unsigned int>(r * g.c_pitch + col_in_tile) * Epi::out_bytes : OUT_OF_RANGE, words);
+					});
+				});
+			}
+			else
+				drain_tile<TE, TM, 2, W>(lds + 2 * LDS_TILE, acc, [&](int r, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
+				{
+					if (row0 + r < g.rows && col < g.cols)
+						epi.template store_at<ACT_SIMPLE, true, W>(c0 + r * g.c_pitch, col, v, columns);
+				});
 		}
 	}
 
