@@ -180,6 +180,47 @@ def time_tower(hip, ctx, dtype, steps, warmup):
     return out
 
 
+def two_half_batch_chains(hip, dtype, steps):
+    """NOT the headline: what a caller gains by driving the same 256 images as two independent towers of 128 on two contexts
+    (two streams).  In one chain every convolution is one round of lock-stepped workgroups, so nothing overlaps the first
+    loads, the epilogue and the gap between dependent launches of a kernel; two chains fill those with each other's MFMAs.
+    Timed from an event on the first stream to an event the first stream records after waiting for the second."""
+    hip.rt.hipStreamWaitEvent.argtypes = [C.c_void_p, C.c_void_p, C.c_uint]
+    ctxs = [cb.Context(0), cb.Context(0)]
+    towers, graphs = [], []
+    for c in ctxs:
+        t = Tower(c, dtype, N=128)
+        t.step()
+        c.synchronize()
+        towers.append(t)
+        graphs.append(hip.capture(c.stream(), t.step))
+    s0, s1 = ctxs[0].stream(), ctxs[1].stream()
+
+    def run(passes):
+        for _ in range(passes):
+            hip.launch(graphs[0], s0)
+            hip.launch(graphs[1], s1)
+    run(3)
+    for c in ctxs:
+        c.synchronize()
+    e0, e1, joined = hip.event(), hip.event(), hip.event()
+    hip.record(e0, s0)
+    assert hip.rt.hipStreamWaitEvent(s1, e0, 0) == 0  # the second chain starts no earlier than the clock
+    run(steps)
+    hip.record(joined, s1)
+    assert hip.rt.hipStreamWaitEvent(s0, joined, 0) == 0
+    hip.record(e1, s0)
+    ms = hip.elapsed_ms(e0, e1) / steps
+    flops = 2 * towers[0].flops_step
+    for g in graphs:
+        hip.rt.hipGraphExecDestroy(g)
+    for t in towers:
+        t.close()
+    for c in ctxs:
+        c.close()
+    return {"ms_per_pass_of_256_images": ms, "tflops": flops / (ms * 1e-3) / 1e12}
+
+
 def time_calls(hip, ctx, fn, iters, warmup=3):
     """Average duration of one call of fn: ten calls are captured into a graph, the graph is replayed."""
     stream = ctx.stream()
@@ -436,6 +477,7 @@ def main():
         for other in ("f32", "bf16", "f16"):
             if other != args.dtype:
                 detail["tower_" + other] = time_tower(hip, ctx, other, max(3, args.steps // 2), 2)
+        detail["caller_level_two_chains_of_128"] = two_half_batch_chains(hip, args.dtype, args.steps)
         detail["int8_config4"] = int8_leg(hip, ctx, it)
         detail["nonfused_winograd_f32_F4"] = nonfused_stages(hip, ctx, "f32", "f32", 4, it)
         detail["nonfused_winograd_bf16_F2_fp16mat"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it)
