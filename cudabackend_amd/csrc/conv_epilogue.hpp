@@ -187,12 +187,17 @@ namespace avhip
 		static constexpr bool masked_stores = true;
 		static constexpr int out_bytes = sizeof(TE);
 		__device__ __forceinline__ char *out() const { return reinterpret_cast<char*>(y); }
+		/* 16-bit tensors: a caller that walks tiles may fetch the residual of a pass of rows ahead (Residual, one 16-byte run
+		 * each) and hand it in; the fp32 kernels have no registers left for that */
+		static constexpr bool residual_ahead = sizeof(TE) == 2;
+		__device__ __forceinline__ const char *residual() const { return reinterpret_cast<const char*>(z); }
 		template<int W, typename Sink>
-		__device__ __forceinline__ void store_masked(bool exists, int64_t idx, int k, const float (&v)[W], const ColumnsT<W> &c, const Sink &sink) const
+		__device__ __forceinline__ void store_masked(bool exists, int64_t idx, int k, const float (&v)[W], const ColumnsT<W> &c, const Sink &sink,
+				const Residual<W> *fetched = nullptr) const
 		{
 			static_assert(W * sizeof(TE) == 16, "one 16-byte run");
 			float t[W];
-			values<ACT_SIMPLE, true, W>(t, exists, idx, k, v, c, nullptr);
+			values<ACT_SIMPLE, true, W>(t, exists, idx, k, v, c, fetched);
 			typedef unsigned int words_t __attribute__((ext_vector_type(4)));
 			union
 			{

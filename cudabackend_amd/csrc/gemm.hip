@@ -184,6 +184,7 @@ namespace
 			store_vec<TC, W, float, true>(c + idx, W, t, true); /* streaming: C is not read back by this kernel */
 		}
 		static constexpr bool masked_stores = true;
+		static constexpr bool residual_ahead = false;
 		static constexpr int out_bytes = sizeof(TC);
 		__device__ __forceinline__ char *out() const { return reinterpret_cast<char*>(c); }
 		template<int W, typename Sink>

@@ -314,8 +314,10 @@ namespace avhip
 			return (rl >> 5) * (TM * 32) + tm * 32 + (rl & 31);
 		}
 	};
-	template<typename TE, int TM, int WAVES_N, int CPL = 4, typename F>
-	__device__ __forceinline__ void drain_tile(char *lds, const typename Mma<TE>::acc_t (&acc)[TM][2], const F &f)
+	/* `before_pass(tm)` runs ahead of the LDS hand-over of pass tm: the place to request per-row data (a residual) whose
+	 * latency the hand-over then hides */
+	template<typename TE, int TM, int WAVES_N, int CPL = 4, typename F, typename P>
+	__device__ __forceinline__ void drain_tile(char *lds, const typename Mma<TE>::acc_t (&acc)[TM][2], const F &f, const P &before_pass)
 	{
 		typedef typename Mma<TE>::scalar_t S;
 		typedef DrainShape<WAVES_N, CPL> D;
@@ -332,6 +334,7 @@ namespace avhip
 #pragma unroll
 		for (int tm = 0; tm < TM; tm++)
 		{
+			before_pass(tm);
 			__syncthreads();
 #pragma unroll
 			for (int tn = 0; tn < 2; tn++)
@@ -361,6 +364,11 @@ namespace avhip
 		}
 	}
 
+	template<typename TE, int TM, int WAVES_N, int CPL = 4, typename F>
+	__device__ __forceinline__ void drain_tile(char *lds, const typename Mma<TE>::acc_t (&acc)[TM][2], const F &f)
+	{
+		drain_tile<TE, TM, WAVES_N, CPL>(lds, acc, f, [](int) {});
+	}
 	/*
 	 * The same hand-over for workgroups whose four wavefronts are stacked (each owns TM 32-row tiles by 64 columns, the
 	 * workgroup (4 * TM * 32) rows by 64 columns), without workgroup barriers after the first: a wavefront passes its own

@@ -267,14 +267,49 @@ namespace avhip
 				/* every work-item issues every store, rows and columns that do not exist at an out-of-range offset: a store
 				 * behind a condition would make each later wait for the next tile's operands wait for the stores as well */
 				const __amdgpu_buffer_rsrc_t rc = make_buffer(epi.out() + c_tile * Epi::out_bytes, 0x7FFFFFF0u);
-				drain_tile<TE, TM, 2, W>(lds + 2 * LDS_TILE, acc, [&](int r, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
+				auto run_offset = [&](int r) __attribute__((always_inline))
 				{
-					const bool exists = row0 + r < g.rows && col < g.cols;
-					epi.template store_masked<W>(exists, c0 + r * g.c_pitch, col, v, columns, [&](auto words) __attribute__((always_inline))
+					return (row0 + r < g.rows && col < g.cols) ? static_cast<unsigned int>(r * g.c_pitch + col_in_tile) * Epi::out_bytes : OUT_OF_RANGE;
+				};
+				if constexpr (Epi::residual_ahead)
+				{
+					/* the residual of the rows of a pass is requested before the pass goes through LDS, unconditionally (no
+					 * residual: an empty buffer), instead of row by row between the stores */
+					typedef DrainRows<TM, 2, W> Rows;
+					const bool has_z = epi.residual() != nullptr;
+					const __amdgpu_buffer_rsrc_t rz = make_buffer(has_z ? epi.residual() + c_tile * Epi::out_bytes : nullptr, has_z ? 0x7FFFFFF0u : 0u);
+					typename Epi::template Residual<W> residual[Rows::iterations];
+					drain_tile<TE, TM, 2, W>(lds + 2 * LDS_TILE, acc, [&](int r, const typename Epi::scalar_t (&v)[W], int slot) __attribute__((always_inline))
 					{
-						buffer_put(rc, exists ? static_cast<unsigned int>(r * g.c_pitch + col_in_tile) * Epi::out_bytes : OUT_OF_RANGE, words);
+						const unsigned int offset = run_offset(r);
+						epi.template store_masked<W>(offset != OUT_OF_RANGE, c0 + r * g.c_pitch, col, v, columns, [&](auto words) __attribute__((always_inline))
+						{
+							buffer_put(rc, offset, words);
+						}, &residual[slot % Rows::iterations]);
+					}, [&](int tm) __attribute__((always_inline))
+					{
+#pragma unroll
+						for (int it = 0; it < Rows::iterations; it++)
+						{
+							union
+							{
+								uint4 u;
+								decltype(residual[0].raw) p;
+							} cast;
+							cast.u = buffer_fetch(rz, run_offset(Rows::row(tm * Rows::iterations + it)));
+							residual[it].raw = cast.p;
+						}
 					});
-				});
+				}
+				else
+					drain_tile<TE, TM, 2, W>(lds + 2 * LDS_TILE, acc, [&](int r, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
+					{
+						const unsigned int offset = run_offset(r);
+						epi.template store_masked<W>(offset != OUT_OF_RANGE, c0 + r * g.c_pitch, col, v, columns, [&](auto words) __attribute__((always_inline))
+						{
+							buffer_put(rc, offset, words);
+						});
+					});
 			}
 			else
 				drain_tile<TE, TM, 2, W>(lds + 2 * LDS_TILE, acc, [&](int r, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
