@@ -52,6 +52,7 @@ namespace
 		int H, W, C, K, R, S, Ho, Wo, pad_h, pad_w, flip;
 		int TH, TW; /* output tile */
 		int HH, HW; /* halo = (TH + R - 1) x (TW + S - 1) */
+		unsigned int hw_magic; /* 2^20 / HW + 1: (v * hw_magic) >> 20 == v / HW while v * HW < 2^20 */
 		int tiles_h, tiles_w;
 		int slices; /* 128-byte channel slices */
 		int images;
@@ -80,11 +81,18 @@ namespace
 		const int part = tid % STEP_CHUNKS;
 		const int chunk_channel = part * E;
 
+		/* Everything up to the first halo request is latency the matrix cores sit through: no division on that path when the
+		 * tile is the whole image, and divisions by the halo width as a multiplication (hw_magic). */
 		int b = static_cast<int>(xcd_block(blockIdx.x, gridDim.x)); /* tiles of an image share halo pixels: one XCD, one L2 */
-		const int tw = b % g.tiles_w;
-		b /= g.tiles_w;
-		const int th = b % g.tiles_h;
-		const int n = b / g.tiles_h;
+		int tw = 0, th = 0, n = b;
+		if (g.tiles_w * g.tiles_h != 1)
+		{
+			tw = b % g.tiles_w;
+			b /= g.tiles_w;
+			th = b % g.tiles_h;
+			n = b / g.tiles_h;
+		}
+		auto over_halo_width = [&](int v) { return static_cast<int>((static_cast<unsigned int>(v) * g.hw_magic) >> 20); }; /* v / HW for v * HW < 2^20 */
 		const int oh0 = th * g.TH, ow0 = tw * g.TW;
 		const int k0 = blockIdx.y * TILE_N;
 		constexpr int W = Epi::wide; /* filters per work-item in the epilogue: one 16-byte store each */
@@ -157,12 +165,13 @@ namespace
 		 * additions are exact modulo 2^32). */
 		{
 			constexpr int STRIDE = 256 / STEP_CHUNKS; /* halo pixels between two fetches of a work-item */
-			const int dy = STRIDE / g.HW, dx = STRIDE - dy * g.HW;
+			const int dy = over_halo_width(STRIDE), dx = STRIDE - dy * g.HW;
 			const unsigned int pixel_bytes = static_cast<unsigned int>(g.C) * SZ, line_bytes = static_cast<unsigned int>(g.W) * pixel_bytes;
 			const unsigned int step_bytes = dy * line_bytes + dx * pixel_bytes, wrap_bytes = line_bytes - g.HW * pixel_bytes;
 			int h = tid / STEP_CHUNKS;
-			const int hy = h / g.HW;
+			const int hy = over_halo_width(h);
 			int hx = h - hy * g.HW;
+			const bool first_slice_exists = chunk_channel < g.C;
 			int ih = oh0 + g.pad_h + hy, iw = ow0 + g.pad_w + hx;
 			unsigned int offset = static_cast<unsigned int>((n * g.H + ih) * g.W + iw) * pixel_bytes + static_cast<unsigned int>(chunk_channel) * SZ;
 #pragma unroll
@@ -171,6 +180,7 @@ namespace
 				const bool inside = (h < halo_pixels) & (static_cast<unsigned int>(ih) < static_cast<unsigned int>(g.H))
 						& (static_cast<unsigned int>(iw) < static_cast<unsigned int>(g.W));
 				halo_src[f] = inside ? offset : OUT_OF_RANGE;
+				hr[f] = buffer_fetch(rx, first_slice_exists ? halo_src[f] : OUT_OF_RANGE); /* slice 0 goes out as soon as its address exists */
 				h += STRIDE;
 				ih += dy;
 				iw += dx;
@@ -185,12 +195,11 @@ namespace
 				}
 			}
 		}
-		fetch_halo(0, hr);
 		epi.load_columns(kcol, columns); /* needed in the epilogue only: behind everything the first MFMA waits for */
 		int *row_table = reinterpret_cast<int*>(lds + ROW_TABLE);
 		{
 			/* GEMM row -> offset of its output pixel inside the image, in pixels; -1 for rows that are not stored */
-			const int py = tid / g.HW, px = tid - py * g.HW;
+			const int py = over_halo_width(tid), px = tid - py * g.HW;
 			const int oh = oh0 + py, ow = ow0 + px;
 			row_table[tid] = (py < g.TH && px < g.TW && oh < g.Ho && ow < g.Wo) ? oh * g.Wo + ow : -1;
 		}
@@ -512,6 +521,7 @@ namespace avhip
 		g.flip = s.mode != 0 ? 1 : 0;
 		g.HH = g.TH + s.R - 1;
 		g.HW = g.TW + s.S - 1;
+		g.hw_magic = (1u << 20) / static_cast<unsigned int>(g.HW) + 1u; /* HW <= 300 and the dividends are below 320 */
 		g.tiles_h = (s.Ho + g.TH - 1) / g.TH;
 		g.tiles_w = (s.Wo + g.TW - 1) / g.TW;
 		g.slices = (s.C * static_cast<int>(sizeof(TE)) + STEP_BYTES - 1) / STEP_BYTES;
