@@ -187,6 +187,29 @@ namespace avhip
 		static constexpr bool masked_stores = true;
 		static constexpr int out_bytes = sizeof(TE);
 		__device__ __forceinline__ char *out() const { return reinterpret_cast<char*>(y); }
+		/* The same hand-over with everything about the call decided at compile time (ReLU or not, residual or not, beta = 0,
+		 * the residual already fetched): no branch at all, for epilogues that run eight of these per work-item back to back
+		 * and are otherwise paced by the branches between them. */
+		template<bool RELU, bool HAS_Z, int W, typename Sink>
+		__device__ __forceinline__ void store_fast(const float (&v)[W], const ColumnsT<W> &c, const Residual<W> &fetched, const Sink &sink) const
+		{
+			static_assert(W * sizeof(TE) == 16, "one 16-byte run");
+			float t[W], zv[W];
+#pragma unroll
+			for (int q = 0; q < W; q++)
+				zv[q] = HAS_Z ? Traits<TE>::load(fetched.raw.v[q]) : 0.0f;
+			combine<RELU, HAS_Z, W>(t, v, c, zv);
+			typedef unsigned int words_t __attribute__((ext_vector_type(4)));
+			union
+			{
+				Pack<TE, W> p;
+				words_t words;
+			} u;
+#pragma unroll
+			for (int q = 0; q < W; q++)
+				u.p.v[q] = Traits<TE>::store(t[q]);
+			sink(u.words);
+		}
 		/* 16-bit tensors: a caller that walks tiles may fetch the residual of a pass of rows ahead (Residual, one 16-byte run
 		 * each) and hand it in; the fp32 kernels have no registers left for that */
 		static constexpr bool residual_ahead = sizeof(TE) == 2;

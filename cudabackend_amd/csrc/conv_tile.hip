@@ -458,6 +458,38 @@ namespace
 			step(s + 5, 1, fr[2], fr[0]);
 		}
 
+		if constexpr (std::is_same<Epi, FloatEpilogue<TE>>::value && sizeof(TE) == 2)
+		{
+			/* 16-bit tensors with beta = 0: the epilogue without a single branch.  Which of the four forms (ReLU, residual) is
+			 * decided once, rows that are not stored go to an out-of-range offset of a buffer over this image of y, and the
+			 * eight runs of a work-item can be scheduled into each other. */
+			if (epi.beta == 0.0f)
+			{
+				const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
+				auto drain = [&](auto relu, auto has_z) __attribute__((always_inline))
+				{
+					drain_tile_private<TE, 2, W>(lds, acc, [&](int row, const float (&v)[W], int slot) __attribute__((always_inline))
+					{
+						const int e = row_table[row];
+						const unsigned int offset = (e >= 0 && kcol < g.K) ? static_cast<unsigned int>(e * g.K + kcol) * SZ : OUT_OF_RANGE;
+						epi.template store_fast<decltype(relu)::value, decltype(has_z)::value, W>(v, columns, residual[slot], [&](auto words) __attribute__((always_inline))
+						{
+							buffer_put(ry, offset, words);
+						});
+					});
+				};
+				const bool relu = epi.activation == ACT_RELU, has_z = epi.z != nullptr;
+				if (relu && has_z)
+					drain(std::true_type(), std::true_type());
+				else if (relu)
+					drain(std::true_type(), std::false_type());
+				else if (has_z)
+					drain(std::false_type(), std::true_type());
+				else
+					drain(std::false_type(), std::false_type());
+				return;
+			}
+		}
 		drain_tile_private<TE, 2, W>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[W], int slot) __attribute__((always_inline))
 		{
 			const int e = row_table[row];
