@@ -346,19 +346,20 @@ namespace avhip
 			__syncthreads();
 			/* all LDS reads of the pass first, then the stores: the reads are independent and overlap */
 			constexpr int ITERS = D::rows_per_pass / ROW_STEP;
-			Pack<S, 4> vals[ITERS][CPL / 4];
+			typedef S quad_t __attribute__((ext_vector_type(4))); /* a true vector type keeps the 16-byte LDS reads whole */
+			quad_t vals[ITERS][CPL / 4];
 #pragma unroll
 			for (int it = 0; it < ITERS; it++)
 #pragma unroll
 				for (int part = 0; part < CPL / 4; part++)
-					vals[it][part] = *reinterpret_cast<const Pack<S, 4>*>(sm + (tid / D::threads_per_row + it * ROW_STEP) * D::pitch + col + 4 * part);
+					vals[it][part] = *reinterpret_cast<const quad_t*>(sm + (tid / D::threads_per_row + it * ROW_STEP) * D::pitch + col + 4 * part);
 #pragma unroll
 			for (int it = 0; it < ITERS; it++)
 			{
 				S v[CPL];
 #pragma unroll
 				for (int q = 0; q < CPL; q++)
-					v[q] = vals[it][q / 4].v[q % 4];
+					v[q] = vals[it][q / 4][q % 4];
 				f(DrainRows<TM, WAVES_N, CPL>::row(tm * ITERS + it), v, tm * ITERS + it);
 			}
 		}
@@ -416,12 +417,15 @@ namespace avhip
 			/* what other lanes of this wavefront wrote is read next: LDS serves a wavefront's accesses in order, the fence keeps
 			 * the compiler from reordering them */
 			__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-			Pack<S, 4> vals[D::iterations][CPL / 4];
+			/* read back as 16-byte vectors (a true vector type: a struct of four is taken apart by the compiler and put back
+			 * together as 12 + 8 + 8 + 4 bytes) */
+			typedef S quad_t __attribute__((ext_vector_type(4)));
+			quad_t vals[D::iterations][CPL / 4];
 #pragma unroll
 			for (int it = 0; it < D::iterations; it++)
 #pragma unroll
 				for (int part = 0; part < CPL / 4; part++)
-					vals[it][part] = *reinterpret_cast<const Pack<S, 4>*>(sm + (lane / D::threads_per_row + it * D::rows_per_sweep) * D::pitch + col + 4 * part);
+					vals[it][part] = *reinterpret_cast<const quad_t*>(sm + (lane / D::threads_per_row + it * D::rows_per_sweep) * D::pitch + col + 4 * part);
 			__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront"); /* the next pass overwrites what was just read */
 #pragma unroll
 			for (int it = 0; it < D::iterations; it++)
@@ -429,7 +433,7 @@ namespace avhip
 				S v[CPL];
 #pragma unroll
 				for (int q = 0; q < CPL; q++)
-					v[q] = vals[it][q / 4].v[q % 4];
+					v[q] = vals[it][q / 4][q % 4];
 				f(D::row(tm * D::iterations + it), v, tm * D::iterations + it);
 			}
 		}
