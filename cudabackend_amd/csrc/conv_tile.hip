@@ -198,10 +198,10 @@ namespace
 		epi.load_columns(kcol, columns); /* needed in the epilogue only: behind everything the first MFMA waits for */
 		int *row_table = reinterpret_cast<int*>(lds + ROW_TABLE);
 		{
-			/* GEMM row -> offset of its output pixel inside the image, in pixels; -1 for rows that are not stored */
+			/* GEMM row -> offset of its output pixel inside the image of y, in elements; -1 for rows that are not stored */
 			const int py = over_halo_width(tid), px = tid - py * g.HW;
 			const int oh = oh0 + py, ow = ow0 + px;
-			row_table[tid] = (py < g.TH && px < g.TW && oh < g.Ho && ow < g.Wo) ? oh * g.Wo + ow : -1;
+			row_table[tid] = (py < g.TH && px < g.TW && oh < g.Ho && ow < g.Wo) ? (oh * g.Wo + ow) * g.K : -1; /* times K here, once, not in every use */
 		}
 
 		/* MFMA operand addresses: lane l supplies row (l % 32) of a 32-row tile and k-chunk (l / 32) */
@@ -286,7 +286,7 @@ namespace
 			{
 				const int e = row_table[Rows::row(slot)];
 				if (e >= 0 && kcol < g.K)
-					epi.load_residual(image_base + e * g.K, residual[RESIDUAL_AHEAD ? slot : 0]);
+					epi.load_residual(image_base + e, residual[RESIDUAL_AHEAD ? slot : 0]);
 			}
 		};
 
@@ -390,7 +390,7 @@ namespace
 							uint4 u;
 							decltype(residual[0].raw) p;
 						} cast;
-						cast.u = buffer_fetch(rz, (e >= 0 && kcol < g.K) ? static_cast<unsigned int>(e * g.K + kcol) * SZ : OUT_OF_RANGE);
+						cast.u = buffer_fetch(rz, (e >= 0 && kcol < g.K) ? static_cast<unsigned int>(e + kcol) * SZ : OUT_OF_RANGE);
 						residual[slot].raw = cast.p;
 					}
 				}
@@ -471,7 +471,7 @@ namespace
 					drain_tile_private<TE, 2, W>(lds, acc, [&](int row, const float (&v)[W], int slot) __attribute__((always_inline))
 					{
 						const int e = row_table[row];
-						const unsigned int offset = (e >= 0 && kcol < g.K) ? static_cast<unsigned int>(e * g.K + kcol) * SZ : OUT_OF_RANGE;
+						const unsigned int offset = (e >= 0 && kcol < g.K) ? static_cast<unsigned int>(e + kcol) * SZ : OUT_OF_RANGE;
 						epi.template store_fast<decltype(relu)::value, decltype(has_z)::value, W>(v, columns, residual[slot], [&](auto words) __attribute__((always_inline))
 						{
 							buffer_put(ry, offset, words);
@@ -494,7 +494,7 @@ namespace
 		{
 			const int e = row_table[row];
 			if (e >= 0 && kcol < g.K)
-				epi.template store_at<ACT_SIMPLE, true, W>(image_base + e * g.K, kcol, v, columns, RESIDUAL_AHEAD ? &residual[slot] : nullptr);
+				epi.template store_at<ACT_SIMPLE, true, W>(image_base + e, kcol, v, columns, RESIDUAL_AHEAD ? &residual[slot] : nullptr);
 		});
 	}
 
