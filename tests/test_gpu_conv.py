@@ -206,6 +206,49 @@ def test_tile_kernel_int8_bit_exact(oracle, case):
         np.testing.assert_array_equal(got, oracle.requant_i8(oracle.conv2d_i8(x, w, b, pad=case["pad"]), scale))
 
 
+WALK_CASES = [
+    # more (image, tile) pairs than workgroups stay resident: several rounds of workgroups, several filter blocks
+    dict(x=(48, 30, 30, 32), w=(136, 3, 3, 32), pad=(-1, -1)),       # 3 filter blocks, 5 tiles per image, a partial last round
+    dict(x=(130, 15, 15, 64), w=(200, 3, 3, 64), pad=(-1, -1)),      # 4 filter blocks, one whole-image tile each
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("case", WALK_CASES, ids=[str(i) for i in range(len(WALK_CASES))])
+def test_tile_kernel_many_tiles(oracle, tiling, dtype, case):
+    if tiling != "workgroup_tiles":
+        pytest.skip("same kernel either way: the shape is far above the small-problem threshold")
+    g = h.rng(42)
+    x = h.rounded(oracle, g.standard_normal(case["x"]), dtype)
+    w = he(g, case["w"], dtype, oracle)
+    ys = out_shape(oracle, case)
+    b = g.uniform(-0.1, 0.1, ys[3]).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal(ys), dtype)
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, bias=b, z=z, activation=cb.ACTIVATION_RELU, pad=case["pad"])
+    want = oracle.conv2d(x, w, b, z, activation=oracle.RELU, pad=case["pad"])
+    assert oracle.rel_l2(got, want) < BAR[dtype]
+    # every image separately: a tile that went to the wrong place would hide in a global norm
+    per_image = [oracle.rel_l2(got[i], want[i]) for i in range(ys[0])]
+    assert max(per_image) < 2 * BAR[dtype], int(np.argmax(per_image))
+
+
+@pytest.mark.parametrize("case", WALK_CASES, ids=[str(i) for i in range(len(WALK_CASES))])
+def test_tile_kernel_many_tiles_int8(oracle, tiling, case):
+    if tiling != "workgroup_tiles":
+        pytest.skip("same kernel either way")
+    g = h.rng(43)
+    x = g.integers(-127, 128, case["x"], dtype=np.int8)
+    w = g.integers(-127, 128, case["w"], dtype=np.int8)
+    K = case["w"][0]
+    b = g.integers(-2 ** 15, 2 ** 15, K).astype(np.int32)
+    ys = out_shape(oracle, case)
+    got = h.conv_forward("implicit_gemm", x, w, ys, "i8", y_dtype="i32", bias=b, bias_dtype="i32", activation=cb.ACTIVATION_RELU, pad=case["pad"])
+    np.testing.assert_array_equal(got, oracle.conv2d_i8(x, w, b, activation=cb.ACTIVATION_RELU, pad=case["pad"]))
+    scale = g.uniform(1e-4, 1e-3, K).astype(np.float32)
+    got = h.conv_forward("requant", x, w, ys, "i8", y_dtype="i8", bias=b, bias_dtype="i32", scale=scale, activation=cb.ACTIVATION_LINEAR, pad=case["pad"])
+    np.testing.assert_array_equal(got, oracle.requant_i8(oracle.conv2d_i8(x, w, b, pad=case["pad"]), scale))
+
+
 # ---- fused Winograd F(2x2, 3x3) ------------------------------------------------------------------------------------------
 WINOGRAD_BAR = {"f32": 1e-4, "f16": 2e-3, "bf16": 2e-3}
 
