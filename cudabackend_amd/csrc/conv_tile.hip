@@ -402,14 +402,6 @@ namespace
 				for (int tap = 0; tap < TAPS; tap++)
 				{
 					__syncthreads(); /* ring[(tap + 1) % 3] and, at tap 0, the halo are visible; everyone is done with the step before */
-					fetch_filters_at(slice, tap + 3, fr[tap % 3]);
-					if (tap == PREFETCH_TAP)
-					{
-						if constexpr (LAST)
-							fetch_residual_rows();
-						else
-							fetch_halo(slice + 1, hr);
-					}
 					if (tap == 0)
 						read(0, 0, a[0], bq[0]); /* the halo changed under the barrier above: nothing could be read ahead */
 #pragma unroll
@@ -434,6 +426,15 @@ namespace
 					{
 						__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 						__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+					}
+					/* requests for later steps cost only issue slots: behind the MFMAs of this one */
+					fetch_filters_at(slice, tap + 3, fr[tap % 3]);
+					if (tap == PREFETCH_TAP)
+					{
+						if constexpr (LAST)
+							fetch_residual_rows();
+						else
+							fetch_halo(slice + 1, hr);
 					}
 					stash_filters((tap + 2) % FILTER_RING, fr[(tap + 2) % FILTER_RING]);
 				}
