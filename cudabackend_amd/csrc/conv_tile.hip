@@ -475,7 +475,7 @@ namespace
 						const unsigned int offset = (e >= 0 && kcol < g.K) ? static_cast<unsigned int>(e + kcol) * SZ : OUT_OF_RANGE;
 						epi.template store_fast<decltype(relu)::value, decltype(has_z)::value, W>(v, columns, residual[slot], [&](auto words) __attribute__((always_inline))
 						{
-							buffer_put(ry, offset, words);
+							buffer_put<STORE_STREAM_THROUGH>(ry, offset, words);
 						});
 					});
 				};
