@@ -390,7 +390,7 @@ namespace
 							uint4 u;
 							decltype(residual[0].raw) p;
 						} cast;
-						cast.u = buffer_fetch(rz, (e >= 0 && kcol < g.K) ? static_cast<unsigned int>(e + kcol) * SZ : OUT_OF_RANGE);
+						cast.u = buffer_fetch<2>(rz, (e >= 0 && kcol < g.K) ? static_cast<unsigned int>(e + kcol) * SZ : OUT_OF_RANGE);
 						residual[slot].raw = cast.p;
 					}
 				}

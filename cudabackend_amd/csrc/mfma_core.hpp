@@ -116,9 +116,10 @@ namespace avhip
 	{
 		return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
 	}
+	template<int POLICY = 0>
 	__device__ inline uint4 buffer_fetch(__amdgpu_buffer_rsrc_t rsrc, unsigned int byte_offset)
 	{
-		const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(byte_offset), 0, 0);
+		const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(byte_offset), 0, POLICY);
 		return make_uint4(v[0], v[1], v[2], v[3]);
 	}
 	/* The store counterpart: 16 or 8 bytes at a 32-bit byte offset, non-temporal (the writing kernel never reads them back);
