@@ -284,7 +284,7 @@ namespace avhip
 						const unsigned int offset = run_offset(r);
 						epi.template store_masked<W>(offset != OUT_OF_RANGE, c0 + r * g.c_pitch, col, v, columns, [&](auto words) __attribute__((always_inline))
 						{
-							buffer_put(rc, offset, words);
+							buffer_put<STORE_STREAM_THROUGH>(rc, offset, words);
 						}, &residual[slot % Rows::iterations]);
 					}, [&](int tm) __attribute__((always_inline))
 					{
@@ -307,7 +307,7 @@ namespace avhip
 						const unsigned int offset = run_offset(r);
 						epi.template store_masked<W>(offset != OUT_OF_RANGE, c0 + r * g.c_pitch, col, v, columns, [&](auto words) __attribute__((always_inline))
 						{
-							buffer_put(rc, offset, words);
+							buffer_put<STORE_STREAM_THROUGH>(rc, offset, words);
 						});
 					});
 			}
