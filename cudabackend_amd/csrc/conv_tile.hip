@@ -464,7 +464,8 @@ namespace
 			/* 16-bit tensors with beta = 0: the epilogue without a single branch.  Which of the four forms (ReLU, residual) is
 			 * decided once, rows that are not stored go to an out-of-range offset of a buffer over this image of y, and the
 			 * eight runs of a work-item can be scheduled into each other. */
-			if (epi.beta == 0.0f)
+			/* (an image of y must stay below the out-of-range marker, or a row that is not stored would land inside it) */
+			if (epi.beta == 0.0f && static_cast<int64_t>(g.Ho) * g.Wo * g.K * SZ < (1ll << 31))
 			{
 				const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
 				auto drain = [&](auto relu, auto has_z) __attribute__((always_inline))
