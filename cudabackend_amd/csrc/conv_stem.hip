@@ -14,6 +14,7 @@
  */
 #include "conv_stem.hpp"
 #include "mfma_core.hpp"
+#include <type_traits>
 
 namespace
 {
@@ -116,6 +117,33 @@ namespace
 				for (int tn = 0; tn < 2; tn++)
 					Mma<TE>::run(a[tm][s], b[tn][s], acc[tm][tn]);
 
+		if constexpr (std::is_same<Epi, FloatEpilogue<TE>>::value && sizeof(TE) == 2)
+		{
+			/* the usual first layer (16-bit tensors, no residual, beta = 0): no branch in the epilogue, rows past the end go to an
+			 * out-of-range offset of a buffer over the 256 pixels of this workgroup, runs are written through as they go */
+			if (epi.z == nullptr && epi.beta == 0.0f && g.K < (1 << 22))
+			{
+				constexpr unsigned int SZ = sizeof(TE);
+				const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + static_cast<int64_t>(p0) * g.K, 0x7FFFFFF0u);
+				auto drain = [&](auto relu) __attribute__((always_inline))
+				{
+					drain_tile_private<TE, 2, W>(lds, acc, [&](int row, const float (&v)[W], int) __attribute__((always_inline))
+					{
+						const unsigned int offset = (p0 + row < g.pixels && kcol < g.K) ? static_cast<unsigned int>(row * g.K + kcol) * SZ : OUT_OF_RANGE;
+						typename Epi::template Residual<W> none;
+						epi.template store_fast<decltype(relu)::value, false, W>(v, columns, none, [&](auto words) __attribute__((always_inline))
+						{
+							buffer_put<STORE_STREAM_THROUGH>(ry, offset, words);
+						});
+					});
+				};
+				if (epi.activation == ACT_RELU)
+					drain(std::true_type());
+				else
+					drain(std::false_type());
+				return;
+			}
+		}
 		drain_tile_private<TE, 2, W>(lds, acc, [&](int row, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
 		{
 			const int p = p0 + row;
