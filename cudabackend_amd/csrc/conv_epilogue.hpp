@@ -37,6 +37,8 @@ namespace avhip
 			return 0;
 		float r = rintf(v);
 		r = r < lo ? lo : r;
+		if (r >= 2147483648.0f) /* hi = 2^31 stands for INT32_MAX, which fp32 cannot hold */
+			return 2147483647;
 		r = r > hi ? hi : r;
 		return static_cast<int>(r);
 	}
@@ -449,7 +451,7 @@ namespace avhip
 						t = t + beta * yv;
 					}
 					if (MODE == I8_FLOAT_I32)
-						static_cast<int*>(y)[idx + q] = round_saturate(t, -2147483648.0f, 2147483520.0f);
+						static_cast<int*>(y)[idx + q] = round_saturate(t, -2147483648.0f, 2147483648.0f);
 					else if (MODE == I8_FLOAT_I8)
 						static_cast<int8_t*>(y)[idx + q] = static_cast<int8_t>(round_saturate(t, -128.0f, 127.0f));
 					else

@@ -16,8 +16,10 @@
  *                             delta-kernel / all-ones / linearity / 1x1==matmul invariants.
  *   orc_conv2d_i8             pinned: exact integer arithmetic against numpy int64 einsum and the
  *                             fp64 routine (exact for these magnitudes).
- *   orc_requant_i8            pinned by definition only (numpy restatement with np.rint); the
- *                             reference has no requantisation step: parity unpinned.
+ *   orc_requant_i8            pinned: hand-written table of exact products (ties to even, saturation at both
+ *                             ends, the int32 -> fp32 rounding of the sum, per-filter scale).  The reference has no
+ *                             requantisation step; the definition is the benchmark's:
+ *                             q = sat_i8(rne(float(sum + bias) * scale[k])), each step one fp32 rounding.
  *   orc_winograd_*_transform  pinned: A^T[(G g G^T) .* (B^T d B)]A == direct correlation to 1e-12
  *                             for every (m, r) table, partial tiles and offsets included.
  *   orc_winograd_gradient_transform, orc_winograd_update_transform
@@ -32,8 +34,14 @@
  *   orc_affine_forward        pinned: with weight 1 it is orc_add_bias (itself pinned); numpy broadcast form.
  *   orc_batchnorm_inference   pinned: torch.nn.functional.batch_norm(training=False) in fp64; equals
  *                             orc_affine_forward on the folded parameters.
- *   orc_conv2d_i8_float_epilogue  parity unpinned: the float epilogue on integer tensors follows
- *                             the header's prose convention only.
+ *   orc_conv2d_i8_float_epilogue  pinned: with alpha1 = 1 and integer-valued terms below 2^24 it equals the exact
+ *                             integer routine bit for bit (int32, int8 after clamping, fp32); hand-written cases for
+ *                             ties, saturation of int8 and int32, NaN, infinities, the separate fp32 roundings of
+ *                             product / bias / residual (a fused multiply-add or a wider intermediate fails them)
+ *                             and the order of the steps (every other order fails a case).
+ *                             Deviation, stated: the reference kernel stores the float through C's implicit
+ *                             conversion (toward zero, src/conv2d_implicit_gemm.cu:285); this build rounds to nearest
+ *                             even and saturates, as its cudaChangeType and the requantised output do.
  *
  * Reference lines followed (paths relative to the reference checkout):
  *   app/CudaBackend.cu:122-201               direct convolution loop nest, offset padding
@@ -197,7 +205,7 @@ static inline int32_t saturate_round(float v, int32_t lo, int32_t hi)
 	float r = nearbyintf(v); /* default rounding mode: nearest even */
 	if (r < (float) lo)
 		return lo;
-	if (r > (float) hi)
+	if (r >= (float) hi) /* (float) INT32_MAX is 2^31: everything from there up saturates */
 		return hi;
 	return (int32_t) r;
 }
@@ -245,7 +253,7 @@ void orc_conv2d_i8_float_epilogue(const int32_t *acc, const float *bias, const v
 				t = t + beta * yv;
 			}
 			if (out_kind == 0)
-				((int32_t*) y)[idx] = saturate_round(t, INT32_MIN, INT32_MAX - 127 /* largest fp32 below 2^31 */);
+				((int32_t*) y)[idx] = saturate_round(t, INT32_MIN, INT32_MAX);
 			else if (out_kind == 1)
 				((int8_t*) y)[idx] = (int8_t) saturate_round(t, -128, 127);
 			else

@@ -375,8 +375,8 @@ def test_int8_requantised_bit_exact(oracle, case):
 @pytest.mark.parametrize("y_dtype", ["i32", "i8", "f32"])
 def test_int8_float_epilogue(oracle, y_dtype):
     """The header's convention for integer tensors: cast the int32 sum to fp32, scale and add in fp32, round to nearest even
-    and saturate on store (include/Avocado/cuda_backend.h:43-49).  Parity unpinned in the reference; the oracle restates the
-    same sequence of single roundings, so the comparison is exact for LINEAR / RELU."""
+    and saturate on store (include/Avocado/cuda_backend.h:43-49, src/conv2d_implicit_gemm.cu:278-286,330-338).  The oracle's
+    sequence of single roundings is pinned by hand-written cases in test_oracle.py, so the comparison is exact for LINEAR / RELU."""
     g = h.rng(27)
     x = g.integers(-127, 128, (2, 6, 6, 64), dtype=np.int8)
     w = g.integers(-127, 128, (16, 3, 3, 64), dtype=np.int8)
@@ -394,6 +394,22 @@ def test_int8_float_epilogue(oracle, y_dtype):
         np.testing.assert_array_equal(np.asarray(got, dtype=np.float32), want)
     else:
         np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("y_dtype", ["i32", "i8"])
+def test_int8_float_epilogue_saturates(oracle, y_dtype):
+    """Scaled sums beyond the integer range clamp to the type's extremes (INT32_MAX although fp32 cannot hold it), ties go to even."""
+    g = h.rng(28)
+    x = g.integers(-127, 128, (2, 5, 5, 32), dtype=np.int8)
+    w = g.integers(-127, 128, (8, 3, 3, 32), dtype=np.int8)
+    acc = oracle.conv2d_i8(x, w, None)
+    np_dt = {"i32": np.int32, "i8": np.int8}[y_dtype]
+    for a1 in (0.5, 1.0e5 if y_dtype == "i32" else 0.01):
+        got = h.conv_forward("implicit_gemm", x, w, acc.shape, "i8", y_dtype=y_dtype, alpha1=a1)
+        want = oracle.conv2d_i8_float_epilogue(acc, None, None, np.zeros(acc.shape, np_dt), a1, 1.0, 0.0, oracle.LINEAR)
+        np.testing.assert_array_equal(got, want)
+    info = np.iinfo(np_dt)
+    assert want.max() == info.max and want.min() == info.min
 
 
 # ---- dispatcher and argument checking -----------------------------------------------------------------------------------

@@ -135,16 +135,170 @@ def test_int8_conv_is_exact(oracle):
     np.testing.assert_array_equal(s2, want[:, ::2, ::2, :].astype(np.int32))
 
 
-def test_requant_definition(oracle):
-    acc = RNG.integers(-2 ** 22, 2 ** 22, (50, 8)).astype(np.int32)
-    acc[0, :] = [0, 1, -1, 2 ** 30, -2 ** 30, 500, 1500, -1500]
-    scale = RNG.uniform(1e-4, 1e-3, 8).astype(np.float32)
-    scale[5:8] = 1e-3  # 500*1e-3 = 0.5 -> 0 (ties to even); 1.5 -> 2; -1.5 -> -2
-    q = oracle.requant_i8(acc, scale)
-    want = np.clip(np.rint(acc.astype(np.float32) * scale), -128, 127).astype(np.int8)
-    np.testing.assert_array_equal(q, want)
-    assert q[0, 3] == 127 and q[0, 4] == -128
-    assert q[0, 5] == 0 and q[0, 6] == 2 and q[0, 7] == -2
+def test_requant_hand_cases(oracle):
+    """q = sat_i8(rne(float(acc) * scale)), every expected value written out.  Scales are powers of two (or small
+    integers), so each product is exact and the expected value follows from the rounding rule alone."""
+    table = [  # acc, scale, q
+        (0, 2.0 ** -10, 0),
+        (512, 2.0 ** -10, 0),        # 0.5 ties to even
+        (1536, 2.0 ** -10, 2),       # 1.5 -> 2
+        (2560, 2.0 ** -10, 2),       # 2.5 -> 2
+        (3584, 2.0 ** -10, 4),       # 3.5 -> 4
+        (-512, 2.0 ** -10, 0),       # -0.5 -> -0
+        (-1536, 2.0 ** -10, -2),
+        (-2560, 2.0 ** -10, -2),
+        (513, 2.0 ** -10, 1),        # just above the tie
+        (-513, 2.0 ** -10, -1),
+        (1023, 2.0 ** -10, 1),       # 0.999 -> 1
+        (130048, 2.0 ** -10, 127),   # 127.0
+        (130560, 2.0 ** -10, 127),   # 127.5 -> 128 -> saturates
+        (-131072, 2.0 ** -10, -128),  # -128.0
+        (-131584, 2.0 ** -10, -128),  # -128.5 -> -128
+        (-132096, 2.0 ** -10, -128),  # -129 saturates
+        (2 ** 30, 2.0 ** -10, 127),
+        (-2 ** 30, 2.0 ** -10, -128),
+        (2 ** 31 - 1, 1.0, 127),
+        (-2 ** 31, 1.0, -128),
+        (16777217, 2.0 ** -18, 64),  # int32 -> fp32 rounds 2^24+1 to 2^24 first: 64.0 exactly
+        (100, 0.0, 0),
+        (7, 3.0, 21),
+        (-43, 3.0, -128),            # -129
+    ]
+    acc = np.array([[t[0] for t in table]], dtype=np.int64).astype(np.int32)
+    scale = np.array([t[1] for t in table], dtype=np.float32)
+    want = np.array([[t[2] for t in table]], dtype=np.int8)
+    np.testing.assert_array_equal(oracle.requant_i8(acc, scale), want)
+    # the scale belongs to the filter (last axis), not to the row
+    acc2 = np.array([[1024, 1024], [3072, 3072]], dtype=np.int32)
+    np.testing.assert_array_equal(oracle.requant_i8(acc2, np.array([2.0 ** -10, 2.0 ** -9], dtype=np.float32)), np.array([[1, 2], [3, 6]], dtype=np.int8))
+    # a non-trivial scale: 1e-3f = 0x3A83126F = 0.001000000047497451...; 500 * that = 0.50000002..., which fp32 rounds to 0.5 -> 0
+    assert np.float32(1e-3).view(np.uint32) == 0x3A83126F
+    np.testing.assert_array_equal(oracle.requant_i8(np.array([[500, 1500, -1500, 2500]], dtype=np.int32), np.full(4, 1e-3, dtype=np.float32)),
+                                  np.array([[0, 2, -2, 2]], dtype=np.int8))
+
+
+def _float_epilogue_1(oracle, acc, out_dtype, bias=None, z=None, y0=0, alpha1=1.0, alpha2=1.0, beta=0.0, activation=0):
+    """One element through the float epilogue of the integer convolution."""
+    a = np.array([[acc]], dtype=np.int32)
+    b = None if bias is None else np.array([bias], dtype=np.float32)
+    zz = None if z is None else np.array([[z]], dtype=out_dtype)
+    y = np.array([[y0]], dtype=out_dtype)
+    return oracle.conv2d_i8_float_epilogue(a, b, zz, y, alpha1, alpha2, beta, activation)[0, 0]
+
+
+def test_int8_float_epilogue_reduces_to_exact_integer_path(oracle):
+    """alpha1 = 1, integer-valued fp32 bias, |sum| < 2^24: every fp32 step is exact, so the float epilogue must reproduce the
+    exact integer convolution (pinned above) bit for bit, as int32 and, after clamping, as int8.
+    (src/conv2d_implicit_gemm.cu:278-286,330-338)"""
+    x = RNG.integers(-127, 128, (2, 5, 6, 16), dtype=np.int8)
+    w = RNG.integers(-127, 128, (7, 3, 3, 16), dtype=np.int8)
+    b = RNG.integers(-2 ** 15, 2 ** 15, 7).astype(np.int32)
+    raw = oracle.conv2d_i8(x, w, None)
+    assert np.abs(raw.astype(np.int64)).max() + 2 ** 15 < 2 ** 24
+    for act in (oracle.LINEAR, oracle.RELU):
+        exact = oracle.conv2d_i8(x, w, b, activation=act)
+        got32 = oracle.conv2d_i8_float_epilogue(raw, b.astype(np.float32), None, np.zeros(raw.shape, np.int32), 1.0, 1.0, 0.0, act)
+        np.testing.assert_array_equal(got32, exact)
+        got8 = oracle.conv2d_i8_float_epilogue(raw, b.astype(np.float32), None, np.zeros(raw.shape, np.int8), 1.0, 1.0, 0.0, act)
+        np.testing.assert_array_equal(got8, np.clip(exact, -128, 127).astype(np.int8))
+        gotf = oracle.conv2d_i8_float_epilogue(raw, b.astype(np.float32), None, np.zeros(raw.shape, np.float32), 1.0, 1.0, 0.0, act)
+        np.testing.assert_array_equal(gotf, exact.astype(np.float32))
+    # no bias: the term is skipped
+    np.testing.assert_array_equal(oracle.conv2d_i8_float_epilogue(raw, None, None, np.zeros(raw.shape, np.int32), 1.0, 1.0, 0.0, 0), raw)
+    # integer-valued residual and old output with power-of-two scalars stay exact as well
+    z = RNG.integers(-1000, 1000, raw.shape).astype(np.int32)
+    y0 = RNG.integers(-1000, 1000, raw.shape).astype(np.int32)
+    want = np.maximum(raw.astype(np.int64) + b + 2 * z.astype(np.int64), 0) + 4 * y0.astype(np.int64)
+    got = oracle.conv2d_i8_float_epilogue(raw, b.astype(np.float32), z, y0.copy(), 1.0, 2.0, 4.0, oracle.RELU)
+    np.testing.assert_array_equal(got, want.astype(np.int32))
+
+
+def test_int8_float_epilogue_rounding_hand_cases(oracle):
+    """Cast back to the integer type: round to nearest even, saturate, NaN -> 0.  Expected values written out by hand."""
+    i32, i8, f32 = np.int32, np.int8, np.float32
+    one = lambda *a, **k: _float_epilogue_1(oracle, *a, **k)
+    # ties, alpha1 = 0.5 (products exact)
+    for acc, want in [(1, 0), (3, 2), (5, 2), (7, 4), (-1, 0), (-3, -2), (-5, -2), (2, 1), (-2, -1)]:
+        assert one(acc, i32, alpha1=0.5) == want
+        assert one(acc, i8, alpha1=0.5) == want
+        assert one(acc, f32, alpha1=0.5) == acc / 2.0  # fp32 output is not rounded to an integer
+    # -0.5 rounds to minus zero, which is integer 0
+    assert one(-1, i32, alpha1=0.5) == 0
+    # saturation of int8
+    assert one(255, i8, alpha1=0.5) == 127       # 127.5 -> 128 -> 127
+    assert one(254, i8, alpha1=0.5) == 127
+    assert one(253, i8, alpha1=0.5) == 126       # 126.5 -> 126
+    assert one(-257, i8, alpha1=0.5) == -128     # -128.5 -> -128
+    assert one(-259, i8, alpha1=0.5) == -128     # -129.5 -> saturates
+    assert one(10 ** 9, i8) == 127
+    assert one(-10 ** 9, i8) == -128
+    # saturation of int32: 2^30 * 2 = 2^31 and beyond clamp to INT32_MAX; -2^31 is representable; below it clamps
+    assert one(2 ** 30, i32, alpha1=2.0) == 2 ** 31 - 1
+    assert one(2 ** 30, i32, alpha1=1024.0) == 2 ** 31 - 1
+    assert one(-2 ** 30, i32, alpha1=2.0) == -2 ** 31
+    assert one(-2 ** 30, i32, alpha1=4.0) == -2 ** 31
+    assert one(2 ** 30, i32, alpha1=1.0) == 2 ** 30
+    assert one(2 ** 31 - 1, i32) == 2 ** 31 - 1            # float(2^31 - 1) = 2^31 -> saturates to INT32_MAX
+    assert one(2 ** 31 - 129, i32) == 2 ** 31 - 128        # float() rounds to the nearest multiple of 128
+    assert one(2147483520, i32) == 2147483520              # largest fp32 below 2^31 passes unchanged
+    # NaN (inf * 0, NaN bias) -> 0; infinities saturate
+    assert one(0, i32, alpha1=float("inf")) == 0
+    assert one(5, i8, bias=float("nan")) == 0
+    assert one(1, i32, alpha1=float("inf")) == 2 ** 31 - 1
+    assert one(-1, i8, alpha1=float("inf")) == -128
+    assert np.isnan(one(5, f32, bias=float("nan")))
+    # int32 -> fp32 conversion of the sum is itself a rounding: 2^24 + 1 -> 2^24 (ties to even), 2^24 + 3 -> 2^24 + 4
+    assert one(2 ** 24 + 1, f32) == 16777216.0
+    assert one(2 ** 24 + 3, f32) == 16777220.0
+    assert one(2 ** 24 + 1, i32) == 16777216
+    # separate roundings, no fused multiply-add and no wider intermediate:
+    #   alpha1 = 1 + 2^-12, acc = 4097: exact product 4098 + 2^-12 lies half-way between 4098 and 4098 + 2^-11 -> 4098 (even);
+    #   + bias -4098 -> 0.  A fused multiply-add or a double intermediate gives 2^-12.
+    assert one(4097, f32, bias=-4098.0, alpha1=1.0 + 2.0 ** -12) == 0.0
+    #   alpha1 = 4097, acc = 4097: 4097^2 = 2^24 + 8193 is odd, fp32 spacing there is 2 -> ties to 16785408; - 16785408 -> 0 (wider: 1)
+    assert one(4097, i32, bias=-16785408.0, alpha1=4097.0) == 0
+    #   product rounds, then the bias addition rounds again: 2^24 (+1 -> tie -> 2^24) (+ 1*z=1 -> tie -> 2^24); adding b + z first gives 2^24 + 2
+    assert one(2 ** 24, f32, bias=1.0, z=1.0) == 16777216.0
+    assert one(2 ** 24, i32, bias=1.0, z=1) == 16777216
+    # a product that is inexact in fp32: 0.1f = 0x3DCCCCCD; 3 * 0.1f = 0.3000000044703484 -> 0x3E99999A; + 0.2f (0x3E4CCCCD) = 0.5000000149 -> 0x3F000000
+    r = one(3, f32, bias=np.float32(0.2), alpha1=np.float32(0.1))
+    assert np.float32(r).view(np.uint32) == 0x3F000000
+    r = one(3, f32, alpha1=np.float32(0.1))
+    assert np.float32(r).view(np.uint32) == 0x3E99999A
+    # -56228 * 0x3FF35336 + 0xC28E560E: two roundings give 0xC7D0E7A7, one rounding of the exact value 0xC7D0E7A6
+    a1 = np.array([0x3FF35336], dtype=np.uint32).view(np.float32)[0]
+    bb = np.array([0xC28E560E], dtype=np.uint32).view(np.float32)[0]
+    r = one(-56228, f32, bias=bb, alpha1=a1)
+    assert np.float32(r).view(np.uint32) == 0xC7D0E7A7
+
+
+def test_int8_float_epilogue_order(oracle):
+    """t = alpha1*float(sum); t += b; t += alpha2*z; t = act(t); t += beta*y_old  (src/conv2d_implicit_gemm.cu:278-286 with the
+    bias term of include/Avocado/cuda_backend.h:796).  Every other order of these steps gives a different number here."""
+    i32, i8, f32 = np.int32, np.int8, np.float32
+    one = lambda *a, **k: _float_epilogue_1(oracle, *a, **k)
+    # sum -10, b 2, z 3, y_old 8, beta 0.5, ReLU:  relu(-10 + 2 + 3) = 0, + 4 = 4
+    #   beta*y before the activation: relu(-5 + 4) = 0;  bias after the activation: relu(-7) + 2 = 2;  z after the activation: relu(-8) + 3 = 3
+    for dt in (i32, i8, f32):
+        assert one(-10, dt, bias=2.0, z=3, y0=8, beta=0.5, activation=oracle.RELU) == 4
+    # alpha2 scales z only, alpha1 the sum only: 3*5 + 1 + 2*4 = 24
+    for dt in (i32, i8, f32):
+        assert one(5, dt, bias=1.0, z=4, alpha1=3.0, alpha2=2.0) == 24
+    # beta = 0: the old output is not read (a NaN there must not leak); beta != 0 reads it
+    assert one(5, f32, y0=float("nan"), beta=0.0) == 5.0
+    assert np.isnan(one(5, f32, y0=float("nan"), beta=1.0))
+    # z and y_old are of the output's kind: int8 z = -128, y_old = 127
+    assert one(0, i8, z=-128, alpha2=0.5) == -64
+    assert one(0, i8, y0=127, beta=1.0) == 127
+    assert one(1, i8, y0=127, beta=1.0) == 127     # 128 saturates
+    # fp32 kind keeps fractions of z
+    assert one(1, f32, z=0.25, alpha2=2.0) == 1.5
+    # another activation than ReLU sits at the same place: tanh(0.5*2 + 0) + 1*3
+    np.testing.assert_allclose(one(2, f32, y0=3.0, alpha1=0.5, beta=1.0, activation=oracle.TANH), np.float32(np.tanh(1.0)) + np.float32(3.0), rtol=1e-6)
+    # filters index the bias (last axis)
+    acc = np.array([[1, 1, 1], [2, 2, 2]], dtype=np.int32)
+    got = oracle.conv2d_i8_float_epilogue(acc, np.array([10, 20, 30], dtype=np.float32), None, np.zeros((2, 3), np.int32), 1.0, 1.0, 0.0, 0)
+    np.testing.assert_array_equal(got, [[11, 21, 31], [12, 22, 32]])
 
 
 @pytest.mark.parametrize("m,r", [(2, 3), (4, 3), (2, 5)])
