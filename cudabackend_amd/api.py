@@ -70,6 +70,7 @@ PROTOTYPES = {
     "cudaIm2Row": (i32, [i64, i64, i64, i64, i64, i64, i64]),
     "cudaConvolutionImplicitGemmForward": (i32, [i64, i64, vp, i64, i64, i64, i64, i64, i64, vp, i64, i64, vp, i64, i64, i32]),
     "cudaConvolutionWinogradFusedForward": (i32, [i64, i64, vp, i64, i64, i64, i64, i64, i64, vp, i64, i64, vp, i64, i64, i32]),
+    "avhipConvolutionWinogradFusedForwardNoAlloc": (i32, [i64, i64, vp, i64, i64, i64, i64, i64, i64, vp, i64, i64, vp, i64, i64, i32]),
     "cudaWinogradWeightTransform": (i32, [i64, i64, i32, i64, i64, i64, i64]),
     "cudaWinogradInputTransform": (i32, [i64, i64, i32, i64, i64, i64, i64, i64]),
     "cudaWinogradOutputTransform": (i32, [i64, i64, i32, i64, vp, i64, i64, i64, i64, i64, i64, vp, i64, i64, vp, i32]),

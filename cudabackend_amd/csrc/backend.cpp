@@ -13,7 +13,7 @@
  * Memory blocks carry a version that every API call writing to them increments.  It keys the cache of transformed weights
  * used by the fused Winograd path, so a weight tensor is re-transformed exactly when it was written since the last call.
  */
-#include <hip/hip_runtime_api.h>
+#include <hip/hip_runtime.h>
 
 #include <cmath>
 #include <cstring>
@@ -716,6 +716,37 @@ namespace
 		return from_launcher(rc);
 	}
 
+	/* ------------------------------------------------------------------------------------------------------------
+	 * Scratch of the one entry point that allocates nothing (avhipConvolutionWinogradFusedForwardNoAlloc): the transformed
+	 * weights [16, K, C] of a call live in this fixed array instead of library-allocated memory.  Every device holds its
+	 * own copy of the array at its own address until the process ends; the name below is a host-side stand-in, never a
+	 * device address, so host code only ever uses the pointer that hipGetSymbolAddress returned for the current device.
+	 * ------------------------------------------------------------------------------------------------------------ */
+	static __device__ __align__(256) unsigned char scratch[AVHIP_NOALLOC_SCRATCH_BYTES];
+	constexpr int NOALLOC_MAX_DEVICES = 64;
+	/* Device address of `scratch` on `device`, which must be the current device.  Looked up once per device. */
+	avStatus_t noalloc_scratch_pointer(int device, void **out)
+	{
+		static std::mutex mutex;
+		static void *pointers[NOALLOC_MAX_DEVICES] = { nullptr };
+		if (device < 0 || device >= NOALLOC_MAX_DEVICES)
+			return AVOCADO_STATUS_BAD_PARAM;
+		std::lock_guard<std::mutex> lock(mutex);
+		if (pointers[device] == nullptr)
+		{
+			void *p = nullptr;
+			const hipError_t err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+			if (err != hipSuccess || p == nullptr)
+			{
+				(void) hipGetLastError();
+				return AVOCADO_STATUS_INTERNAL_ERROR;
+			}
+			pointers[device] = p;
+		}
+		out[0] = pointers[device];
+		return AVOCADO_STATUS_SUCCESS;
+	}
+
 	/* Shared validation of the two per-channel transforms: the parameter tensors hold one value per element of x's
 	 * trailing dimensions (volume(params) must divide volume(x)); fp32 parameters for 16-bit and fp32 tensors, fp64 for fp64. */
 	avStatus_t per_channel_view(const Tensor *x, const Tensor *y, const Tensor *params, av_int64 &first, av_int64 &last)
@@ -1340,6 +1371,39 @@ namespace avocado
 			if (st != AVOCADO_STATUS_SUCCESS)
 				return st;
 			return run_fused_winograd(call, wMem, yMem, activation);
+		}
+
+		avStatus_t avhipConvolutionWinogradFusedForwardNoAlloc(avContextDescriptor_t context, const avConvolutionDescriptor_t config, const void *alpha1,
+				const avTensorDescriptor_t xDesc, const avMemoryDescriptor_t xMem, const avTensorDescriptor_t wDesc, const avMemoryDescriptor_t wMem,
+				const avTensorDescriptor_t bDesc, const avMemoryDescriptor_t bMem, const void *alpha2, const avTensorDescriptor_t zDesc,
+				const avMemoryDescriptor_t zMem, const void *beta, const avTensorDescriptor_t yDesc, avMemoryDescriptor_t yMem,
+				avActivationType_t activation)
+		{
+			ConvCall call;
+			const avStatus_t st = prepare_conv(context, config, alpha1, xDesc, xMem, wDesc, wMem, bDesc, bMem, alpha2, zDesc, zMem, beta, yDesc, yMem, call);
+			if (st != AVOCADO_STATUS_SUCCESS)
+				return st;
+			const ConvProblem &p = call.problem;
+			if (!fused_winograd_applicable(p))
+				return AVOCADO_STATUS_NOT_SUPPORTED;
+			if (call.bias != nullptr && call.bias_dtype != AVOCADO_DTYPE_FLOAT32)
+				return AVOCADO_STATUS_UNSUPPORTED_DATATYPE;
+			const avDataType_t mat_dtype = (p.w_dtype == AVOCADO_DTYPE_FLOAT32) ? AVOCADO_DTYPE_FLOAT32 : AVOCADO_DTYPE_FLOAT16;
+			const av_int64 u_bytes = static_cast<av_int64>(16) * p.shape.K * p.shape.C * size_of(mat_dtype);
+			if (u_bytes > static_cast<av_int64>(AVHIP_NOALLOC_SCRATCH_BYTES))
+				return AVOCADO_STATUS_NOT_SUPPORTED; /* the transformed weights do not fit the fixed scratch array */
+			void *U = nullptr; /* prepare_conv made the context's device current */
+			const avStatus_t ss = noalloc_scratch_pointer(call.ctx.device, &U);
+			if (ss != AVOCADO_STATUS_SUCCESS)
+				return ss;
+			/* the transform overwrites all of [16, K, C], so nothing of the previous call's contents is read */
+			int rc = avhip_winograd_weight_transform(call.ctx.stream, p.w_dtype, mat_dtype, 2, 3, p.shape.mode, call.w->data, U, p.shape.K, p.shape.C);
+			if (rc != 0)
+				return from_launcher(rc);
+			touch(yMem);
+			rc = avhip_conv2d_winograd_fused(call.ctx.stream, p.x_dtype, &p.shape, call.x->data, U, call.bias, call.z, call.y->data, call.alpha1,
+					call.alpha2, call.beta, activation);
+			return from_launcher(rc);
 		}
 
 		avStatus_t avhipConvolutionRequantForward(avContextDescriptor_t context, const avConvolutionDescriptor_t config, const avTensorDescriptor_t xDesc,

@@ -209,6 +209,20 @@ namespace avocado
 					const avTensorDescriptor_t xDesc, const avMemoryDescriptor_t xMem, const avTensorDescriptor_t wDesc, const avMemoryDescriptor_t wMem,
 					const avTensorDescriptor_t bDesc, const avMemoryDescriptor_t bMem, const avTensorDescriptor_t scaleDesc,
 					const avMemoryDescriptor_t scaleMem, const avTensorDescriptor_t yDesc, avMemoryDescriptor_t yMem, avActivationType_t activation);
+			/* No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph capture,
+			 * tight serving loops, harnesses that forbid hipMalloc): cudaConvolutionWinogradFusedForward with the transformed
+			 * weights [16, K, C] (FLOAT16 for 16-bit tensors, FLOAT32 for fp32) kept in a fixed device array of
+			 * AVHIP_NOALLOC_SCRATCH_BYTES inside the library instead of library-allocated memory; the weights are transformed on
+			 * the context's stream in every call, nothing is cached, and no allocating routine is called.  Returns
+			 * AVOCADO_STATUS_NOT_SUPPORTED when 16 * K * C matrix elements exceed the array.  Every call on a device shares that
+			 * device's array: calls that overlap in time on one device (different contexts) race; calls on one context are ordered
+			 * by its stream.  The first call on a device looks the array's address up (no allocation, but do it outside capture). */
+#define AVHIP_NOALLOC_SCRATCH_BYTES (4u << 20)
+			DLL_PUBLIC avStatus_t avhipConvolutionWinogradFusedForwardNoAlloc(avContextDescriptor_t context, const avConvolutionDescriptor_t config,
+					const void *alpha1, const avTensorDescriptor_t xDesc, const avMemoryDescriptor_t xMem, const avTensorDescriptor_t wDesc,
+					const avMemoryDescriptor_t wMem, const avTensorDescriptor_t bDesc, const avMemoryDescriptor_t bMem, const void *alpha2,
+					const avTensorDescriptor_t zDesc, const avMemoryDescriptor_t zMem, const void *beta, const avTensorDescriptor_t yDesc,
+					avMemoryDescriptor_t yMem, avActivationType_t activation);
 			/* Interop for harnesses: the HIP stream (hipStream_t) of a context and the device address behind a memory
 			 * descriptor.  Writing through the raw address bypasses the library's change tracking of weight tensors: call
 			 * avhipInvalidateCaches afterwards. */
