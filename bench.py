@@ -114,11 +114,13 @@ class Tower:
         self.x0 = cb.DeviceTensor.from_numpy(x0, d)
         self.conv = cb.ConvolutionDescriptor(padding=(-1, -1), dtype=d)
         self.layers = []
+        self.host_layers = []  # the same weights and biases on the host, for the self-check
         cin = planes
         for _ in range(1 + 2 * blocks):
             w = g.standard_normal((ch, 3, 3, cin)).astype(np.float32) * np.float32(np.sqrt(2.0 / (9 * cin)))
             b = g.uniform(-0.1, 0.1, ch).astype(np.float32)
             self.layers.append((cb.DeviceTensor.from_numpy(w, d), cb.DeviceTensor.from_numpy(b, cb.DTYPE_FLOAT32)))
+            self.host_layers.append((w, b))
             cin = ch
         self.act = [cb.DeviceTensor((N, HW, HW, ch), d) for _ in range(3)]
         need = C.c_int64(0)
@@ -139,23 +141,34 @@ class Tower:
     def stem(self):
         self._conv(self.x0, 0, None, self.act[0])
 
-    def step(self):
+    def step(self, after=None):
+        """One forward pass: stem, then per block [conv -> t, conv + residual -> b] with the three activation buffers rotating.
+        after(layer, x, z, y), when given, is called behind each enqueued convolution with its input, residual and output tensors."""
+        after = after or (lambda *args: None)
         a, t, b = self.act
         self._conv(self.x0, 0, None, a)
+        after(0, self.x0, None, a)
         layer = 1
         for _ in range(self.blocks):
             self._conv(a, layer, None, t)
+            after(layer, a, None, t)
             self._conv(t, layer + 1, a, b)
+            after(layer + 1, t, a, b)
             layer += 2
             a, b = b, a
         return a
+
+    def set_weights(self, layer, w):
+        """Rewrites the weights of one layer through the API (the library tracks the write and re-transforms what it cached)."""
+        self.layers[layer][0].upload(w)
+        self.host_layers[layer] = (np.asarray(w, dtype=np.float32), self.host_layers[layer][1])
 
     def close(self):
         for t in [self.x0, self.workspace] + self.act + [t for pair in self.layers for t in pair]:
             t.close()
 
 
-def time_tower(hip, ctx, dtype, steps, warmup):
+def time_tower(hip, ctx, dtype, steps, warmup, check=True):
     """Times `steps` forward passes of the tower.  One pass is captured into a HIP graph and replayed, so the timed region
     holds 21 * steps kernels back to back on the context's stream, bracketed by HIP events on that stream.  The duration of
     the dominant kernel (the 20 identical 128->128 body convolutions of a pass) is (pass - stem) / 20 with the stem
@@ -165,15 +178,29 @@ def time_tower(hip, ctx, dtype, steps, warmup):
     for _ in range(max(1, warmup)):
         tower.step()  # also fills the library's transformed-weight cache, so that nothing allocates during capture
     ctx.synchronize()
-    full = hip.capture(stream, tower.step)
+    final = []
+    full = hip.capture(stream, lambda: final.append(tower.step()))
     stem = hip.capture(stream, lambda: [tower.stem() for _ in range(10)])
     hip.sync()
     ms_step = hip.time_graph(full, stream, steps, warmup)
+    ctx.synchronize()
+    checked = self_check(tower, final[0]) if check else {"checked": False}  # what the timed replays left behind, against the CPU oracle
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tower.step()  # the same pass as 21 eager calls: launch and host cost of the API included
+    ctx.synchronize()
+    ms_eager = (time.perf_counter() - t0) * 1e3 / steps
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tower.step()
+    host_us_per_call = (time.perf_counter() - t0) * 1e6 / (steps * (1 + 2 * tower.blocks))  # enqueue only: the stream runs behind
+    ctx.synchronize()
     ms_stem = hip.time_graph(stem, stream, max(steps, 10), warmup) / 10
     ctx.synchronize()
     body_us = (ms_step - ms_stem) * 1e3 / (2 * tower.blocks)
     out = {"ms_per_step": ms_step, "tflops": tower.flops_step / (ms_step * 1e-3) / 1e12, "stem_conv_us": ms_stem * 1e3,
-           "body_conv_us": body_us, "body_conv_tflops": tower.flops_body / (body_us * 1e-6) / 1e12, "workspace_bytes": tower.workspace_bytes}
+           "body_conv_us": body_us, "body_conv_tflops": tower.flops_body / (body_us * 1e-6) / 1e12, "workspace_bytes": tower.workspace_bytes,
+           "ms_per_step_eager_calls": ms_eager, "host_us_per_call": host_us_per_call, "self_check": checked}
     hip.rt.hipGraphExecDestroy(full)
     hip.rt.hipGraphExecDestroy(stem)
     tower.close()
@@ -426,6 +453,62 @@ def counter_calibration(ctx, launches=3):
     b.close()
 
 
+# ---- CPU legs: the oracle as checker of the timed region's output, and the timed CPU baseline ------------------------------------
+LAYER_BAR = {"bf16": 2e-3, "f16": 2e-3, "f32": 1e-4}   # one convolution against the oracle on the same inputs (rel-L2)
+# 21 chained convolutions against the oracle chained the same way: output roundings that fall the other way propagate through
+# the layers (measured 7e-3 / 1e-3 / 2e-6), while a layer that used wrong weights or a wrong buffer gives an error of order one
+CHAIN_BAR = {"bf16": 2e-2, "f16": 4e-3, "f32": 2e-4}
+
+
+def check_layer(orc, tower, layer, x, z, y, images):
+    """One convolution of the tower against the oracle on the GPU's own input (and residual) of that layer, for some images.
+    Returns the largest rel-L2 error over the images."""
+    w, b = tower.host_layers[layer]
+    wr = orc.round_to(w, tower.dtype)
+    worst = 0.0
+    for n in images:
+        xin = x.download_slice(n)
+        zin = z.download_slice(n) if z is not None else None
+        want = orc.conv2d(xin, wr, b.astype(np.float64), zin, activation=orc.RELU)
+        worst = max(worst, orc.rel_l2(y.download_slice(n), want))
+    return worst
+
+
+def check_chain(orc, tower, out, images):
+    """The whole pass for some images: the oracle chained through all 21 layers with the tower's buffer rotation restated on the host
+    (each layer's output rounded to the tensor dtype, as the device stores it), against the final activation `out`."""
+    worst = 0.0
+    for n in images:
+        a = tower.x0.download_slice(n)
+        layer = 0
+        w, b = tower.host_layers[0]
+        a = orc.round_to(orc.conv2d(a, orc.round_to(w, tower.dtype), b.astype(np.float64), activation=orc.RELU), tower.dtype)
+        layer = 1
+        for _ in range(tower.blocks):
+            w, b = tower.host_layers[layer]
+            t = orc.round_to(orc.conv2d(a, orc.round_to(w, tower.dtype), b.astype(np.float64), activation=orc.RELU), tower.dtype)
+            w, b = tower.host_layers[layer + 1]
+            a = orc.round_to(orc.conv2d(t, orc.round_to(w, tower.dtype), b.astype(np.float64), a, activation=orc.RELU), tower.dtype)
+            layer += 2
+        worst = max(worst, orc.rel_l2(out.download_slice(n), a))
+    return worst
+
+
+def self_check(tower, out, images=(0,)):
+    """Checks what the timed region left in the tower's buffers: the last convolution teacher-forced on the device's own
+    inputs, and the whole chain of 21.  Raises when either misses its bar, so that no figure is reported for wrong results."""
+    from oracle import oracle as orc
+    a, t, b = tower.act
+    last = 2 * tower.blocks
+    residual = [buf for buf in tower.act if buf is not out and buf is not t][0]
+    e_layer = check_layer(orc, tower, last, t, residual, out, images)
+    e_chain = check_chain(orc, tower, out, images)
+    if not (e_layer < LAYER_BAR[tower.dtype] and e_chain < CHAIN_BAR[tower.dtype]):
+        raise AssertionError("tower self-check failed (%s): last layer rel-L2 %.3e (bar %.0e), chain of 21 rel-L2 %.3e (bar %.0e)"
+                             % (tower.dtype, e_layer, LAYER_BAR[tower.dtype], e_chain, CHAIN_BAR[tower.dtype]))
+    return {"checked": True, "images": list(images), "last_layer_rel_l2": e_layer, "chain_rel_l2": e_chain}
+
+
 def cpu_baseline(seconds=12.0):
     """fp32 direct convolution of the body layer (128->128, 15x15, 3x3) on a batch slice, all host cores."""
     from oracle import oracle as orc
@@ -455,7 +538,7 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"])
     ap.add_argument("--quick", action="store_true", help="headline tower only (no side legs, no CPU baseline)")
     ap.add_argument("--calibrate", action="store_true", help="also launch a streaming kernel of known traffic (for counter runs)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (for counter runs, where only the GPU side matters)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU legs: the baseline and the oracle check of the towers' outputs (for counter runs, where only the GPU side matters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards over the batch with no collectives)." % args.gpus,
@@ -467,7 +550,7 @@ def main():
         sys.exit(3)
     hip = Hip()
     ctx = cb.Context(0)
-    head = time_tower(hip, ctx, args.dtype, args.steps, args.warmup)
+    head = time_tower(hip, ctx, args.dtype, args.steps, args.warmup, check=not args.no_cpu)
     detail = {"headline": head}
     cpu = None
     if args.calibrate:
@@ -476,7 +559,7 @@ def main():
         it = max(5, args.steps)
         for other in ("f32", "bf16", "f16"):
             if other != args.dtype:
-                detail["tower_" + other] = time_tower(hip, ctx, other, max(3, args.steps // 2), 2)
+                detail["tower_" + other] = time_tower(hip, ctx, other, max(3, args.steps // 2), 2, check=not args.no_cpu)
         detail["caller_level_two_chains_of_128"] = two_half_batch_chains(hip, args.dtype, args.steps)
         detail["int8_config4"] = int8_leg(hip, ctx, it)
         detail["nonfused_winograd_f32_F4"] = nonfused_stages(hip, ctx, "f32", "f32", 4, it)

@@ -238,6 +238,15 @@ class DeviceTensor:
         """float64 values for floating tensors, the integer array otherwise."""
         return from_device_repr(self.download_raw(), self.dtype)
 
+    def download_slice(self, first, count=1):
+        """Entries first .. first + count - 1 along the leading dimension, as download() returns them."""
+        assert 0 <= first and first + count <= self.shape[0]
+        raw = np.empty((count,) + self.shape[1:], dtype=HOST_DTYPE[self.dtype])
+        row = self.nbytes // self.shape[0]
+        check(self.lib.cudaCopyMemoryToHost(self.lib.cudaGetDefaultContext(self.device), raw.ctypes.data_as(vp), self.mem, first * row, count * row),
+              "cudaCopyMemoryToHost")
+        return from_device_repr(raw, self.dtype)
+
     def pointer(self):
         p = vp()
         check(self.lib.avhipGetMemoryPointer(self.mem, C.byref(p)), "avhipGetMemoryPointer")
