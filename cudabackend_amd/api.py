@@ -83,6 +83,7 @@ PROTOTYPES = {
     "avhipGetContextStream": (i32, [i64, C.POINTER(vp)]),
     "avhipGetMemoryPointer": (i32, [i64, C.POINTER(vp)]),
     "avhipInvalidateCaches": (i32, []),
+    "avhipGetWeightCacheState": (i32, [C.POINTER(i64), C.POINTER(i64), C.POINTER(i64)]),
 }
 # the thin kernel layer of include/avocado_hip_kernels.h (exported, bound only for the symbol check)
 KERNEL_LAYER_SYMBOLS = ["avhip_winograd_weight_transform", "avhip_winograd_input_transform", "avhip_winograd_output_transform",

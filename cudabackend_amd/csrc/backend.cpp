@@ -10,11 +10,12 @@
  * per-kind table.  The default context of device d is the handle (kind = context, device = d, slot = 0xFFFFFFFF); it maps
  * to the null stream and, as in the reference (src/descriptors.cu:120-124), makes copies synchronous.
  *
- * Memory blocks carry a version that every API call writing to them increments.  It keys the cache of transformed weights
- * used by the fused Winograd path, so a weight tensor is re-transformed exactly when it was written since the last call.
+ * Owning memory blocks keep a short log of the byte ranges that API calls wrote to them.  The cache of Winograd-transformed
+ * weights reads it, so a weight tensor is re-transformed exactly when its own bytes were written since the cached copy was made.
  */
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <map>
@@ -59,6 +60,39 @@ namespace
 		hipStream_t stream = nullptr;
 		bool is_default = false;
 	};
+	/* The last writes to an owning block through the API: write number v covers bytes [lo, hi) and sits in slot v % LOG. */
+	struct WriteLog
+	{
+		static constexpr int LOG = 64;
+		std::mutex mutex;
+		uint64_t version = 0; /* number of writes so far */
+		av_int64 lo[LOG], hi[LOG];
+		void record(av_int64 first, av_int64 last)
+		{
+			std::lock_guard<std::mutex> lock(mutex);
+			version++;
+			lo[version % LOG] = first;
+			hi[version % LOG] = last;
+		}
+		/* Whether bytes [first, last) were written after write number `seen`; `seen` moves up to the current number when not.
+		 * Writes that have left the log count as hits. */
+		bool written_since(uint64_t &seen, av_int64 first, av_int64 last)
+		{
+			std::lock_guard<std::mutex> lock(mutex);
+			if (version - seen > static_cast<uint64_t>(LOG))
+				return true;
+			for (uint64_t v = seen + 1; v <= version; v++)
+				if (lo[v % LOG] < last && first < hi[v % LOG])
+					return true;
+			seen = version;
+			return false;
+		}
+		uint64_t current()
+		{
+			std::lock_guard<std::mutex> lock(mutex);
+			return version;
+		}
+	};
 	struct Memory
 	{
 		char *data = nullptr;
@@ -66,8 +100,9 @@ namespace
 		int device = 0;
 		bool owning = true;
 		uint32_t owner_slot = 0; /* for a view: slot of the owning block */
-		uint64_t version = 0; /* owning blocks only */
+		uint64_t owner_uid = 0; /* for a view: uid of the owning block, so that a recycled slot is not mistaken for it */
 		uint64_t uid = 0; /* unique over the life of the process */
+		std::unique_ptr<WriteLog> writes; /* owning blocks only */
 	};
 	struct Tensor
 	{
@@ -123,7 +158,8 @@ namespace
 		}
 	};
 
-	/* Slot table with a free list.  Lookups return nullptr for stale or foreign handles. */
+	/* Slot table with a free list.  Lookups return nullptr for foreign handles and for slots that are free; a stale handle whose
+	 * slot was handed out again resolves to the new object (views guard against that with the owner's uid). */
 	template<typename T>
 	class Table
 	{
@@ -239,18 +275,23 @@ namespace
 		Memory *m = get_memory(h);
 		return m != nullptr ? m->data : nullptr;
 	}
+	/* The owning block behind a memory object; nullptr for a view whose owner has been destroyed (even if its slot is in use again). */
 	Memory* owner_of(Memory *m)
 	{
 		if (m == nullptr || m->owning)
 			return m;
-		return memories().get(m->owner_slot);
+		Memory *o = memories().get(m->owner_slot);
+		return (o != nullptr && o->owning && o->uid == m->owner_uid) ? o : nullptr;
 	}
-	/* Records that the block behind h is about to be written. */
-	void touch(avMemoryDescriptor_t h)
+	/* Records that `bytes` bytes from `offset` of the memory behind h are about to be written (bytes < 0: all of it). */
+	void touch(avMemoryDescriptor_t h, av_int64 offset = 0, av_int64 bytes = -1)
 	{
-		Memory *o = owner_of(get_memory(h));
-		if (o != nullptr)
-			o->version++;
+		Memory *m = get_memory(h);
+		Memory *o = owner_of(m);
+		if (o == nullptr || !o->writes || m->data == nullptr)
+			return;
+		const av_int64 first = (m->data - o->data) + offset;
+		o->writes->record(first, first + (bytes < 0 ? m->size - offset : bytes));
 	}
 
 	avStatus_t from_hip(hipError_t err)
@@ -388,41 +429,106 @@ namespace
 	}
 
 	/* ------------------------------------------------------------------------------------------------------------
-	 * Cache of Winograd-transformed weights for the fused path, keyed by the identity and version of the weight block.
+	 * Cache of Winograd-transformed weights [t*t, K, C], keyed by the weight tensor (owning block, offset, shape, dtype, mode,
+	 * tile size).  Rules that keep it safe with several contexts, rewritten weights and captured graphs:
+	 *  - An entry records the event behind its transform and the stream that ran it.  A call on another stream waits for
+	 *    that event (hipStreamWaitEvent) until the event is known to have completed.
+	 *  - When the weight bytes were written through the API since the transform, the SAME buffer is transformed again on the
+	 *    calling stream.  Whatever ordering the caller needs anyway between the write of the weights and other streams still
+	 *    reading them also orders the rewrite of the matrices, and a captured graph that holds the buffer's address keeps
+	 *    reading valid memory.  Nothing is freed on that path.
+	 *  - Buffers are freed only by avhipInvalidateCaches, by the destruction of the weight block, or when the cache outgrows
+	 *    its budget at the insertion of a new tensor, then after a device synchronisation and outside the cache's mutex.
+	 *  - A stream that is capturing never changes the cache: no allocation, no transform, no event.  It may use an entry that
+	 *    is up to date and whose transform ran on the same stream or is known to be complete; otherwise the lookup reports
+	 *    AVOCADO_STATUS_BAD_ALLOC ("cannot allocate here": call once outside capture first) and the dispatcher takes the
+	 *    implicit-GEMM plan, which needs no matrices.
 	 * ------------------------------------------------------------------------------------------------------------ */
 	struct WeightKey
 	{
 		uint64_t uid;
-		uint64_t version;
 		av_int64 offset;
 		int K, C, dtype, mode, m; /* m: Winograd output tile, 2 = F(2x2,3x3) for the fused kernel, 4 = F(4x4,3x3) for the non-fused plan */
 		bool operator<(const WeightKey &o) const
 		{
-			return std::tie(uid, version, offset, K, C, dtype, mode, m) < std::tie(o.uid, o.version, o.offset, o.K, o.C, o.dtype, o.mode, o.m);
+			return std::tie(uid, offset, K, C, dtype, mode, m) < std::tie(o.uid, o.offset, o.K, o.C, o.dtype, o.mode, o.m);
 		}
+	};
+	struct WeightEntry
+	{
+		void *U = nullptr;
+		size_t bytes = 0;
+		int device = 0;
+		hipEvent_t ready = nullptr; /* recorded behind the last transform */
+		hipStream_t stream = nullptr; /* the stream that ran it */
+		bool complete = false; /* the event has been seen complete */
+		uint64_t seen = 0; /* write number of the weight block the matrices are known to be current for */
+		uint64_t last_use = 0;
 	};
 	struct WeightCache
 	{
+		static constexpr size_t BUDGET = static_cast<size_t>(4) << 30; /* bytes of matrices kept before the least recently used go */
 		std::mutex mutex;
-		std::map<WeightKey, void*> entries;
+		std::map<WeightKey, WeightEntry> entries;
+		size_t total = 0;
+		uint64_t clock = 0;
+		uint64_t transforms = 0; /* weight transforms launched so far */
+		static void release(std::vector<WeightEntry> &victims)
+		{
+			if (victims.empty())
+				return;
+			/* kernels on any stream may still read the matrices */
+			(void) hipDeviceSynchronize();
+			for (WeightEntry &e : victims)
+			{
+				(void) hipSetDevice(e.device);
+				(void) hipFree(e.U);
+				(void) hipEventDestroy(e.ready);
+			}
+			victims.clear();
+		}
 		void clear()
 		{
-			std::lock_guard<std::mutex> lock(mutex);
-			for (auto &e : entries)
-				(void) hipFree(e.second);
-			entries.clear();
+			std::vector<WeightEntry> victims;
+			{
+				std::lock_guard<std::mutex> lock(mutex);
+				for (auto &e : entries)
+					victims.push_back(e.second);
+				entries.clear();
+				total = 0;
+			}
+			release(victims);
 		}
 		void drop_block(uint64_t uid)
 		{
-			std::lock_guard<std::mutex> lock(mutex);
-			for (auto it = entries.begin(); it != entries.end();)
-				if (it->first.uid == uid)
-				{
-					(void) hipFree(it->second);
-					it = entries.erase(it);
-				}
-				else
-					++it;
+			std::vector<WeightEntry> victims;
+			{
+				std::lock_guard<std::mutex> lock(mutex);
+				for (auto it = entries.begin(); it != entries.end();)
+					if (it->first.uid == uid)
+					{
+						victims.push_back(it->second);
+						total -= it->second.bytes;
+						it = entries.erase(it);
+					}
+					else
+						++it;
+			}
+			release(victims);
+		}
+		/* with the mutex held: moves least recently used entries out until `incoming` more bytes fit the budget */
+		void make_room(size_t incoming, std::vector<WeightEntry> &victims)
+		{
+			while (!entries.empty() && total + incoming > BUDGET)
+			{
+				auto oldest = entries.begin();
+				for (auto it = entries.begin(); it != entries.end(); ++it)
+					if (it->second.last_use < oldest->second.last_use)
+						oldest = it;
+				victims.push_back(oldest->second);
+				total -= oldest->second.bytes;
+				entries.erase(oldest);
+			}
 		}
 	};
 	WeightCache& weight_cache()
@@ -432,59 +538,113 @@ namespace
 	}
 	uint64_t next_uid()
 	{
-		static std::mutex m;
-		static uint64_t uid = 0;
-		std::lock_guard<std::mutex> lock(m);
+		static std::atomic<uint64_t> uid { 0 };
 		return ++uid;
 	}
+	bool is_capturing(hipStream_t stream)
+	{
+		if (stream == nullptr)
+			return false; /* the null stream cannot be captured */
+		hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+		if (hipStreamIsCapturing(stream, &status) != hipSuccess)
+		{
+			(void) hipGetLastError();
+			return true; /* be careful: behave as under capture */
+		}
+		return status != hipStreamCaptureStatusNone;
+	}
 
-	/* Returns the [t*t, K, C] Winograd weight matrices F(m x m, 3x3) of a weight tensor in `mat_dtype`, transforming on the
-	 * context's stream when the weight block changed since the cached copy was made. */
+	/* Returns the [t*t, K, C] Winograd weight matrices F(m x m, 3x3) of a weight tensor in `mat_dtype`, (re)transforming on the
+	 * context's stream when the cache has none or the weight bytes were written since. */
 	avStatus_t cached_winograd_weights(const Context &ctx, const ConvProblem &p, avMemoryDescriptor_t wMem, int m, avDataType_t mat_dtype, const void **U)
 	{
 		Memory *wm = get_memory(wMem);
 		Memory *owner = owner_of(wm);
-		if (wm == nullptr || owner == nullptr)
+		if (wm == nullptr || owner == nullptr || !owner->writes)
 			return AVOCADO_STATUS_BAD_PARAM;
-		const WeightKey key { owner->uid, owner->version, static_cast<av_int64>(wm->data - owner->data), p.shape.K, p.shape.C,
-				static_cast<int>(p.w_dtype), p.shape.mode, m };
-		WeightCache &cache = weight_cache();
-		std::lock_guard<std::mutex> lock(cache.mutex);
-		auto it = cache.entries.find(key);
-		if (it != cache.entries.end())
-		{
-			*U = it->second;
-			return AVOCADO_STATUS_SUCCESS;
-		}
-		/* copies of older versions of the same tensor are of no further use */
-		for (auto e = cache.entries.begin(); e != cache.entries.end();)
-			if (e->first.uid == key.uid && e->first.offset == key.offset && e->first.version != key.version)
-			{
-				/* the kernel that last read it may still be running on another stream: order the free behind all work */
-				(void) hipDeviceSynchronize();
-				(void) hipFree(e->second);
-				e = cache.entries.erase(e);
-			}
-			else
-				++e;
-		void *buf = nullptr;
+		const av_int64 offset = wm->data - owner->data;
+		const av_int64 w_bytes = static_cast<av_int64>(p.shape.K) * 9 * p.shape.C * size_of(p.w_dtype);
+		const WeightKey key { owner->uid, offset, p.shape.K, p.shape.C, static_cast<int>(p.w_dtype), p.shape.mode, m };
 		const int t = m + 2;
 		const size_t bytes = static_cast<size_t>(t * t) * p.shape.K * p.shape.C * size_of(mat_dtype);
-		if (hipMalloc(&buf, bytes) != hipSuccess)
+		WeightCache &cache = weight_cache();
+		std::vector<WeightEntry> victims;
+		avStatus_t status = AVOCADO_STATUS_SUCCESS;
 		{
-			(void) hipGetLastError();
-			return AVOCADO_STATUS_ALLOC_FAILED;
+			std::lock_guard<std::mutex> lock(cache.mutex);
+			auto it = cache.entries.find(key);
+			const bool found = it != cache.entries.end();
+			const bool current = found && !owner->writes->written_since(it->second.seen, offset, offset + w_bytes);
+			if (current)
+			{
+				WeightEntry &e = it->second;
+				e.last_use = ++cache.clock;
+				U[0] = e.U;
+				if (e.complete || e.stream == ctx.stream)
+					return AVOCADO_STATUS_SUCCESS; /* stream order, or nothing left to wait for */
+				if (is_capturing(ctx.stream))
+					return AVOCADO_STATUS_BAD_ALLOC; /* an event from outside must not enter the capture */
+				if (hipEventQuery(e.ready) == hipSuccess)
+				{
+					e.complete = true;
+					return AVOCADO_STATUS_SUCCESS;
+				}
+				(void) hipGetLastError(); /* hipErrorNotReady is not an error here */
+				return from_hip(hipStreamWaitEvent(ctx.stream, e.ready, 0));
+			}
+			if (is_capturing(ctx.stream))
+				return AVOCADO_STATUS_BAD_ALLOC;
+			if (!found)
+			{
+				cache.make_room(bytes, victims);
+				WeightEntry e;
+				e.bytes = bytes;
+				e.device = ctx.device;
+				if (hipMalloc(&e.U, bytes) != hipSuccess)
+				{
+					(void) hipGetLastError();
+					status = AVOCADO_STATUS_ALLOC_FAILED;
+				}
+				else if (hipEventCreateWithFlags(&e.ready, hipEventDisableTiming) != hipSuccess)
+				{
+					(void) hipGetLastError();
+					(void) hipFree(e.U);
+					status = AVOCADO_STATUS_ALLOC_FAILED;
+				}
+				else
+				{
+					it = cache.entries.emplace(key, e).first;
+					cache.total += bytes;
+				}
+			}
+			if (status == AVOCADO_STATUS_SUCCESS)
+			{
+				WeightEntry &e = it->second;
+				/* the write number is read before the transform is enqueued: a write that slips in between is seen next time */
+				e.seen = owner->writes->current();
+				const int rc = avhip_winograd_weight_transform(ctx.stream, p.w_dtype, mat_dtype, m, 3, p.shape.mode, wm->data, e.U, p.shape.K, p.shape.C);
+				status = from_launcher(rc);
+				cache.transforms++;
+				if (status == AVOCADO_STATUS_SUCCESS)
+					status = from_hip(hipEventRecord(e.ready, ctx.stream));
+				if (status == AVOCADO_STATUS_SUCCESS)
+				{
+					e.stream = ctx.stream;
+					e.complete = false;
+					e.last_use = ++cache.clock;
+					U[0] = e.U;
+				}
+				else
+				{
+					/* the buffer holds nothing usable: drop the entry (freed below, outside the mutex) */
+					victims.push_back(e);
+					cache.total -= e.bytes;
+					cache.entries.erase(it);
+				}
+			}
 		}
-		const int rc = avhip_winograd_weight_transform(ctx.stream, p.w_dtype, mat_dtype, m, 3, p.shape.mode, wm->data, buf, p.shape.K, p.shape.C);
-		const avStatus_t st = from_launcher(rc);
-		if (st != AVOCADO_STATUS_SUCCESS)
-		{
-			(void) hipFree(buf);
-			return st;
-		}
-		cache.entries[key] = buf;
-		*U = buf;
-		return AVOCADO_STATUS_SUCCESS;
+		WeightCache::release(victims);
+		return status;
 	}
 	/* [16, K, C] for the fused kernel: fp16 matrices for 16-bit tensors, fp32 for fp32 */
 	avStatus_t fused_weights(const Context &ctx, const ConvProblem &p, avMemoryDescriptor_t wMem, const void **U)
@@ -692,8 +852,8 @@ namespace
 	{
 		return plan.tiles >= 2048 && p.shape.C >= 64 && p.shape.K >= 64;
 	}
-	avStatus_t run_nonfused_winograd(const ConvCall &c, const NonFusedPlan &plan, Memory *ws, avMemoryDescriptor_t wMem, avMemoryDescriptor_t yMem,
-			avActivationType_t activation)
+	avStatus_t run_nonfused_winograd(const ConvCall &c, const NonFusedPlan &plan, Memory *ws, avMemoryDescriptor_t wMem, avMemoryDescriptor_t wsMem,
+			avMemoryDescriptor_t yMem, avActivationType_t activation)
 	{
 		const avhipConvShape &s = c.problem.shape;
 		char *V = ws->data, *Mx = V + plan.v_bytes;
@@ -702,6 +862,7 @@ namespace
 		const avStatus_t ws_status = cached_winograd_weights(c.ctx, c.problem, wMem, 4, plan.mat_dtype, &U);
 		if (ws_status != AVOCADO_STATUS_SUCCESS)
 			return ws_status;
+		touch(wsMem, 0, plan.total);
 		int rc = avhip_winograd_input_transform(st, AVOCADO_DTYPE_FLOAT32, plan.mat_dtype, 4, 3, c.x->data, V, s.N, s.H, s.W, s.C, s.pad_h, s.pad_w,
 					padding_value_or_null(c.problem.conv));
 		if (rc == 0)
@@ -907,6 +1068,7 @@ namespace avocado
 			m->size = sizeInBytes;
 			m->owning = true;
 			m->uid = next_uid();
+			m->writes.reset(new WriteLog());
 			if (sizeInBytes > 0)
 			{
 				if (hipSetDevice(deviceIndex) != hipSuccess)
@@ -934,6 +1096,7 @@ namespace avocado
 			m->size = sizeInBytes;
 			m->owning = false;
 			m->owner_slot = handle_slot(desc);
+			m->owner_uid = src->uid;
 			m->data = src->data != nullptr ? src->data + offsetInBytes : nullptr;
 			m->uid = next_uid();
 			result[0] = make_handle(KIND_MEMORY, src->device, memories().insert(std::move(m)));
@@ -975,7 +1138,7 @@ namespace avocado
 				return AVOCADO_STATUS_EXECUTION_FAILED;
 			if (dstSize == 0)
 				return AVOCADO_STATUS_SUCCESS;
-			touch(dst);
+			touch(dst, dstOffset, dstSize);
 			avStatus_t st;
 			if (pattern == nullptr)
 			{
@@ -1012,7 +1175,7 @@ namespace avocado
 				return AVOCADO_STATUS_SUCCESS;
 			if (hipSetDevice(ctx.device) != hipSuccess)
 				return AVOCADO_STATUS_EXECUTION_FAILED;
-			touch(dst);
+			touch(dst, dstOffset, count);
 			if (ctx.is_default)
 				return from_hip(hipMemcpy(d->data + dstOffset, s->data + srcOffset, static_cast<size_t>(count), hipMemcpyDeviceToDevice));
 			return from_hip(hipMemcpyAsync(d->data + dstOffset, s->data + srcOffset, static_cast<size_t>(count), hipMemcpyDeviceToDevice, ctx.stream));
@@ -1049,7 +1212,7 @@ namespace avocado
 				return AVOCADO_STATUS_SUCCESS;
 			if (hipSetDevice(ctx.device) != hipSuccess)
 				return AVOCADO_STATUS_EXECUTION_FAILED;
-			touch(dst);
+			touch(dst, dstOffset, bytes);
 			if (ctx.is_default)
 				return from_hip(hipMemcpy(d->data + dstOffset, src, static_cast<size_t>(bytes), hipMemcpyHostToDevice));
 			return from_hip(hipMemcpyAsync(d->data + dstOffset, src, static_cast<size_t>(bytes), hipMemcpyHostToDevice, ctx.stream));
@@ -1193,7 +1356,7 @@ namespace avocado
 				return AVOCADO_STATUS_SUCCESS;
 			if (hipSetDevice(ctx.device) != hipSuccess)
 				return AVOCADO_STATUS_EXECUTION_FAILED;
-			touch(dst);
+			touch(dst, 0, elements * size_of(dstType));
 			return from_launcher(avhip_change_type(ctx.stream, d->data, dstType, s->data, srcType, elements));
 		}
 
@@ -1661,22 +1824,32 @@ namespace avocado
 			Memory *ws = get_memory(workspaceMem);
 			const bool nonfused_ready = nonfused_plan(p, plan) && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32 && ws != nullptr && ws->data != nullptr
 					&& ws->size >= plan.total && reinterpret_cast<uintptr_t>(ws->data) % 256 == 0;
+			/* AVOCADO_STATUS_BAD_ALLOC from a Winograd plan means that the stream is capturing and the transformed weights are not
+			 * in the library's cache yet (nothing was launched): the implicit-GEMM plan needs none and takes over. */
 			if (nonfused_ready && nonfused_preferred(p, plan))
 			{
-				touch(workspaceMem);
-				return run_nonfused_winograd(call, plan, ws, wMem, yMem, activation);
+				const avStatus_t ns = run_nonfused_winograd(call, plan, ws, wMem, workspaceMem, yMem, activation);
+				if (ns != AVOCADO_STATUS_BAD_ALLOC)
+					return ns;
 			}
-			if (fused_winograd_applicable(p) && p.x_dtype == AVOCADO_DTYPE_FLOAT32 && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32
+			else if (fused_winograd_applicable(p) && p.x_dtype == AVOCADO_DTYPE_FLOAT32 && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32
 					&& p.shape.Ho == p.shape.H && p.shape.Wo == p.shape.W && fused_workgroups >= 128)
 			{
 				const avStatus_t fs = run_fused_winograd(call, wMem, yMem, activation);
-				if (fs != AVOCADO_STATUS_NOT_SUPPORTED)
+				if (fs != AVOCADO_STATUS_NOT_SUPPORTED && fs != AVOCADO_STATUS_BAD_ALLOC)
 					return fs;
+				if (fs == AVOCADO_STATUS_NOT_SUPPORTED && nonfused_ready)
+				{
+					const avStatus_t ns = run_nonfused_winograd(call, plan, ws, wMem, workspaceMem, yMem, activation);
+					if (ns != AVOCADO_STATUS_BAD_ALLOC)
+						return ns;
+				}
 			}
-			if (nonfused_ready)
+			else if (nonfused_ready)
 			{
-				touch(workspaceMem);
-				return run_nonfused_winograd(call, plan, ws, wMem, yMem, activation);
+				const avStatus_t ns = run_nonfused_winograd(call, plan, ws, wMem, workspaceMem, yMem, activation);
+				if (ns != AVOCADO_STATUS_BAD_ALLOC)
+					return ns;
 			}
 			return run_implicit_gemm(call, yMem, activation, nullptr);
 		}
@@ -1711,6 +1884,18 @@ namespace avocado
 			if (hipDeviceSynchronize() != hipSuccess)
 				return AVOCADO_STATUS_EXECUTION_FAILED;
 			weight_cache().clear();
+			return AVOCADO_STATUS_SUCCESS;
+		}
+		avStatus_t avhipGetWeightCacheState(av_int64 *entries, av_int64 *bytes, av_int64 *transforms)
+		{
+			WeightCache &cache = weight_cache();
+			std::lock_guard<std::mutex> lock(cache.mutex);
+			if (entries != nullptr)
+				entries[0] = static_cast<av_int64>(cache.entries.size());
+			if (bytes != nullptr)
+				bytes[0] = static_cast<av_int64>(cache.total);
+			if (transforms != nullptr)
+				transforms[0] = static_cast<av_int64>(cache.transforms);
 			return AVOCADO_STATUS_SUCCESS;
 		}
 	} /* namespace backend */

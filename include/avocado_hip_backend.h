@@ -224,11 +224,23 @@ namespace avocado
 					const avTensorDescriptor_t zDesc, const avMemoryDescriptor_t zMem, const void *beta, const avTensorDescriptor_t yDesc,
 					avMemoryDescriptor_t yMem, avActivationType_t activation);
 			/* Interop for harnesses: the HIP stream (hipStream_t) of a context and the device address behind a memory
-			 * descriptor.  Writing through the raw address bypasses the library's change tracking of weight tensors: call
-			 * avhipInvalidateCaches afterwards. */
+			 * descriptor. */
 			DLL_PUBLIC avStatus_t avhipGetContextStream(avContextDescriptor_t context, void **stream);
 			DLL_PUBLIC avStatus_t avhipGetMemoryPointer(avMemoryDescriptor_t mem, void **pointer);
+			/* The Winograd plans (cudaConvolutionWinogradFusedForward, and the dispatcher where it picks one) keep transformed
+			 * weights in library memory, one buffer per weight tensor, and transform again, into the same buffer and on the
+			 * calling stream, when the weight bytes were written through this API since.  What callers must know:
+			 *  - writes the library cannot see (through the raw address, or by a replayed graph): call avhipInvalidateCaches
+			 *    afterwards.  It synchronises the device and frees every buffer, so no captured graph that contains a Winograd
+			 *    call may be replayed after it; capture again.
+			 *  - under stream capture the library neither allocates nor transforms: a Winograd entry whose weights are not cached
+			 *    and up to date returns AVOCADO_STATUS_BAD_ALLOC without launching anything (run the call once outside capture,
+			 *    or use the NoAlloc entry); the dispatcher takes its implicit-GEMM plan instead.
+			 *  - a call on another context than the one whose call transformed the weights waits for that transform by event.
+			 * avhipGetWeightCacheState reports buffers held, their bytes and the number of weight transforms launched so far
+			 * (any pointer may be null). */
 			DLL_PUBLIC avStatus_t avhipInvalidateCaches(void);
+			DLL_PUBLIC avStatus_t avhipGetWeightCacheState(av_int64 *entries, av_int64 *bytes, av_int64 *transforms);
 
 #ifdef __cplusplus
 		} /* extern "C" */
