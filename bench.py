@@ -40,7 +40,13 @@ class Hip:
     """The few HIP runtime calls the harness needs itself: events on a given stream."""
 
     def __init__(self):
-        self.rt = C.CDLL("libamdhip64.so")
+        # symbols are looked up through the backend library, i.e. in the HIP runtime IT is linked against: a process may hold a
+        # second copy of the runtime (PyTorch ships its own), and a stream of one copy means nothing to the other
+        self.rt = cb.load_library()
+        for name in ("hipEventCreate", "hipEventRecord", "hipEventSynchronize", "hipEventElapsedTime", "hipEventDestroy", "hipStreamBeginCapture",
+                     "hipStreamEndCapture", "hipGraphInstantiate", "hipGraphLaunch", "hipGraphExecDestroy", "hipGraphDestroy", "hipDeviceSynchronize",
+                     "hipStreamWaitEvent"):
+            getattr(self.rt, name).restype = C.c_int
         self.rt.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
         self.rt.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
         self.rt.hipEventSynchronize.argtypes = [C.c_void_p]
@@ -74,12 +80,15 @@ class Hip:
         """Records what `enqueue()` launches on `stream` into a HIP graph and returns the executable graph.  The library
         launches plain kernels only (no memset nodes, no allocation once its weight cache is warm), so a step of the tower
         is a chain of 21 kernel nodes that replays without any host work between the kernels."""
-        assert self.rt.hipStreamBeginCapture(stream, 0) == 0  # hipStreamCaptureModeGlobal
+        rc = self.rt.hipStreamBeginCapture(stream, 0)  # hipStreamCaptureModeGlobal
+        assert rc == 0, "hipStreamBeginCapture: error %d" % rc
         enqueue()
         graph = C.c_void_p()
-        assert self.rt.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        rc = self.rt.hipStreamEndCapture(stream, C.byref(graph))
+        assert rc == 0, "hipStreamEndCapture: error %d" % rc
         exe = C.c_void_p()
-        assert self.rt.hipGraphInstantiate(C.byref(exe), graph, None, None, 0) == 0
+        rc = self.rt.hipGraphInstantiate(C.byref(exe), graph, None, None, 0)
+        assert rc == 0, "hipGraphInstantiate: error %d" % rc
         self.rt.hipGraphDestroy(graph)
         return exe
 
@@ -308,22 +317,25 @@ def int8_leg(hip, ctx, iters):
     return out
 
 
-def nonfused_stages(hip, ctx, dtype, mat_dtype, m, iters):
-    """The four-call non-fused Winograd sequence on the body convolution of config 2, one timing per stage."""
+def nonfused_stages(hip, ctx, dtype, mat_dtype, m, iters, shape=(256, 15, 128), acc_dtype="f32"):
+    """The four-call non-fused Winograd sequence F(m x m, 3x3) on one layer, one timing per stage.  shape = (N, H = W, C = K):
+    the body convolution of config 2 by default, (64, 56, 256) for config 3.  mat_dtype: U and V, acc_dtype: M.
+    Algorithmic bytes per stage: input x + V; GEMM V + U + M; output M + y + bias (weight transform w + U).  The GEMM stage is
+    reported against the MFMA peak and against min(MFMA peak, arithmetic intensity x 8 TB/s), the roof a product that streams V
+    and M through HBM has."""
     lib = cb.load_library()
     g = np.random.default_rng(SEED + 5)
-    N, HW, ch = 256, 15, 128
-    d, md = DT[dtype], DT[mat_dtype]
+    N, HW, ch = shape
+    d, md, ad = DT[dtype], DT[mat_dtype], DT[acc_dtype]
     t = m + 2
     tiles = N * ((HW + m - 1) // m) ** 2
-    esz, msz = cb.DTYPE_SIZE[d], cb.DTYPE_SIZE[md]
+    esz, msz, asz = cb.DTYPE_SIZE[d], cb.DTYPE_SIZE[md], cb.DTYPE_SIZE[ad]
     x = cb.DeviceTensor.from_numpy(g.standard_normal((N, HW, HW, ch)).astype(np.float32), d)
     w = cb.DeviceTensor.from_numpy((g.standard_normal((ch, 3, 3, ch)) * np.sqrt(2.0 / (9 * ch))).astype(np.float32), d)
     b = cb.DeviceTensor.from_numpy(g.uniform(-0.1, 0.1, ch).astype(np.float32), cb.DTYPE_FLOAT32)
     U = cb.DeviceTensor((t * t, ch, ch), md)
     V = cb.DeviceTensor((t * t, tiles, ch), md)
-    acc_dtype = cb.DTYPE_FLOAT32
-    Mx = cb.DeviceTensor((t * t, tiles, ch), acc_dtype)
+    Mx = cb.DeviceTensor((t * t, tiles, ch), ad)
     y = cb.DeviceTensor((N, HW, HW, ch), d)
     conv = cb.ConvolutionDescriptor(padding=(-1, -1), dtype=d)
     h = ctx.handle
@@ -336,16 +348,24 @@ def nonfused_stages(hip, ctx, dtype, mat_dtype, m, iters):
     }
     xbytes = N * HW * HW * ch * esz
     alg_bytes = {"weight_transform": ch * 9 * ch * esz + t * t * ch * ch * msz, "input_transform": xbytes + t * t * tiles * ch * msz,
-                 "gemm": t * t * tiles * ch * msz + t * t * ch * ch * msz + t * t * tiles * ch * 4, "output_transform": t * t * tiles * ch * 4 + xbytes + 4 * ch}
+                 "gemm": t * t * tiles * ch * msz + t * t * ch * ch * msz + t * t * tiles * ch * asz,
+                 "output_transform": t * t * tiles * ch * asz + xbytes + 4 * ch}
     gemm_flops = 2.0 * t * t * tiles * ch * ch
-    out = {}
+    out = {"shape": {"N": N, "HW": HW, "channels": ch, "tiles": tiles}, "matrices": mat_dtype, "M": acc_dtype}
     total = 0.0
     for name, fn in calls.items():
         ms = time_calls(hip, ctx, fn, iters)
-        rec = {"us": ms * 1e3, "GBs": alg_bytes[name] / (ms * 1e-3) / 1e9, "hbm_frac": alg_bytes[name] / (ms * 1e-3) / 1e9 / PEAK["hbm_GBs"]}
+        rec = {"us": ms * 1e3, "MB": alg_bytes[name] / 1e6, "GBs": alg_bytes[name] / (ms * 1e-3) / 1e9,
+               "hbm_frac": alg_bytes[name] / (ms * 1e-3) / 1e9 / PEAK["hbm_GBs"]}
         if name == "gemm":
+            rec["gflop"] = gemm_flops / 1e9
             rec["tflops"] = gemm_flops / (ms * 1e-3) / 1e12
             rec["mfma_frac"] = rec["tflops"] / PEAK[mat_dtype]
+            intensity = gemm_flops / alg_bytes[name]
+            roof = min(PEAK[mat_dtype], intensity * PEAK["hbm_GBs"] / 1e3)
+            rec["flop_per_byte"] = intensity
+            rec["roof_min_mfma_hbm_tflops"] = roof
+            rec["frac_of_that_roof"] = rec["tflops"] / roof
         out[name] = rec
         if name != "weight_transform":
             total += ms
@@ -564,6 +584,14 @@ def main():
         detail["int8_config4"] = int8_leg(hip, ctx, it)
         detail["nonfused_winograd_f32_F4"] = nonfused_stages(hip, ctx, "f32", "f32", 4, it)
         detail["nonfused_winograd_bf16_F2_fp16mat"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it)
+        detail["nonfused_winograd_f16_F2_fp16mat_fp16M"] = nonfused_stages(hip, ctx, "f16", "f16", 2, it, acc_dtype="f16")
+        cfg3 = (64, 56, 256)
+        detail["config3_nonfused_winograd"] = {
+            "bf16_F2_fp16mat": nonfused_stages(hip, ctx, "bf16", "f16", 2, it, shape=cfg3),
+            "f16_F2_fp16mat_fp16M": nonfused_stages(hip, ctx, "f16", "f16", 2, it, shape=cfg3, acc_dtype="f16"),
+            "bf16_F4_fp32mat": nonfused_stages(hip, ctx, "bf16", "f32", 4, it, shape=cfg3),
+            "f16_F4_fp32mat": nonfused_stages(hip, ctx, "f16", "f32", 4, it, shape=cfg3),
+        }
         detail["copy_GBs_measured"] = copy_bandwidth(hip, ctx)
         detail["stream_GBs_measured"] = stream_rates(hip, ctx)
         detail["mfma_rate_measured"] = mfma_rates(hip, ctx)

@@ -8,6 +8,7 @@
  */
 #include "conv_pointwise.hpp"
 #include "persistent_gemm.hpp"
+#include "resident_gemm.hpp"
 
 namespace
 {
@@ -19,6 +20,27 @@ namespace
 		__shared__ __attribute__((aligned(16))) char lds[PERSISTENT_LDS_BYTES];
 		persistent_nt_gemm<TE, Epi, STEPS>(lds, x, w, g, epi);
 	}
+
+	/* the same product with the filters resident in registers and only x streaming (resident_gemm.hpp) */
+	template<typename TE, typename Epi, int STEPS>
+	__global__ __launch_bounds__(256, RESIDENT_OCCUPANCY) void k_conv_pointwise_resident(const TE *__restrict__ x, const TE *__restrict__ w, ResidentGeom g, Epi epi)
+	{
+		__shared__ __attribute__((aligned(16))) char lds[RESIDENT_LDS_BYTES];
+		resident_nt_gemm<TE, Epi, STEPS>(lds, x, w, g, epi);
+	}
+}
+
+namespace avhip
+{
+	std::atomic<int>& short_k_engine()
+	{
+		static std::atomic<int> engine { 0 };
+		return engine;
+	}
+}
+extern "C" int avhip_set_short_k_engine(int engine)
+{
+	return avhip::short_k_engine().exchange(engine == 1 ? 1 : 0);
 }
 
 namespace avhip
@@ -38,6 +60,32 @@ namespace avhip
 		const int64_t tiles = row_blocks * col_blocks;
 		if (pixels >= (1ll << 31) - BLOCK_M || tiles >= (1ll << 31) - 1024 || s.K >= (1 << 22))
 			return false;
+		const unsigned int x_row_bytes = static_cast<unsigned int>(s.C) * static_cast<unsigned int>(sizeof(TE));
+		const int x_steps = static_cast<int>((x_row_bytes + STEP_BYTES - 1) / STEP_BYTES);
+		if (short_k_engine().load(std::memory_order_relaxed) == 0 && x_steps <= RESIDENT_MAX_STEPS && x_row_bytes % 16 == 0
+				&& static_cast<size_t>(s.K) * sizeof(typename Epi::template ColumnsT<1>) <= static_cast<size_t>(RESIDENT_TABLE_BYTES))
+		{
+			ResidentGeom r;
+			r.rows = static_cast<int>(pixels);
+			r.cols = s.K;
+			r.row_bytes = x_row_bytes;
+			r.a_pitch = r.b_pitch = x_row_bytes;
+			r.a_batch = r.b_batch = 0;
+			r.a_bytes = static_cast<unsigned int>(pixels) * x_row_bytes; /* the caller vouches for tensors below 2 GiB */
+			r.b_bytes = static_cast<unsigned int>(s.K) * x_row_bytes;
+			r.c_batch = 0;
+			r.c_pitch = s.K;
+			r.table_columns = s.K;
+			const dim3 grid(resident_plan(r, 1));
+			const TE *xp = static_cast<const TE*>(x), *wp = static_cast<const TE*>(w);
+			if (x_steps == 1)
+				hipLaunchKernelGGL((k_conv_pointwise_resident<TE, Epi, 1>), grid, dim3(256), 0, stream, xp, wp, r, epi);
+			else if (x_steps == 2)
+				hipLaunchKernelGGL((k_conv_pointwise_resident<TE, Epi, 2>), grid, dim3(256), 0, stream, xp, wp, r, epi);
+			else
+				hipLaunchKernelGGL((k_conv_pointwise_resident<TE, Epi, 4>), grid, dim3(256), 0, stream, xp, wp, r, epi);
+			return true;
+		}
 		PersistentGeom g;
 		g.rows = static_cast<int>(pixels);
 		g.cols = s.K;

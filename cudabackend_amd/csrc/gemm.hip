@@ -13,6 +13,7 @@
 
 #include "mfma_core.hpp"
 #include "persistent_gemm.hpp"
+#include "resident_gemm.hpp"
 
 namespace
 {
@@ -152,6 +153,9 @@ namespace
 		template<int W> struct ColumnsT
 		{
 		};
+		template<int W> struct Residual /* C has no residual term */
+		{
+		};
 		TC *c;
 		float alpha, beta;
 		__device__ __forceinline__ void pin()
@@ -221,6 +225,13 @@ namespace
 	{
 		__shared__ __attribute__((aligned(16))) char lds[PERSISTENT_LDS_BYTES];
 		persistent_nt_gemm<TE, GemmEpilogue<TC>, STEPS, TM>(lds, A, B, g, epi);
+	}
+
+	template<typename TE, typename TC, int STEPS>
+	__global__ __launch_bounds__(256, RESIDENT_OCCUPANCY) void k_gemm_nt_resident(const TE *__restrict__ A, const TE *__restrict__ B, ResidentGeom g, GemmEpilogue<TC> epi)
+	{
+		__shared__ __attribute__((aligned(16))) char lds[RESIDENT_LDS_BYTES];
+		resident_nt_gemm<TE, GemmEpilogue<TC>, STEPS>(lds, A, B, g, epi);
 	}
 
 	/* Any operand form, any supported type: 16 x 16 outputs per workgroup, k in slices of 16 through LDS. */
@@ -303,6 +314,32 @@ namespace
 			const int64_t tiles = row_blocks * col_blocks * batch;
 			if (sA < 0 || sB < 0 || a_bytes >= (1ll << 31) || b_bytes >= (1ll << 31) || tiles >= (1ll << 31) - 1024)
 				return false;
+			if (short_k_engine().load(std::memory_order_relaxed) == 0 && row_bytes % 16 == 0 && steps <= RESIDENT_MAX_STEPS)
+			{
+				ResidentGeom r;
+				r.rows = M;
+				r.cols = N;
+				r.row_bytes = static_cast<unsigned int>(row_bytes);
+				r.a_pitch = static_cast<unsigned int>(lda * sizeof(TE));
+				r.b_pitch = static_cast<unsigned int>(ldb * sizeof(TE));
+				r.a_batch = static_cast<unsigned int>(sA * sizeof(TE));
+				r.b_batch = static_cast<unsigned int>(sB * sizeof(TE));
+				r.a_bytes = static_cast<unsigned int>(a_bytes);
+				r.b_bytes = static_cast<unsigned int>(b_bytes);
+				r.c_batch = sC;
+				r.c_pitch = ldc;
+				r.table_columns = 0;
+				const Epi epi { static_cast<TC*>(C), static_cast<float>(alpha), static_cast<float>(beta) };
+				const dim3 grid(resident_plan(r, batch));
+				const TE *ap = static_cast<const TE*>(A), *bp = static_cast<const TE*>(B);
+				if (steps == 1)
+					hipLaunchKernelGGL((k_gemm_nt_resident<TE, TC, 1>), grid, dim3(256), 0, s, ap, bp, r, epi);
+				else if (steps == 2)
+					hipLaunchKernelGGL((k_gemm_nt_resident<TE, TC, 2>), grid, dim3(256), 0, s, ap, bp, r, epi);
+				else
+					hipLaunchKernelGGL((k_gemm_nt_resident<TE, TC, 4>), grid, dim3(256), 0, s, ap, bp, r, epi);
+				return true;
+			}
 			PersistentGeom g;
 			g.rows = M;
 			g.cols = N;

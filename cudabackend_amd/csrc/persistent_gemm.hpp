@@ -320,6 +320,10 @@ namespace avhip
 		}
 	}
 
+	/* Which engine runs short-k NT products (1x1 convolutions, the batched GEMM of non-fused Winograd): 0 = B resident in
+	 * registers (resident_gemm.hpp, the default), 1 = both operands through LDS (this file).  Set by avhip_set_short_k_engine. */
+	std::atomic<int>& short_k_engine();
+
 	/* How many workgroups to launch: two per compute unit stay resident; with fewer tiles every workgroup has one. */
 	inline unsigned int persistent_workgroups(int64_t tiles)
 	{

@@ -124,6 +124,12 @@ extern "C"
 	 * the 256 compute units of an MI355X; 0 never uses that kernel).  Returns the previous value.  Process-wide. */
 	AVHIP_API int avhip_set_small_problem_threshold(int workgroups);
 
+	/* Tuning knob without a counterpart in the reference.  Products with a short k (at most 512 bytes per operand row: 1x1
+	 * convolutions, the batched GEMM of non-fused Winograd) run on one of two engines: 0 (default) keeps the B operand (filters,
+	 * transformed weights) in registers and streams only A through LDS; 1 passes both operands through LDS.  Returns the previous
+	 * value.  Process-wide. */
+	AVHIP_API int avhip_set_short_k_engine(int engine);
+
 	/* Measurement aid without a counterpart in the reference: keeps every matrix core busy with register-resident
 	 * 32x32 MFMAs of `dtype` (FLOAT16, BFLOAT16, INT8 or FLOAT32) and nothing else, so that a harness can time the rate the
 	 * matrix cores sustain on this machine (clock under load included) next to the datasheet peak.  operands = 0: nearly

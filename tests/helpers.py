@@ -11,6 +11,16 @@ DT = {"f16": cb.DTYPE_FLOAT16, "bf16": cb.DTYPE_BFLOAT16, "f32": cb.DTYPE_FLOAT3
 SEED = 0xA70CAD0
 
 
+def short_k_engine_fixture(request):
+    """Body of a parametrised autouse fixture: runs a test once per engine of the short-k products (1x1 convolutions, Winograd's
+    batched GEMM): B operand resident in registers (the default) and both operands through LDS."""
+    lib = cb.load_library()
+    lib.avhip_set_short_k_engine.restype = int
+    previous = lib.avhip_set_short_k_engine(1 if request.param == "both_through_lds" else 0)
+    yield
+    lib.avhip_set_short_k_engine(previous)
+
+
 def rng(offset=0):
     return np.random.default_rng(SEED + offset)
 
@@ -242,3 +252,27 @@ def batchnorm_inference(x, scale, bias, mean, var, dtype, y0=None, alpha=None, b
         assert st == expect, cb.STATUS_NAMES[st]
         c.finish()
         return y.download() if st == cb.STATUS_SUCCESS else None
+
+
+def winograd_nonfused(x, w, dtype, m, mat_dtype, acc_dtype, bias=None, z=None, activation=0, pad=(-1, -1), mode=0):
+    """The four-call non-fused Winograd sequence with the matrices staying on the device, as a front-end runs it
+    (src/winograd_nonfused.cu:881,906,932 and src/gemm.cpp:126 of the reference): weight transform, input transform, batched GEMM
+    M = V U^T, output transform with the fused epilogue.  mat_dtype: dtype of U and V, acc_dtype: dtype of M."""
+    N, H, W, Cin = x.shape
+    K, r = w.shape[0], w.shape[1]
+    t = m + r - 1
+    tiles = N * ((H + m - 1) // m) * ((W + m - 1) // m)
+    with Call() as c:
+        conv = cb.ConvolutionDescriptor(mode=mode, padding=pad, dtype=DT[dtype])
+        xt, wt = c.tensor(x, dtype), c.tensor(w, dtype)
+        b, zt = c.tensor(bias, "f32"), c.tensor(z, dtype)
+        U, V, M = c.empty((t * t, K, Cin), mat_dtype), c.empty((t * t, tiles, Cin), mat_dtype), c.empty((t * t, tiles, K), acc_dtype)
+        y = c.empty((N, H, W, K), dtype)
+        hdl = c.ctx.handle
+        cb.check(c.lib.cudaWinogradWeightTransform(hdl, conv.handle, m, wt.desc, wt.mem, U.desc, U.mem), "weight transform")
+        cb.check(c.lib.cudaWinogradInputTransform(hdl, conv.handle, m, wt.desc, xt.desc, xt.mem, V.desc, V.mem), "input transform")
+        cb.check(c.lib.cudaGemmBatched(hdl, 0, 1, None, V.desc, V.mem, U.desc, U.mem, None, M.desc, M.mem), "batched GEMM")
+        cb.check(c.lib.cudaWinogradOutputTransform(hdl, conv.handle, m, wt.desc, None, M.desc, M.mem, y.desc, y.mem, _d(b), _m(b), None, _d(zt), _m(zt), None,
+                                                   activation), "output transform")
+        c.finish()
+        return y.download()

@@ -81,6 +81,23 @@ def test_config3_large_spatial(oracle, dtype):
     assert oracle.rel_l2(fused, direct) < 2 * BAR[dtype]
 
 
+@pytest.mark.parametrize("dtype,m,mat,acc", [("bf16", 2, "f16", "f32"), ("f16", 2, "f16", "f32"), ("f16", 2, "f16", "f16"), ("bf16", 4, "f32", "f32"),
+                                               ("f16", 4, "f32", "f32")])
+def test_config3_nonfused_winograd(oracle, dtype, m, mat, acc):
+    """N=64, 56x56, 256->256 as the four-call non-fused Winograd sequence (src/winograd_nonfused.cu:906,932, src/gemm.cpp:126-209 of
+    the reference; call order of app/CudaBackend.cu:401-420), matrices resident on the device: F(2x2,3x3) with fp16 matrices (and
+    fp16 M for fp16 tensors), F(4x4,3x3) with fp32 matrices, bias + ReLU fused in the output transform; sampled images against the
+    oracle at the 16-bit bar 2e-3."""
+    g = h.rng(45)
+    N = 64
+    x = h.rounded(oracle, g.standard_normal((N, 56, 56, 256)), dtype)
+    w = h.rounded(oracle, he(g, (256, 3, 3, 256)), dtype)
+    b = g.uniform(-0.1, 0.1, 256).astype(np.float32).astype(np.float64)
+    print("config 3 non-fused", dtype, "F(%d,3)" % m, "matrices", mat, "M", acc, flush=True)
+    got = h.winograd_nonfused(x, w, dtype, m, mat, acc, bias=b, activation=cb.ACTIVATION_RELU)
+    check_images(oracle, got, x, w, b, None, (0, 37, 63), BAR[dtype])
+
+
 def test_config4_int8(oracle):
     """N=128, 20x20, 128->128 int8: sampled images exact, requantised exact, linearity in the weights and delta kernels exact."""
     g = h.rng(43)

@@ -9,7 +9,12 @@ import helpers as h
 
 pytestmark = pytest.mark.gpu
 
-TOL = {"f64": 1e-12, "f32": 2e-6, "f16": 1e-3, "bf16": 8e-3}
+
+@pytest.fixture(autouse=True, params=["b_resident", "both_through_lds"])
+def short_k_engine(request):
+    yield from h.short_k_engine_fixture(request)
+
+TOL = {"f64": 1e-12, "f32": 2e-6, "f16": 4e-4, "bf16": 3e-3}  # 16-bit: the rounding of the result itself is 2.1e-4 / 1.7e-3 rel-L2
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32", "f64"])

@@ -10,6 +10,11 @@ import helpers as h
 
 pytestmark = pytest.mark.gpu
 
+
+@pytest.fixture(autouse=True, params=["b_resident", "both_through_lds"])
+def short_k_engine(request):
+    yield from h.short_k_engine_fixture(request)
+
 BAR = {"f32": 1e-5, "f16": 2e-3, "bf16": 2e-3}
 
 FLOAT_CASES = [
@@ -19,6 +24,8 @@ FLOAT_CASES = [
     ("f32", (4, 63, 63, 96), 520, "bias+beta"),       # 125 x 5 = 625 tiles, 3 k-steps
     ("bf16", (3, 75, 75, 256), 512, "bias+relu"),     # 132 x 4 = 528 tiles, 4 k-steps
     ("f32", (1, 40, 40, 32), 136, "bias+relu"),       # 13 x 2 tiles: fewer tiles than resident workgroups
+    ("bf16", (1, 37, 41, 64), 72, "bias+z+relu"),     # one step; 1517 pixels: ranges that end in a partial granule
+    ("f16", (2, 100, 100, 128), 128, "bias+relu"),    # two steps, one column block: 512 ranges of 40 rows (one short tile each)
 ]
 
 
