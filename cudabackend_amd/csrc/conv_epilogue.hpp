@@ -78,6 +78,29 @@ namespace avhip
 			for (int q = 0; q < W; q++)
 				c.bias[q] = (bias != nullptr && k + q < K) ? bias[k + q] : 0.0f;
 		}
+		/* The same constants requested with 16-byte buffer loads and nothing else: filters past the last one and an absent bias
+		 * read zeros through the buffer's bounds, so no instruction between here and the epilogue depends on the loaded values
+		 * and a kernel does not wait for them before its k loop (a select on a loaded value would sit in the prologue and wait
+		 * there).  k a multiple of 4, bias 16-byte aligned; finish_columns() before the first use. */
+		template<int W>
+		__device__ __forceinline__ void request_columns(int k, ColumnsT<W> &c) const
+		{
+			static_assert(W % 4 == 0, "whole 16-byte runs");
+			const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(bias), 0, bias != nullptr ? K * 4 : 0, 0x00020000);
+#pragma unroll
+			for (int part = 0; part < W / 4; part++)
+			{
+				typedef float f32x4 __attribute__((ext_vector_type(4)));
+				const f32x4 v = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rb, (k + 4 * part) * 4, 0, 0));
+#pragma unroll
+				for (int q = 0; q < 4; q++)
+					c.bias[4 * part + q] = v[q];
+			}
+		}
+		template<int W>
+		__device__ __forceinline__ void finish_columns(ColumnsT<W>&) const
+		{
+		}
 		/* the same constants out of a table of one-filter records (a kernel that walks several filter blocks stages
 		 * load_columns(k, table[k]) for every k in LDS once) */
 		template<int W>
@@ -301,6 +324,57 @@ namespace avhip
 				sc = (sc == sc) ? sc : 0.0f;
 				sc = sc > 3.0e38f ? 3.0e38f : (sc < -3.0e38f ? -3.0e38f : sc);
 				c.scale[q] = sc;
+			}
+		}
+		/* Requested with 16-byte buffer loads and left untouched until finish_columns() (see FloatEpilogue::request_columns):
+		 * k a multiple of 4, bias and scale 16-byte aligned. */
+		template<int W>
+		__device__ __forceinline__ void request_columns(int k, ColumnsT<W> &c) const
+		{
+			static_assert(W % 4 == 0, "whole 16-byte runs");
+			const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(bias), 0, bias != nullptr ? K * 4 : 0, 0x00020000);
+			const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(scale), 0, (MODE == I8_REQUANT && scale != nullptr) ? K * 4 : 0,
+					0x00020000);
+#pragma unroll
+			for (int part = 0; part < W / 4; part++)
+			{
+				typedef float f32x4 __attribute__((ext_vector_type(4)));
+				typedef int i32x4 __attribute__((ext_vector_type(4)));
+				const auto raw = __builtin_amdgcn_raw_buffer_load_b128(rb, (k + 4 * part) * 4, 0, 0);
+#pragma unroll
+				for (int q = 0; q < 4; q++)
+				{
+					c.ibias[4 * part + q] = MODE <= I8_REQUANT ? __builtin_bit_cast(i32x4, raw)[q] : 0;
+					c.fbias[4 * part + q] = MODE > I8_REQUANT ? __builtin_bit_cast(f32x4, raw)[q] : 0.0f;
+				}
+				if (MODE == I8_REQUANT)
+				{
+					const f32x4 sv = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (k + 4 * part) * 4, 0, 0));
+#pragma unroll
+					for (int q = 0; q < 4; q++)
+						c.scale[4 * part + q] = sv[q];
+				}
+				else
+				{
+#pragma unroll
+					for (int q = 0; q < 4; q++)
+						c.scale[4 * part + q] = 0.0f;
+				}
+			}
+		}
+		/* the clean-up of the scales that load_columns does at once (NaN -> 0, infinities -> the largest finite value) */
+		template<int W>
+		__device__ __forceinline__ void finish_columns(ColumnsT<W> &c) const
+		{
+			if (MODE == I8_REQUANT)
+			{
+#pragma unroll
+				for (int q = 0; q < W; q++)
+				{
+					float sc = c.scale[q];
+					sc = (sc == sc) ? sc : 0.0f;
+					c.scale[q] = sc > 3.0e38f ? 3.0e38f : (sc < -3.0e38f ? -3.0e38f : sc);
+				}
 			}
 		}
 		template<int W>

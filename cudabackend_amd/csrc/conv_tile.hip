@@ -30,6 +30,17 @@
 #include "mfma_core.hpp"
 #include <type_traits>
 
+#ifdef CONV_TILE_STAMPS
+__device__ unsigned long long g_stamps[4096 * 8];
+#define STAMP(i) do { if (threadIdx.x == 0) g_stamps[((blockIdx.y * gridDim.x + blockIdx.x) % 4096) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+extern "C" __attribute__((visibility("default"))) int avhip_debug_stamps(void *out)
+{
+	return static_cast<int>(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_stamps), sizeof(g_stamps)));
+}
+#else
+#define STAMP(i) do { } while (0)
+#endif
+
 namespace
 {
 	using namespace avhip;
@@ -63,12 +74,14 @@ namespace
 	template<typename TE, typename Epi, int FS>
 	__global__ __launch_bounds__(256, 2) void k_conv_tile(const TE *__restrict__ x, const TE *__restrict__ w, TileGeom g, Epi epi)
 	{
+		STAMP(0);
 		epi.pin();
 		keep_in_sgpr(g.TW);
 		keep_in_sgpr(g.TH);
 		keep_in_sgpr(g.Ho);
 		keep_in_sgpr(g.Wo);
 		keep_in_sgpr(g.K);
+		STAMP(6);
 		__shared__ __attribute__((aligned(16))) char lds[TILE_LDS];
 		char *halo = lds;
 		char *filt = lds + HALO_BYTES;
@@ -159,43 +172,40 @@ namespace
 		fetch_filters(fr[0]);
 		fetch_filters(fr[1]);
 		fetch_filters(fr[2]);
+		STAMP(7);
 		/* where this work-item's halo chunks come from (slice 0).  Integer division by a run-time divisor costs about thirty
 		 * instructions and a 32-bit multiply four issue slots: the work-item divides once and then walks, position and byte
 		 * offset alike (the offset of a pixel outside the image is never used; inside the image it is below 2 GiB and the
 		 * additions are exact modulo 2^32). */
 		{
+			/* Ten independent address computations, none waiting for another and none behind a branch: vector instructions of a
+			 * wavefront issue every fourth clock and two wavefronts share a SIMD, so every instruction here is eight clocks of
+			 * the time before the first MFMA.  The halo position divides by the halo width with a 24-bit multiplication. */
 			constexpr int STRIDE = 256 / STEP_CHUNKS; /* halo pixels between two fetches of a work-item */
-			const int dy = over_halo_width(STRIDE), dx = STRIDE - dy * g.HW;
-			const unsigned int pixel_bytes = static_cast<unsigned int>(g.C) * SZ, line_bytes = static_cast<unsigned int>(g.W) * pixel_bytes;
-			const unsigned int step_bytes = dy * line_bytes + dx * pixel_bytes, wrap_bytes = line_bytes - g.HW * pixel_bytes;
-			int h = tid / STEP_CHUNKS;
-			const int hy = over_halo_width(h);
-			int hx = h - hy * g.HW;
+			const unsigned int pixel_bytes = static_cast<unsigned int>(g.C) * SZ;
 			const bool first_slice_exists = chunk_channel < g.C;
-			int ih = oh0 + g.pad_h + hy, iw = ow0 + g.pad_w + hx;
-			unsigned int offset = static_cast<unsigned int>((n * g.H + ih) * g.W + iw) * pixel_bytes + static_cast<unsigned int>(chunk_channel) * SZ;
+			const unsigned int line_bytes = static_cast<unsigned int>(g.W) * pixel_bytes;
+			const int ih0 = oh0 + g.pad_h, iw0 = ow0 + g.pad_w;
+			/* byte offset of halo pixel (0, 0), which may lie outside the image: the sum with a pixel's (hy, hx) part is exact
+			 * modulo 2^32 and only used when the pixel is inside */
+			const unsigned int base = (static_cast<unsigned int>(n) * static_cast<unsigned int>(g.H) + static_cast<unsigned int>(ih0)) * line_bytes
+					+ static_cast<unsigned int>(iw0) * pixel_bytes + static_cast<unsigned int>(chunk_channel) * SZ;
 #pragma unroll
 			for (int f = 0; f < HALO_FETCHES; f++)
 			{
-				const bool inside = (h < halo_pixels) & (static_cast<unsigned int>(ih) < static_cast<unsigned int>(g.H))
-						& (static_cast<unsigned int>(iw) < static_cast<unsigned int>(g.W));
+				const unsigned int h = static_cast<unsigned int>(tid / STEP_CHUNKS + f * STRIDE);
+				const unsigned int hy = __umul24(h, g.hw_magic) >> 20; /* h < 512, hw_magic <= 2^20 / 3 + 1 */
+				const unsigned int hx = h - __umul24(hy, static_cast<unsigned int>(g.HW));
+				const bool inside = (h < static_cast<unsigned int>(halo_pixels)) & (static_cast<unsigned int>(ih0) + hy < static_cast<unsigned int>(g.H))
+						& (static_cast<unsigned int>(iw0) + hx < static_cast<unsigned int>(g.W));
+				/* both factors of either product are below 2^24 (the launcher checks the row and pixel sizes) */
+				const unsigned int offset = base + __umul24(hy, line_bytes) + __umul24(hx, pixel_bytes);
 				halo_src[f] = inside ? offset : OUT_OF_RANGE;
 				hr[f] = buffer_fetch(rx, first_slice_exists ? halo_src[f] : OUT_OF_RANGE); /* slice 0 goes out as soon as its address exists */
-				h += STRIDE;
-				ih += dy;
-				iw += dx;
-				hx += dx;
-				offset += step_bytes;
-				if (hx >= g.HW)
-				{
-					hx -= g.HW;
-					iw -= g.HW;
-					ih++;
-					offset += wrap_bytes;
-				}
 			}
 		}
-		epi.load_columns(kcol, columns); /* needed in the epilogue only: behind everything the first MFMA waits for */
+		STAMP(4);
+		epi.request_columns(kcol, columns); /* needed in the epilogue only: behind everything the first MFMA waits for, and nothing waits for it */
 		int *row_table = reinterpret_cast<int*>(lds + ROW_TABLE);
 		{
 			/* GEMM row -> offset of its output pixel inside the image of y, in elements; -1 for rows that are not stored */
@@ -209,13 +219,16 @@ namespace
 		const int b_off = (lane & 31) * LDS_ROW + (lane >> 5) * 16;
 
 		typename Mma<TE>::acc_t acc[2][2];
+		if constexpr (FS == 0)
+		{
 #pragma unroll
-		for (int i = 0; i < 2; i++)
+			for (int i = 0; i < 2; i++)
 #pragma unroll
-			for (int j = 0; j < 2; j++)
+				for (int j = 0; j < 2; j++)
 #pragma unroll
-				for (int v = 0; v < 16; v++)
-					acc[i][j][v] = 0;
+					for (int v = 0; v < 16; v++)
+						acc[i][j][v] = 0;
+		}
 
 		/* compute side */
 		int c_slice = 0, c_i = 0, c_j = 0;
@@ -267,6 +280,7 @@ namespace
 			a_off[tm] = (wave * 64 + tm * 32 + (lane & 31)) * PIXEL_PITCH + (lane >> 5) * 16;
 		stash_halo(hr);
 		stash_filters(0, fr[0]);
+		STAMP(5);
 
 		/* The residual of every row this work-item will store is requested during the last channel slice: its latency and its
 		 * HBM traffic run under the MFMAs of that slice instead of in the epilogue, and the registers are held for half the
@@ -395,13 +409,21 @@ namespace
 					}
 				}
 			};
-			auto slice_steps = [&](int slice, auto is_last) __attribute__((always_inline))
+			/* FIRST: the very first MFMA of each accumulator starts from the constant zero, so the 64 accumulator registers are
+			 * not cleared (64 moves per wavefront, right on the way to the first MFMA: they share registers with the staged
+			 * halo and cannot be hoisted above the loads' arrival) */
+			auto slice_steps = [&](int slice, auto is_first, auto is_last) __attribute__((always_inline))
 			{
+				constexpr bool FIRST = decltype(is_first)::value;
 				constexpr bool LAST = decltype(is_last)::value;
 #pragma unroll
 				for (int tap = 0; tap < TAPS; tap++)
 				{
 					__syncthreads(); /* ring[(tap + 1) % 3] and, at tap 0, the halo are visible; everyone is done with the step before */
+#ifdef CONV_TILE_STAMPS
+					if (tap == 0 && slice == 0)
+						STAMP(1);
+#endif
 					if (tap == 0)
 						read(0, 0, a[0], bq[0]); /* the halo changed under the barrier above: nothing could be read ahead */
 #pragma unroll
@@ -416,7 +438,12 @@ namespace
 						for (int tm = 0; tm < 2; tm++)
 #pragma unroll
 							for (int tn = 0; tn < 2; tn++)
-								Mma<TE>::run(a[slab & 1][tm], bq[slab & 1][tn], acc[tm][tn]);
+							{
+								if (FIRST && tap == 0 && slab == 0)
+									Mma<TE>::start(a[slab & 1][tm], bq[slab & 1][tn], acc[tm][tn]);
+								else
+									Mma<TE>::run(a[slab & 1][tm], bq[slab & 1][tn], acc[tm][tn]);
+							}
 						if (slab + 1 == SLABS)
 							__builtin_amdgcn_s_setprio(0);
 					}
@@ -444,9 +471,15 @@ namespace
 					stash_halo(hr);
 				}
 			};
-			for (int slice = 0; slice + 1 < g.slices; slice++)
-				slice_steps(slice, std::false_type());
-			slice_steps(g.slices - 1, std::true_type());
+			if (g.slices == 1)
+				slice_steps(0, std::true_type(), std::true_type());
+			else
+			{
+				slice_steps(0, std::true_type(), std::false_type());
+				for (int slice = 1; slice + 1 < g.slices; slice++)
+					slice_steps(slice, std::false_type(), std::false_type());
+				slice_steps(g.slices - 1, std::false_type(), std::true_type());
+			}
 		}
 		else
 		for (int s = 0; s < total; s += 6)
@@ -459,6 +492,8 @@ namespace
 			step(s + 5, 1, fr[2], fr[0]);
 		}
 
+		STAMP(2);
+		epi.finish_columns(columns);
 		if constexpr (std::is_same<Epi, FloatEpilogue<TE>>::value && sizeof(TE) == 2)
 		{
 			/* 16-bit tensors with beta = 0: the epilogue without a single branch.  Which of the four forms (ReLU, residual) is
@@ -489,6 +524,7 @@ namespace
 					drain(std::false_type(), std::true_type());
 				else
 					drain(std::false_type(), std::false_type());
+				STAMP(3);
 				return;
 			}
 		}
@@ -498,6 +534,16 @@ namespace
 			if (e >= 0 && kcol < g.K)
 				epi.template store_at<ACT_SIMPLE, true, W>(image_base + e, kcol, v, columns, RESIDUAL_AHEAD ? &residual[slot] : nullptr);
 		});
+		STAMP(3);
+	}
+
+	template<typename TE> bool columns_aligned(const FloatEpilogue<TE>&)
+	{
+		return true;
+	}
+	template<int MODE> bool columns_aligned(const Int8Epilogue<MODE> &epi)
+	{
+		return aligned_to(epi.scale, 16);
 	}
 
 	/* Picks the output tile: as few tiles per image as possible such that the tile's rows in halo order fit the 256 GEMM rows,
@@ -539,6 +585,9 @@ namespace avhip
 		/* the kernel stores whole runs of Epi::wide filters with one 16-byte instruction */
 		if (!epi.vec || s.K % Epi::wide != 0 || !aligned_to(epi.y, 16) || (epi.z != nullptr && !aligned_to(epi.z, 16)))
 			return false;
+		/* per-filter constants are requested as 16-byte runs */
+		if (!aligned_to(epi.bias, 16) || !columns_aligned(epi))
+			return false;
 		TileGeom g;
 		if (!choose_tile(s, g))
 			return false;
@@ -565,6 +614,9 @@ namespace avhip
 		if (fill < 0.5)
 			return false;
 		if (static_cast<int64_t>(s.Ho) * s.Wo * s.K >= (1ll << 31))
+			return false;
+		/* 24-bit multiplications in the halo addressing */
+		if (static_cast<int64_t>(s.W) * s.C * static_cast<int64_t>(sizeof(TE)) >= (1 << 24))
 			return false;
 		const int64_t blocks = static_cast<int64_t>(s.N) * g.tiles_h * g.tiles_w;
 		const int64_t filter_blocks = (static_cast<int64_t>(s.K) + TILE_N - 1) / TILE_N;

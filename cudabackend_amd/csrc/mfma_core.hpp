@@ -50,6 +50,12 @@ namespace avhip
 		{
 			c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.bf, b.bf, c, 0, 0, 0);
 		}
+		/* the first product of an accumulator: C is the constant zero, so no register has to be cleared beforehand */
+		__device__ static inline void start(const Chunk &a, const Chunk &b, acc_t &c)
+		{
+			const acc_t zero = {};
+			c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.bf, b.bf, zero, 0, 0, 0);
+		}
 	};
 	template<> struct Mma<f16_t>
 	{
@@ -58,6 +64,11 @@ namespace avhip
 		__device__ static inline void run(const Chunk &a, const Chunk &b, acc_t &c)
 		{
 			c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.hf, b.hf, c, 0, 0, 0);
+		}
+		__device__ static inline void start(const Chunk &a, const Chunk &b, acc_t &c)
+		{
+			const acc_t zero = {};
+			c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.hf, b.hf, zero, 0, 0, 0);
 		}
 	};
 	template<> struct Mma<int8_t>
@@ -68,6 +79,11 @@ namespace avhip
 		{
 			c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a.i4, b.i4, c, 0, 0, 0);
 		}
+		__device__ static inline void start(const Chunk &a, const Chunk &b, acc_t &c)
+		{
+			const acc_t zero = {};
+			c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a.i4, b.i4, zero, 0, 0, 0);
+		}
 	};
 	template<> struct Mma<float>
 	{
@@ -77,6 +93,14 @@ namespace avhip
 		{
 #pragma unroll
 			for (int i = 0; i < 4; i++)
+				c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.f[i], b.f[i], c, 0, 0, 0);
+		}
+		__device__ static inline void start(const Chunk &a, const Chunk &b, acc_t &c)
+		{
+			const acc_t zero = {};
+			c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.f[0], b.f[0], zero, 0, 0, 0);
+#pragma unroll
+			for (int i = 1; i < 4; i++)
 				c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.f[i], b.f[i], c, 0, 0, 0);
 		}
 	};
