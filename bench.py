@@ -585,10 +585,12 @@ def main():
         detail["nonfused_winograd_f32_F4"] = nonfused_stages(hip, ctx, "f32", "f32", 4, it)
         detail["nonfused_winograd_bf16_F2_fp16mat"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it)
         detail["nonfused_winograd_f16_F2_fp16mat_fp16M"] = nonfused_stages(hip, ctx, "f16", "f16", 2, it, acc_dtype="f16")
+        detail["nonfused_winograd_bf16_F2_fp16mat_fp16M"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it, acc_dtype="f16")
         cfg3 = (64, 56, 256)
         detail["config3_nonfused_winograd"] = {
             "bf16_F2_fp16mat": nonfused_stages(hip, ctx, "bf16", "f16", 2, it, shape=cfg3),
             "f16_F2_fp16mat_fp16M": nonfused_stages(hip, ctx, "f16", "f16", 2, it, shape=cfg3, acc_dtype="f16"),
+            "bf16_F2_fp16mat_fp16M": nonfused_stages(hip, ctx, "bf16", "f16", 2, it, shape=cfg3, acc_dtype="f16"),
             "bf16_F4_fp32mat": nonfused_stages(hip, ctx, "bf16", "f32", 4, it, shape=cfg3),
             "f16_F4_fp32mat": nonfused_stages(hip, ctx, "f16", "f32", 4, it, shape=cfg3),
         }

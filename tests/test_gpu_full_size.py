@@ -81,7 +81,7 @@ def test_config3_large_spatial(oracle, dtype):
     assert oracle.rel_l2(fused, direct) < 2 * BAR[dtype]
 
 
-@pytest.mark.parametrize("dtype,m,mat,acc", [("bf16", 2, "f16", "f32"), ("f16", 2, "f16", "f32"), ("f16", 2, "f16", "f16"), ("bf16", 4, "f32", "f32"),
+@pytest.mark.parametrize("dtype,m,mat,acc", [("bf16", 2, "f16", "f32"), ("f16", 2, "f16", "f32"), ("f16", 2, "f16", "f16"), ("bf16", 2, "f16", "f16"), ("bf16", 4, "f32", "f32"),
                                                ("f16", 4, "f32", "f32")])
 def test_config3_nonfused_winograd(oracle, dtype, m, mat, acc):
     """N=64, 56x56, 256->256 as the four-call non-fused Winograd sequence (src/winograd_nonfused.cu:906,932, src/gemm.cpp:126-209 of

@@ -11,7 +11,7 @@ import helpers as h
 pytestmark = pytest.mark.gpu
 
 # rel-L2 bound of one transform whose result is rounded once to the storage type
-TOL = {"f64": 1e-12, "f32": 2e-6, "f16": 1e-3, "bf16": 8e-3}
+TOL = {"f64": 1e-12, "f32": 2e-6, "f16": 5e-4, "bf16": 3e-3}  # 16-bit: storing the result alone is 2.1e-4 / 1.7e-3 rel-L2
 CASES = [(2, 3), (4, 3), (2, 5)]
 
 
