@@ -28,11 +28,12 @@
  */
 #include "conv_tile.hpp"
 #include "mfma_core.hpp"
+#include "persistent_gemm.hpp"
 #include <type_traits>
 
 #ifdef CONV_TILE_STAMPS
 __device__ unsigned long long g_stamps[4096 * 8];
-#define STAMP(i) do { if (threadIdx.x == 0) g_stamps[((blockIdx.y * gridDim.x + blockIdx.x) % 4096) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#define STAMP(i) do { if (threadIdx.x == 0) g_stamps[(blockIdx.x % 4096) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
 extern "C" __attribute__((visibility("default"))) int avhip_debug_stamps(void *out)
 {
 	return static_cast<int>(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_stamps), sizeof(g_stamps)));
@@ -67,6 +68,9 @@ namespace
 		int tiles_h, tiles_w;
 		int slices; /* 128-byte channel slices */
 		int images;
+		int filter_blocks; /* blocks of TILE_N filters */
+		int filter_shift; /* log2(filter_blocks) when that is a power of two, else -1 */
+		int filter_fastest; /* numbering of the workgroups, see the kernel */
 	};
 
 	/* FS = 3: the filter is 3 x 3 and the k loop is written out tap by tap (see the second half of the kernel); FS = 0: any
@@ -96,7 +100,33 @@ namespace
 
 		/* Everything up to the first halo request is latency the matrix cores sit through: no division on that path when the
 		 * tile is the whole image, and divisions by the halo width as a multiplication (hw_magic). */
-		int b = static_cast<int>(xcd_block(blockIdx.x, gridDim.x)); /* tiles of an image share halo pixels: one XCD, one L2 */
+		/* One-dimensional grid over (tile, filter block), tiles XCD-contiguous (the tiles of an image share halo pixels: one L2).
+		 * Grids of several rounds number the filter block fastest: the workgroups that read the same halo are then dispatched next
+		 * to each other and the halo comes from memory once, from L2 afterwards (measured 3-6 % on 56 x 56 x 256 layers).  Grids
+		 * that are resident at once keep the tiles fastest: there both filter blocks of a tile land on one compute unit (measured
+		 * 5 % better on 20 x 20 x 128 in bf16 than the other order). */
+		unsigned int filter_block, tile_number;
+		if (g.filter_fastest)
+		{
+			const unsigned int work = xcd_block(blockIdx.x, gridDim.x);
+			if (g.filter_shift >= 0)
+			{
+				filter_block = work & ((1u << g.filter_shift) - 1u);
+				tile_number = work >> g.filter_shift;
+			}
+			else
+			{
+				tile_number = work / static_cast<unsigned int>(g.filter_blocks);
+				filter_block = work - tile_number * g.filter_blocks;
+			}
+		}
+		else
+		{
+			const unsigned int tiles = gridDim.x / static_cast<unsigned int>(g.filter_blocks);
+			filter_block = g.filter_blocks == 1 ? 0u : blockIdx.x / tiles;
+			tile_number = xcd_block(blockIdx.x - filter_block * tiles, tiles);
+		}
+		int b = static_cast<int>(tile_number);
 		int tw = 0, th = 0, n = b;
 		if (g.tiles_w * g.tiles_h != 1)
 		{
@@ -107,7 +137,7 @@ namespace
 		}
 		auto over_halo_width = [&](int v) { return static_cast<int>((static_cast<unsigned int>(v) * g.hw_magic) >> 20); }; /* v / HW for v * HW < 2^20 */
 		const int oh0 = th * g.TH, ow0 = tw * g.TW;
-		const int k0 = blockIdx.y * TILE_N;
+		const int k0 = static_cast<int>(filter_block) * TILE_N;
 		constexpr int W = Epi::wide; /* filters per work-item in the epilogue: one 16-byte store each */
 		const int kcol = k0 + drain_column<1, W>();
 		typename Epi::template ColumnsT<W> columns;
@@ -620,9 +650,15 @@ namespace avhip
 			return false;
 		const int64_t blocks = static_cast<int64_t>(s.N) * g.tiles_h * g.tiles_w;
 		const int64_t filter_blocks = (static_cast<int64_t>(s.K) + TILE_N - 1) / TILE_N;
-		if (blocks > 0x7FFFFFFFll || filter_blocks > 65535)
+		if (blocks * filter_blocks > 0x7FFFFFFFll)
 			return false;
-		const dim3 grid(static_cast<unsigned int>(blocks), static_cast<unsigned int>(filter_blocks));
+		g.filter_blocks = static_cast<int>(filter_blocks);
+		g.filter_shift = -1;
+		for (int sh = 0; sh < 31; sh++)
+			if ((1ll << sh) == filter_blocks)
+				g.filter_shift = sh;
+		g.filter_fastest = blocks * filter_blocks > static_cast<int64_t>(persistent_workgroups(1ll << 40)) ? 1 : 0;
+		const dim3 grid(static_cast<unsigned int>(blocks * filter_blocks));
 		if (s.R == 3 && s.S == 3)
 			hipLaunchKernelGGL((k_conv_tile<TE, Epi, 3>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
 		else
