@@ -185,6 +185,17 @@ namespace avhip
 		return b < per_xcd * XCDS ? (b % XCDS) * per_xcd + b / XCDS : b;
 	}
 
+	/* Tile of a workgroup in a grid of (row blocks, column blocks): the column block (filters) runs fastest and each XCD owns a
+	 * contiguous run, so the workgroups that read the same rows of the streamed operand run next to each other on one L2 and the
+	 * operand comes from HBM once.  A grid walked in its own order (all row blocks of column block 0 first) reads it once per
+	 * column block. */
+	__device__ inline void xcd_tile(unsigned int &row_block, unsigned int &column_block)
+	{
+		const unsigned int t = xcd_block(blockIdx.y * gridDim.x + blockIdx.x, gridDim.x * gridDim.y);
+		row_block = t / gridDim.y;
+		column_block = t - row_block * gridDim.y;
+	}
+
 	/* Forward activations, src/activations.cuh:202-425 of the reference. */
 	template<typename CT>
 	__device__ inline CT activation_forward(int act, CT x)

@@ -416,14 +416,17 @@ namespace
 	__global__ __launch_bounds__(256, 2) void k_conv_igemm(const TE *__restrict__ x, const TE *__restrict__ w, ConvGeom g, TE padv, int vec_ok, Epi epi)
 	{
 		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
-		/* neighbouring pixel blocks read overlapping input windows: one XCD (one L2) gets a contiguous run of them */
-		const int64_t p0 = static_cast<int64_t>(xcd_block(blockIdx.x, gridDim.x)) * BLOCK_M;
-		const int k = blockIdx.y * BLOCK_N + drain_column<2>();
+		/* neighbouring pixel blocks read overlapping input windows and the filter blocks of a pixel block read the same ones:
+		 * one XCD (one L2) gets a contiguous run of them */
+		unsigned int pixel_block, filter_block;
+		xcd_tile(pixel_block, filter_block);
+		const int64_t p0 = static_cast<int64_t>(pixel_block) * BLOCK_M;
+		const int k = filter_block * BLOCK_N + drain_column<2>();
 		typename Epi::Columns columns;
 		epi.load_columns(k, columns); /* issued before the k loop: its latency is hidden behind the whole convolution */
 
 		PixelLoader<TE, FAST> la(x, g, padv, (vec_ok & 1) != 0, p0);
-		FilterLoader<TE, FAST> lb(w, g, (vec_ok & 1) != 0, blockIdx.y * BLOCK_N);
+		FilterLoader<TE, FAST> lb(w, g, (vec_ok & 1) != 0, filter_block * BLOCK_N);
 		typename Mma<TE>::acc_t acc[2][2];
 		block_mma<TE>(lds, g.R * g.S * g.steps_per_tap, la, lb, acc);
 
@@ -439,14 +442,17 @@ namespace
 	__global__ __launch_bounds__(256, 2) void k_conv_igemm_packed(const TE *__restrict__ x, const TE *__restrict__ w, ConvGeom g, Epi epi)
 	{
 		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
-		/* neighbouring pixel blocks read overlapping input windows: one XCD (one L2) gets a contiguous run of them */
-		const int64_t p0 = static_cast<int64_t>(xcd_block(blockIdx.x, gridDim.x)) * BLOCK_M;
-		const int k = blockIdx.y * BLOCK_N + drain_column<2>();
+		/* neighbouring pixel blocks read overlapping input windows and the filter blocks of a pixel block read the same ones:
+		 * one XCD (one L2) gets a contiguous run of them */
+		unsigned int pixel_block, filter_block;
+		xcd_tile(pixel_block, filter_block);
+		const int64_t p0 = static_cast<int64_t>(pixel_block) * BLOCK_M;
+		const int k = filter_block * BLOCK_N + drain_column<2>();
 		typename Epi::Columns columns;
 		epi.load_columns(k, columns);
 
 		PackedPixelLoader<TE, PB> la(x, g, p0);
-		PackedFilterLoader<TE, PB> lb(w, g, blockIdx.y * BLOCK_N);
+		PackedFilterLoader<TE, PB> lb(w, g, filter_block * BLOCK_N);
 		typename Mma<TE>::acc_t acc[2][2];
 		block_mma<TE>(lds, (g.R * g.S * g.C * static_cast<int>(sizeof(TE)) + STEP_BYTES - 1) / STEP_BYTES, la, lb, acc);
 

@@ -125,8 +125,10 @@ namespace
 		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
 		constexpr int KE = STEP_BYTES / sizeof(TE);
 		const int batch = blockIdx.z;
-		const int m0 = blockIdx.x * BLOCK_M;
-		const int n0 = blockIdx.y * BLOCK_N;
+		unsigned int row_block, column_block;
+		xcd_tile(row_block, column_block); /* the column blocks of a row block share A through one L2 */
+		const int m0 = row_block * BLOCK_M;
+		const int n0 = column_block * BLOCK_N;
 
 		RowLoader<TE, FAST> la(A + batch * strideA, M, K, lda, m0, (vec_ok & 1) != 0);
 		RowLoader<TE, FAST> lb(B + batch * strideB, N, K, ldb, n0, (vec_ok & 1) != 0);
