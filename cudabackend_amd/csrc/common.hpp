@@ -149,6 +149,19 @@ namespace avhip
 		}
 	}
 
+	/* A whole 8- or 16-byte run stored "sc0 sc1 nt": streamed and written through to memory as the kernel runs.  Lines a kernel
+	 * leaves dirty in L2 are written back when it ends, between it and the next dependent kernel; runs that cover only part
+	 * of a cache line (8 int8 results per work-item) otherwise stay behind until then. */
+	template<typename V>
+	__device__ __forceinline__ void store_through(V *dst, const V &value)
+	{
+		static_assert(sizeof(V) == 8 || sizeof(V) == 16, "one dwordx2 or dwordx4 store");
+		if constexpr (sizeof(V) == 8)
+			asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1 nt" : : "v"(dst), "v"(value) : "memory");
+		else
+			asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" : : "v"(dst), "v"(value) : "memory");
+	}
+
 	/* Makes a wavefront-uniform 32-bit value live in a scalar register from here on.  Kernel arguments sit in memory and the
 	 * compiler is free to re-load them wherever they are used; in fully unrolled epilogues that puts a scalar load and a
 	 * wait in front of every store.  Passing the value through an empty asm statement makes it opaque, so it is loaded once.

@@ -298,6 +298,7 @@ namespace avhip
 		float alpha1, alpha2, beta;
 		int activation, K;
 		bool vec;
+		bool through; /* int8 results are written through (store_at); set by kernels whose workgroups store parts of cache lines */
 
 		__device__ __forceinline__ void pin()
 		{
@@ -457,7 +458,11 @@ namespace avhip
 				int t[W];
 				integer_values<W>(t, v, c);
 				/* whole runs leave as streaming vector stores: the kernel never reads y back, so the caches may drain it while
-				 * the kernel runs */
+				 * the kernel runs.  int32 results (16 bytes per work-item, whole cache lines per row) are fastest as plain
+				 * non-temporal stores; so are int8 results of a workgroup that writes whole lines (the 1x1 kernels: 7.5 us
+				 * against 9.8 us written through).  Where a workgroup's row of int8 results is part of a cache line (64 filters
+				 * of the tile kernel) they are written through as well, or the partial lines wait in L2 for the write-back at the
+				 * end of the kernel (config 4, requantised 3x3 layer: 17.0 -> 14.8 us; int32 results there: 14.6 -> 16.6 us) */
 				typedef typename Words<W / 4>::type words_t; /* W int8 values as 32-bit words */
 				if (MODE == I8_EXACT)
 				{
@@ -491,7 +496,17 @@ namespace avhip
 					requantise<W>(o.u, t, c);
 					int8_t *dst = static_cast<int8_t*>(y) + idx;
 					if (vec && valid >= W)
-						__builtin_nontemporal_store(o.w, reinterpret_cast<words_t*>(dst));
+					{
+						if constexpr (sizeof(words_t) >= 8)
+						{
+							if (through)
+								store_through(reinterpret_cast<words_t*>(dst), o.w);
+							else
+								__builtin_nontemporal_store(o.w, reinterpret_cast<words_t*>(dst));
+						}
+						else
+							__builtin_nontemporal_store(o.w, reinterpret_cast<words_t*>(dst));
+					}
 					else
 					{
 #pragma unroll

@@ -571,6 +571,17 @@ namespace
 	{
 		return true;
 	}
+	/* a workgroup of this kernel stores TILE_N = 64 filters of a pixel: int8 results are half a cache line */
+	template<typename TE> FloatEpilogue<TE> for_partial_lines(const FloatEpilogue<TE> &epi)
+	{
+		return epi;
+	}
+	template<int MODE> Int8Epilogue<MODE> for_partial_lines(const Int8Epilogue<MODE> &epi)
+	{
+		Int8Epilogue<MODE> e = epi;
+		e.through = true;
+		return e;
+	}
 	template<int MODE> bool columns_aligned(const Int8Epilogue<MODE> &epi)
 	{
 		return aligned_to(epi.scale, 16);
@@ -608,8 +619,9 @@ namespace
 namespace avhip
 {
 	template<typename TE, typename Epi>
-	bool conv_tile_launch(hipStream_t stream, const avhipConvShape &s, const void *x, const void *w, const Epi &epi)
+	bool conv_tile_launch(hipStream_t stream, const avhipConvShape &s, const void *x, const void *w, const Epi &caller_epi)
 	{
+		const Epi epi = for_partial_lines(caller_epi);
 		if (s.stride_h != 1 || s.stride_w != 1 || s.dil_h != 1 || s.dil_w != 1)
 			return false;
 		/* the kernel stores whole runs of Epi::wide filters with one 16-byte instruction */
