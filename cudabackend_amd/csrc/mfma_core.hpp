@@ -136,9 +136,16 @@ namespace avhip
 	 */
 	typedef __attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int u32x4_t;
 	constexpr unsigned int OUT_OF_RANGE = 0x80000000u;
+	/* Every descriptor made here is the same for all work-items of a wavefront (a tensor, an image, a tile of a workgroup).
+	 * Saying so (readfirstlane) keeps it in scalar registers even where its address or extent came out of 64-bit arithmetic
+	 * that the compiler does on the vector unit; a descriptor it believes to vary per work-item costs a loop around every
+	 * load and store that uses it, and the loop's block boundaries keep those accesses from being scheduled among the MFMAs. */
 	__device__ inline __amdgpu_buffer_rsrc_t make_buffer(const void *base, unsigned int bytes)
 	{
-		return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+		const uint64_t address = reinterpret_cast<uint64_t>(base);
+		const uint64_t lo = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(address & 0xFFFFFFFFu)));
+		const uint64_t hi = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(address >> 32)));
+		return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(hi << 32 | lo), 0, __builtin_amdgcn_readfirstlane(static_cast<int>(bytes)), 0x00020000);
 	}
 	template<int POLICY = 0>
 	__device__ inline uint4 buffer_fetch(__amdgpu_buffer_rsrc_t rsrc, unsigned int byte_offset)
