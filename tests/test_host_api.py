@@ -148,3 +148,42 @@ def test_headers_compile_as_c_and_cxx_and_link(tmp_path):
         assert r.returncode == 0, r.stdout + r.stderr
         r = subprocess.run([str(exe)], capture_output=True, text=True, env=env)
         assert r.returncode == 0, "exit %d: %s%s" % (r.returncode, r.stdout, r.stderr)
+
+
+def test_descriptor_tables_survive_concurrent_callers():
+    """Eight host threads create, set, read back and destroy descriptors at once (ctypes releases the interpreter lock
+    during a call): every handle is unique while it lives, every read-back returns what its own thread wrote, and a
+    destroyed handle is refused.  Host logic only; no device is touched."""
+    import threading
+    lib = cb.load_library()
+    live, lock, errors = set(), threading.Lock(), []
+
+    def worker(seed):
+        try:
+            for i in range(400):
+                t, c = C.c_int64(0), C.c_int64(0)
+                cb.check(lib.cudaCreateTensorDescriptor(C.byref(t)))
+                cb.check(lib.cudaCreateConvolutionDescriptor(C.byref(c)))
+                with lock:
+                    assert t.value not in live and c.value not in live and t.value != c.value
+                    live.update((t.value, c.value))
+                dims = (C.c_int * 4)(seed + 1, i + 1, 7, 9)
+                cb.check(lib.cudaSetTensorDescriptor(t.value, cb.DTYPE_FLOAT16, 4, dims))
+                pad = (C.c_int * 2)(-seed, -i)
+                cb.check(lib.cudaSetConvolutionDescriptor(c.value, cb.CONVOLUTION_MODE, 2, pad, None, None, 1, None))
+                dtype, nb, out = C.c_int(0), C.c_int(0), (C.c_int * 8)()
+                cb.check(lib.cudaGetTensorDescriptor(t.value, C.byref(dtype), C.byref(nb), out))
+                assert dtype.value == cb.DTYPE_FLOAT16 and nb.value == 4 and list(out)[:4] == [seed + 1, i + 1, 7, 9]
+                with lock:
+                    live.difference_update((t.value, c.value))
+                cb.check(lib.cudaDestroyTensorDescriptor(t.value))
+                cb.check(lib.cudaDestroyConvolutionDescriptor(c.value))
+        except Exception as e:  # noqa: BLE001 - collected and re-raised in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(s,)) for s in range(8)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors[0]
