@@ -480,6 +480,22 @@ namespace
 		/* LINEAR / RELU get their own instance: a nine-way switch per element makes the compiler evaluate every function */
 		const bool simple = is_simple_activation(activation);
 		const bool narrow = items < (1ull << 31) && static_cast<uint64_t>(H) * W < (1ull << 31);
+		/* 16-bit matrices and tensors, t = 4, a problem of at most one round of resident workgroups (8 of 256 work-items on each
+		 * of 256 compute units): 8 channels per work-item, i.e. 16-byte loads and stores.  A kernel this short is paced by how
+		 * fast its accesses go out, not by how many wavefronts overlap (config 2, fp16 M: 22 -> 17.5 us); over several rounds
+		 * the narrower work-items win by a few per cent, and the input transform is slower with 8 at every size. */
+		constexpr int WIDE = VecOf<M, R, T, TM>::wide;
+		if constexpr (WIDE == 8 && VecOf<M, R, T, TM>::value == 4 && M + R - 1 == 4)
+		{
+			if (V > 1 && simple && narrow && K % WIDE == 0 && items <= 256u * 8u * 256u && aligned_to(Mx, 16) && aligned_to(y, 16) && (z == nullptr || aligned_to(z, 16)))
+			{
+				const dim3 wide_grid(ceil_div(items / 2, 256));
+				hipLaunchKernelGGL((k_output_transform<M, R, T, TM, WIDE, ACT_SIMPLE, uint32_t>), wide_grid, dim3(256), 0, s, static_cast<const TM*>(Mx), static_cast<T*>(y),
+						static_cast<const CT*>(bias), static_cast<const T*>(z), N, H, W, K, Th, Tw, static_cast<CT>(alpha1), static_cast<CT>(alpha2), static_cast<CT>(beta),
+						activation);
+				return 0;
+			}
+		}
 		if (V > 1 && simple && narrow)
 			AVHIP_LAUNCH_OUTPUT((VecOf<M, R, T, TM>::value), ACT_SIMPLE, uint32_t);
 		else if (V > 1 && narrow)

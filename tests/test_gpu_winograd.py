@@ -79,6 +79,25 @@ def test_output_transform_vector_path_and_activations(oracle):
         assert oracle.rel_l2(got, want) < 5e-6, act
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("use_bias,use_z,beta", [(True, True, 0.0), (True, False, 0.0), (False, True, 0.0), (True, True, 0.1)])
+@pytest.mark.parametrize("shape", [(5, 15, 15, 64), (2, 13, 14, 72), (3, 9, 16, 8)])
+def test_output_transform_sixteen_bit_matrices_wide_work_items(oracle, dtype, use_bias, use_z, beta, shape):
+    """F(2x2, 3x3) with fp16 matrices and a filter count that divides by 8: small problems run with 8 filters per work-item
+    (16-byte accesses); odd heights and widths exercise the clipped tiles.  Same bar as the narrow instance."""
+    g = h.rng(41)
+    N, H, W, K = shape
+    tiles = N * ((H + 1) // 2) * ((W + 1) // 2)
+    M = h.rounded(oracle, g.standard_normal((16, tiles, K)), "f16")
+    bias = g.uniform(-0.1, 0.1, K).astype(np.float32).astype(np.float64) if use_bias else None
+    z = h.rounded(oracle, g.standard_normal(shape), dtype) if use_z else None
+    y0 = h.rounded(oracle, g.standard_normal(shape), dtype)
+    a1, a2, be = float(np.float32(1.1)), float(np.float32(1.2)), float(np.float32(beta))
+    got = h.winograd_output_transform(M, shape, (K, 3, 3, 8), dtype, 2, bias, z, y0, a1, a2, be, activation=3, mat_dtype="f16")
+    want = oracle.winograd_output_transform(M, shape, 2, 3, bias, z, y0, a1, a2, be, oracle.RELU)
+    assert oracle.rel_l2(got, want) < TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32", "f64"])
 @pytest.mark.parametrize("m,r", CASES)
 @pytest.mark.parametrize("shape", [(12, 13, 14, 21), (3, 15, 15, 64)])
