@@ -1494,9 +1494,15 @@ namespace avocado
 			s.dil_h = conv->dilation[0];
 			s.dil_w = conv->dilation[1];
 			s.mode = (conv->mode == AVOCADO_CROSS_CORRELATION_MODE) ? 1 : 0;
-			/* output extent of a stride-1 convolution whose offset padding is mirrored at the far edge */
-			s.Ho = s.H - 2 * s.pad_h - (s.R - 1);
-			s.Wo = s.W - 2 * s.pad_w - (s.S - 1);
+			/* output extent of a convolution whose offset padding is mirrored at the far edge; strides and dilations are
+			 * honoured (the reference's kernel, src/im2row.cu:29-66, is stride 1 only) */
+			if (s.stride_h < 1 || s.stride_w < 1 || s.dil_h < 1 || s.dil_w < 1)
+				return AVOCADO_STATUS_BAD_PARAM;
+			const int span_h = s.H - 2 * s.pad_h - (s.dil_h * (s.R - 1) + 1), span_w = s.W - 2 * s.pad_w - (s.dil_w * (s.S - 1) + 1);
+			if (span_h < 0 || span_w < 0)
+				return AVOCADO_STATUS_BAD_PARAM;
+			s.Ho = span_h / s.stride_h + 1;
+			s.Wo = span_w / s.stride_w + 1;
 			if (s.C != f->dim[3] || s.Ho <= 0 || s.Wo <= 0)
 				return AVOCADO_STATUS_BAD_PARAM;
 			if (row->dim[0] != static_cast<av_int64>(s.N) * s.Ho * s.Wo || row->dim[1] != s.R * s.S * s.C || row->dtype != src->dtype)

@@ -175,7 +175,8 @@ namespace
 		}
 	}
 
-	/* rows[pixel, (i*S + j)*C + c] = x[n, pad_h + oh + i', pad_w + ow + j', c]; one work-item per element of `rows`. */
+	/* rows[pixel, (i*S + j)*C + c] = x[n, pad_h + oh*stride_h + i'*dil_h, pad_w + ow*stride_w + j'*dil_w, c]; one work-item per
+	 * element of `rows`. */
 	template<typename E>
 	__global__ __launch_bounds__(256) void k_im2row(const E *__restrict__ x, E *__restrict__ rows, avhipConvShape s, E padv, int64_t total)
 	{
@@ -195,8 +196,8 @@ namespace
 		const int64_t n = t / s.Ho;
 		const int ii = s.mode ? (s.R - 1 - i) : i;
 		const int jj = s.mode ? (s.S - 1 - j) : j;
-		const int ih = s.pad_h + oh + ii;
-		const int iw = s.pad_w + ow + jj;
+		const int ih = s.pad_h + oh * s.stride_h + ii * s.dil_h;
+		const int iw = s.pad_w + ow * s.stride_w + jj * s.dil_w;
 		E v = padv;
 		if (ih >= 0 && ih < s.H && iw >= 0 && iw < s.W)
 			v = x[((n * s.H + ih) * s.W + iw) * s.C + c];
@@ -371,8 +372,8 @@ extern "C"
 	{
 		if (shape == nullptr || x == nullptr || rows == nullptr)
 			return AVHIP_BAD_PARAM;
-		if (shape->stride_h != 1 || shape->stride_w != 1 || shape->dil_h != 1 || shape->dil_w != 1)
-			return AVHIP_NOT_SUPPORTED;
+		if (shape->stride_h < 1 || shape->stride_w < 1 || shape->dil_h < 1 || shape->dil_w < 1)
+			return AVHIP_BAD_PARAM;
 		hipStream_t s = static_cast<hipStream_t>(stream);
 		switch (elem_size)
 		{

@@ -137,7 +137,8 @@ namespace avocado
 
 			/* ---- convolution ------------------------------------------------------------------------------------- */
 
-			/* cuda_backend.h:791.  rows[N*Ho*Wo, R*S*C] from x[N, H, W, C], stride 1, dilation 1. */
+			/* cuda_backend.h:791.  rows[N*Ho*Wo, R*S*C] from x[N, H, W, C]; the descriptor's strides and dilations are honoured
+			 * (Ho = (H - 2*padding - dilation*(R-1) - 1) / stride + 1; the reference's kernel assumes stride 1, dilation 1). */
 			DLL_PUBLIC avStatus_t cudaIm2Row(avContextDescriptor_t context, const avConvolutionDescriptor_t config, const avTensorDescriptor_t filterDesc,
 					const avTensorDescriptor_t srcDesc, const avMemoryDescriptor_t srcMem, const avTensorDescriptor_t rowDesc, avMemoryDescriptor_t rowMem);
 

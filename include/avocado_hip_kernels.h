@@ -98,7 +98,8 @@ extern "C"
 	AVHIP_API int avhip_add_bias(void *stream, int dtype, const void *x, const void *b, const void *z, void *y, int64_t first, int last, double alpha1,
 			double alpha2, double beta1, double beta2, double beta3, int activation);
 
-	/* Explicit im2row, stride 1.  Replaces kernel_im2row_conv2d, src/im2row.cu:29-66.  elem_size in bytes. */
+	/* Explicit im2row; strides and dilations of `shape` are honoured (the reference's kernel is stride 1 only).  Replaces
+	 * kernel_im2row_conv2d, src/im2row.cu:29-66.  elem_size in bytes. */
 	AVHIP_API int avhip_im2row(void *stream, int elem_size, const avhipConvShape *shape, const void *x, void *rows, const void *padding_value);
 
 	/* y = alpha * act(x * weight[j] + bias[j]) + beta * y over a [first, last] view of x (j = last index).  Replaces

@@ -30,7 +30,9 @@
  *                             (The reference delegates to cuBLAS, whose source is not part of it.)
  *   orc_add_bias              pinned: numpy restatement of the documented formula in two algebraic
  *                             forms; operation order from the reference kernel.
- *   orc_im2row                pinned: rows times flattened weights == orc_conv2d_f64.
+ *   orc_im2row                pinned: rows times flattened weights == orc_conv2d_f64, strides and dilations included
+ *                             (the reference's kernel is stride 1 only; its strided test cases are commented out,
+ *                             test/test_im2row.cpp:31-48).
  *   orc_affine_forward        pinned: with weight 1 it is orc_add_bias (itself pinned); numpy broadcast form.
  *   orc_batchnorm_inference   pinned: torch.nn.functional.batch_norm(training=False) in fp64; equals
  *                             orc_affine_forward on the folded parameters.
@@ -654,8 +656,8 @@ void orc_batchnorm_inference(const double *x, const double *scale, const double 
  * flipped tap in cross-correlation mode, so that rows x flattened-weights^T reproduces the convolution
  * (slot order of src/im2row.cu:47-62 expressed per output pixel).
  */
-void orc_im2row(const double *x, double *rows, int N, int H, int W, int C, int R, int S, int Ho, int Wo, int pad_h, int pad_w, int mode,
-		double padding_value)
+void orc_im2row(const double *x, double *rows, int N, int H, int W, int C, int R, int S, int Ho, int Wo, int pad_h, int pad_w, int stride_h,
+		int stride_w, int dil_h, int dil_w, int mode, double padding_value)
 {
 	for (int n = 0; n < N; n++)
 		for (int oh = 0; oh < Ho; oh++)
@@ -665,7 +667,7 @@ void orc_im2row(const double *x, double *rows, int N, int H, int W, int C, int R
 					{
 						const int ii = (mode == 0) ? i : (R - 1 - i);
 						const int jj = (mode == 0) ? j : (S - 1 - j);
-						const int ih = pad_h + oh + ii, iw = pad_w + ow + jj;
+						const int ih = pad_h + oh * stride_h + ii * dil_h, iw = pad_w + ow * stride_w + jj * dil_w;
 						double *dst = rows + ((((size_t) n * Ho + oh) * Wo + ow) * R * S + (size_t) i * S + j) * C;
 						for (int c = 0; c < C; c++)
 							dst[c] = (ih >= 0 && ih < H && iw >= 0 && iw < W) ? x[(((size_t) n * H + ih) * W + iw) * C + c] : padding_value;

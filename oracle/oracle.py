@@ -261,12 +261,13 @@ def batchnorm_inference(x, scale, bias, mean, variance, y=None, alpha=1.0, beta=
     return out
 
 
-def im2row(x, R, S, pad, mode=CONVOLUTION, padding_value=0.0):
+def im2row(x, R, S, pad, mode=CONVOLUTION, padding_value=0.0, stride=(1, 1), dilation=(1, 1)):
     x = _f64(x)
     N, H, W, Cin = x.shape
-    Ho, Wo = conv_output_shape(H, W, R, S, pad)
+    Ho, Wo = conv_output_shape(H, W, R, S, pad, stride, dilation)
     rows = np.zeros((N * Ho * Wo, R * S * Cin), dtype=np.float64)
-    lib().orc_im2row(_p(x), _p(rows), N, H, W, Cin, R, S, Ho, Wo, pad[0], pad[1], mode, C.c_double(padding_value))
+    lib().orc_im2row(_p(x), _p(rows), N, H, W, Cin, R, S, Ho, Wo, pad[0], pad[1], stride[0], stride[1], dilation[0], dilation[1], mode,
+                     C.c_double(padding_value))
     return rows
 
 

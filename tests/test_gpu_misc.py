@@ -54,6 +54,47 @@ def test_im2row(oracle, R, pad, dtype, mode):
     np.testing.assert_array_equal(np.asarray(got, dtype=np.float64), want)
 
 
+@pytest.mark.parametrize("R,pad,stride,dilation", [(3, (-1, -1), (2, 2), (1, 1)), (3, (-2, -2), (1, 1), (2, 2)), (3, (-1, 0), (2, 1), (1, 2)), (5, (-2, -1), (3, 2), (1, 1))])
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "i8"])
+def test_im2row_strides_and_dilations(oracle, R, pad, stride, dilation, dtype):
+    """Strides, dilations and asymmetric offsets (the cases test/test_im2row.cpp:31-48 leaves commented out), bit-exact against
+    the oracle; then rows x flattened filters through cudaGemm against the implicit-GEMM convolution of the same geometry."""
+    g = h.rng(33)
+    shape = (3, 23, 34, 16)
+    K = 24
+    if dtype == "i8":
+        x = g.integers(-127, 128, shape, dtype=np.int8)
+        w = g.integers(-127, 128, (K, R, R, shape[3]), dtype=np.int8)
+    else:
+        x = h.rounded(oracle, g.standard_normal(shape), dtype)
+        w = h.rounded(oracle, g.standard_normal((K, R, R, shape[3])) * 0.2, dtype)
+    Ho, Wo = oracle.conv_output_shape(shape[1], shape[2], R, R, pad, stride, dilation)
+    out_dtype = "i32" if dtype == "i8" else dtype
+    with h.Call() as c:
+        conv = cb.ConvolutionDescriptor(padding=pad, strides=stride, dilation=dilation, dtype=h.DT[dtype])
+        xt, wt = c.tensor(x, dtype), c.tensor(w, dtype)
+        rows = c.empty((3 * Ho * Wo, R * R * shape[3]), dtype)
+        cb.check(c.lib.cudaIm2Row(c.ctx.handle, conv.handle, wt.desc, xt.desc, xt.mem, rows.desc, rows.mem), "cudaIm2Row")
+        wflat = c.tensor(np.asarray(w).reshape(K, -1), dtype)
+        prod = c.empty((3 * Ho * Wo, K), out_dtype)
+        cb.check(c.lib.cudaGemm(c.ctx.handle, cb.GEMM_OPERATION_N, cb.GEMM_OPERATION_T, None, rows.desc, rows.mem, wflat.desc, wflat.mem, None, prod.desc, prod.mem),
+                 "cudaGemm")
+        y = c.empty((3, Ho, Wo, K), out_dtype)
+        cb.check(c.lib.cudaConvolutionImplicitGemmForward(c.ctx.handle, conv.handle, None, xt.desc, xt.mem, wt.desc, wt.mem, 0, 0, None, 0, 0, None,
+                                                          y.desc, y.mem, cb.ACTIVATION_LINEAR), "implicit GEMM")
+        c.finish()
+        got, explicit, implicit = rows.download(), prod.download(), y.download()
+    want = oracle.im2row(np.asarray(x, dtype=np.float64), R, R, pad, 0, 0.0, stride, dilation)
+    np.testing.assert_array_equal(np.asarray(got, dtype=np.float64), want)
+    explicit = np.asarray(explicit, dtype=np.float64).reshape(3, Ho, Wo, K)
+    implicit = np.asarray(implicit, dtype=np.float64)
+    if dtype == "i8":
+        np.testing.assert_array_equal(explicit, implicit)
+        np.testing.assert_array_equal(implicit, oracle.conv2d_i8(x, w, pad=pad, stride=stride, dilation=dilation))
+    else:
+        assert oracle.rel_l2(explicit, implicit) < (1e-5 if dtype == "f32" else 4e-3)
+
+
 def test_change_type(oracle):
     g = h.rng(32)
     v = np.concatenate([g.standard_normal(1000) * 50, [0.5, 1.5, 2.5, -0.5, -1.5, 127.5, 300.0, -300.0, 1e10, -1e10]]).astype(np.float32)

@@ -452,6 +452,20 @@ def test_im2row_times_weights_is_conv(oracle, R, pad, mode):
     np.testing.assert_allclose(got, oracle.conv2d(x, w, pad=pad, mode=mode), atol=1e-12)
 
 
+@pytest.mark.parametrize("R,pad,stride,dilation,mode", [(3, (-1, -1), (2, 2), (1, 1), 0), (3, (-2, -2), (1, 1), (2, 2), 0), (3, (-1, 0), (2, 1), (1, 2), 1),
+                                                         (5, (-2, -1), (3, 2), (1, 1), 0), (2, (0, -1), (2, 3), (2, 1), 1)])
+def test_im2row_with_strides_and_dilations_times_weights_is_conv(oracle, R, pad, stride, dilation, mode):
+    """The strided and asymmetric cases the reference's test leaves commented out (test/test_im2row.cpp:31-48): the rows
+    against the already pinned direct convolution with the same geometry."""
+    x = RNG.standard_normal((2, 11, 10, 3))
+    w = RNG.standard_normal((4, R, R, 3))
+    Ho, Wo = oracle.conv_output_shape(11, 10, R, R, pad, stride, dilation)
+    rows = oracle.im2row(x, R, R, pad, mode, 0.0, stride, dilation)
+    assert rows.shape == (2 * Ho * Wo, R * R * 3)
+    got = (rows @ w.reshape(4, -1).T).reshape(2, Ho, Wo, 4)
+    np.testing.assert_allclose(got, oracle.conv2d(x, w, pad=pad, stride=stride, dilation=dilation, mode=mode), atol=1e-12)
+
+
 def test_bf16_rounding_helpers(oracle):
     v = np.array([1.0, 1.00390625, 1.01171875, -3.0e38, 1e-40, np.inf], dtype=np.float32)
     bits = oracle.f32_to_bf16_bits(v)
