@@ -500,7 +500,7 @@ namespace
 
 	/* The branch-free loaders need aligned, complete chunks (bit 0 of flags), a zero padding value and 32-bit byte offsets. */
 	template<typename TE>
-	bool fast_path_ok(const avhipConvShape &s, int flags, const void *padding_value)
+	bool fast_path_ok(const avhipConvShape &s, int flags, const void *padding_value, bool tap_mask = true)
 	{
 		bool zero_padding = true;
 		if (padding_value != nullptr)
@@ -509,7 +509,8 @@ namespace
 		const int64_t x_bytes = static_cast<int64_t>(s.N) * s.H * s.W * s.C * sizeof(TE);
 		const int64_t w_bytes = static_cast<int64_t>(s.K) * s.R * s.S * s.C * sizeof(TE);
 		const int64_t pixels = static_cast<int64_t>(s.N) * s.Ho * s.Wo;
-		return (flags & 1) != 0 && zero_padding && x_bytes < (1ll << 31) && w_bytes < (1ll << 31) && pixels < (1ll << 31) - BLOCK_M && s.R * s.S <= 32;
+		return (flags & 1) != 0 && zero_padding && x_bytes < (1ll << 31) && w_bytes < (1ll << 31) && pixels < (1ll << 31) - BLOCK_M
+				&& (!tap_mask || s.R * s.S <= 32); /* the gather kernel keeps one bit per tap: which taps of a pixel lie inside the image */
 	}
 
 	template<typename TE, typename Epi>
@@ -562,7 +563,9 @@ namespace
 		if (fast && s.R * s.S == 1 && conv_pointwise_launch<TE, Epi>(st, s, x, w, epi))
 			return 0;
 		/* stride-1 filters with more than one tap first try the kernel that keeps an image tile resident in LDS */
-		if (fast && s.R * s.S > 1 && conv_tile_launch<TE, Epi>(st, s, x, w, epi))
+		/* (that kernel has no limit on the number of taps) */
+		const bool fast_tile = fast || (fast_path_ok<TE>(s, flags, padding_value, false) && is_simple_activation(epi.activation) && (flags & 2) != 0);
+		if (fast_tile && s.R * s.S > 1 && conv_tile_launch<TE, Epi>(st, s, x, w, epi))
 			return 0;
 		if (fast)
 			hipLaunchKernelGGL((k_conv_igemm<TE, true, Epi>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags, epi);

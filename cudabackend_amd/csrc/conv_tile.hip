@@ -49,15 +49,22 @@ namespace
 	constexpr int TILE_M = 256; /* output pixels per workgroup */
 	constexpr int TILE_N = 64; /* output filters per workgroup */
 	constexpr int PIXEL_PITCH = STEP_BYTES + 16; /* LDS bytes per halo pixel: 128 of channels + 16 of bank stagger */
-	constexpr int HALO_MAX = 300; /* halo pixels that fit */
-	constexpr int HALO_BYTES = HALO_MAX * PIXEL_PITCH;
 	constexpr int FILTER_TILE = TILE_N * LDS_ROW;
 	constexpr int FILTER_RING = 3; /* filter tiles in LDS: two for the general k loop, a ring of three for the unrolled 3x3 one */
-	constexpr int ROW_TABLE = HALO_BYTES + FILTER_RING * FILTER_TILE; /* offset of the table: GEMM row -> offset of its output pixel in the image, -1 if not stored */
-	constexpr int TILE_LDS = ROW_TABLE + TILE_M * 4;
-	constexpr int HALO_FETCHES = (HALO_MAX * STEP_CHUNKS + 255) / 256; /* 16-byte chunks of the halo per work-item */
 	constexpr int FILTER_FETCHES = TILE_N * STEP_CHUNKS / 256;
-	static_assert(4 * PrivateDrainRows<2, 4>::bytes <= ROW_TABLE, "the drain buffers of the four wavefronts reuse the operand buffers");
+	/* LDS of a workgroup, by the halo pixels it can hold: [halo | filter ring | row table].  300 pixels (the 17 x 17 halo of a
+	 * 15 x 15 image) leave room for two workgroups per compute unit; 448 (a 12 x 36 halo: 8 x 32 outputs under a 5 x 5 filter)
+	 * fill a compute unit with one. */
+	constexpr int HALO_SMALL = 300, HALO_BIG = 448;
+	template<int HMAX> struct TileLds
+	{
+		static constexpr int halo_bytes = HMAX * PIXEL_PITCH;
+		static constexpr int row_table = halo_bytes + FILTER_RING * FILTER_TILE; /* GEMM row -> offset of its output pixel in the image, -1 if not stored */
+		static constexpr int bytes = row_table + TILE_M * 4;
+		static constexpr int halo_fetches = (HMAX * STEP_CHUNKS + 255) / 256; /* 16-byte chunks of the halo per work-item */
+		static constexpr int pixels = (halo_bytes + 2 * FILTER_TILE) / PIXEL_PITCH; /* what a read at a halo-order row may reach */
+	};
+	static_assert(4 * PrivateDrainRows<2, 4>::bytes <= TileLds<HALO_SMALL>::row_table, "the drain buffers of the four wavefronts reuse the operand buffers");
 
 	struct TileGeom
 	{
@@ -65,6 +72,8 @@ namespace
 		int TH, TW; /* output tile */
 		int HH, HW; /* halo = (TH + R - 1) x (TW + S - 1) */
 		unsigned int hw_magic; /* 2^20 / HW + 1: (v * hw_magic) >> 20 == v / HW while v * HW < 2^20 */
+		int row_pitch; /* GEMM row r is output pixel (r / row_pitch, r % row_pitch) of the tile: HW (halo order) or TW (dense) */
+		unsigned int row_magic; /* 2^20 / row_pitch + 1 */
 		int tiles_h, tiles_w;
 		int slices; /* 128-byte channel slices */
 		int images;
@@ -75,9 +84,14 @@ namespace
 
 	/* FS = 3: the filter is 3 x 3 and the k loop is written out tap by tap (see the second half of the kernel); FS = 0: any
 	 * filter, general loop. */
-	template<typename TE, typename Epi, int FS>
-	__global__ __launch_bounds__(256, 2) void k_conv_tile(const TE *__restrict__ x, const TE *__restrict__ w, TileGeom g, Epi epi)
+	template<typename TE, typename Epi, int FS, int HMAX = HALO_SMALL>
+	__global__ __launch_bounds__(256, HMAX > HALO_SMALL ? 1 : 2) void k_conv_tile(const TE *__restrict__ x, const TE *__restrict__ w, TileGeom g, Epi epi)
 	{
+		constexpr int HALO_MAX = HMAX;
+		constexpr int HALO_BYTES = TileLds<HMAX>::halo_bytes;
+		constexpr int ROW_TABLE = TileLds<HMAX>::row_table;
+		constexpr int TILE_LDS = TileLds<HMAX>::bytes;
+		constexpr int HALO_FETCHES = TileLds<HMAX>::halo_fetches;
 		STAMP(0);
 		epi.pin();
 		keep_in_sgpr(g.TW);
@@ -135,7 +149,6 @@ namespace
 			th = b % g.tiles_h;
 			n = b / g.tiles_h;
 		}
-		auto over_halo_width = [&](int v) { return static_cast<int>((static_cast<unsigned int>(v) * g.hw_magic) >> 20); }; /* v / HW for v * HW < 2^20 */
 		const int oh0 = th * g.TH, ow0 = tw * g.TW;
 		const int k0 = static_cast<int>(filter_block) * TILE_N;
 		constexpr int W = Epi::wide; /* filters per work-item in the epilogue: one 16-byte store each */
@@ -232,6 +245,7 @@ namespace
 				const unsigned int offset = base + __umul24(hy, line_bytes) + __umul24(hx, pixel_bytes);
 				halo_src[f] = inside ? offset : OUT_OF_RANGE;
 				hr[f] = buffer_fetch(rx, first_slice_exists ? halo_src[f] : OUT_OF_RANGE); /* slice 0 goes out as soon as its address exists */
+				__builtin_amdgcn_sched_barrier(0); /* ... and the scheduler may not collect the requests behind all the address arithmetic */
 			}
 		}
 		STAMP(4);
@@ -239,7 +253,9 @@ namespace
 		int *row_table = reinterpret_cast<int*>(lds + ROW_TABLE);
 		{
 			/* GEMM row -> offset of its output pixel inside the image of y, in elements; -1 for rows that are not stored */
-			const int py = over_halo_width(tid), px = tid - py * g.HW;
+			/* (the written-out 3 x 3 instance is launched in halo order only and spends nothing on the other one) */
+			const unsigned int pitch = FS == 0 ? static_cast<unsigned int>(g.row_pitch) : static_cast<unsigned int>(g.HW), magic = FS == 0 ? g.row_magic : g.hw_magic;
+			const int py = static_cast<int>((static_cast<unsigned int>(tid) * magic) >> 20), px = tid - py * static_cast<int>(pitch);
 			const int oh = oh0 + py, ow = ow0 + px;
 			row_table[tid] = (py < g.TH && px < g.TW && oh < g.Ho && ow < g.Wo) ? (oh * g.Wo + ow) * g.K : -1; /* times K here, once, not in every use */
 		}
@@ -305,9 +321,22 @@ namespace
 			}
 		};
 
+		/* the halo pixel under tap (0, 0) of this work-item's GEMM rows.  In halo order (row pitch = halo width) that is the row
+		 * number itself and rows between the tile's lines are computed and dropped; in dense order (row pitch = tile width: every
+		 * row is a pixel, for tiles whose lines in halo order would not fit 256 rows) rows past the tile read pixel 0 */
 #pragma unroll
 		for (int tm = 0; tm < 2; tm++)
 			a_off[tm] = (wave * 64 + tm * 32 + (lane & 31)) * PIXEL_PITCH + (lane >> 5) * 16;
+		if (FS == 0 && g.row_pitch != g.HW) /* (uniform) */
+		{
+#pragma unroll
+			for (int tm = 0; tm < 2; tm++)
+			{
+				const int r = wave * 64 + tm * 32 + (lane & 31);
+				const int py = static_cast<int>((static_cast<unsigned int>(r) * g.row_magic) >> 20), px = r - py * g.row_pitch;
+				a_off[tm] = (py < g.TH ? py * g.HW + px : 0) * PIXEL_PITCH + (lane >> 5) * 16;
+			}
+		}
 		stash_halo(hr);
 		stash_filters(0, fr[0]);
 		STAMP(5);
@@ -587,32 +616,38 @@ namespace
 		return aligned_to(epi.scale, 16);
 	}
 
-	/* Picks the output tile: as few tiles per image as possible such that the tile's rows in halo order fit the 256 GEMM rows,
-	 * the halo fits its LDS area and the reads of the never-stored rows stay inside the kernel's LDS. */
-	bool choose_tile(const avhipConvShape &s, TileGeom &g)
+	/* Picks the output tile for a halo capacity: as few tiles per image as possible such that the tile's rows fit the 256 GEMM
+	 * rows and its halo fits LDS.  Rows in halo order (the tile's lines at the pitch of the halo: a tap is one constant shift of
+	 * consecutive LDS pixels, conflict-free reads; the reads of the never-stored rows must stay inside the kernel's LDS) are
+	 * preferred; dense order (every row a pixel) takes over where it needs fewer tiles, which is the case for wide tiles under
+	 * large filters. */
+	struct TileChoice
 	{
-		constexpr int LDS_PIXELS = (HALO_BYTES + 2 * FILTER_TILE) / PIXEL_PITCH;
-		int best_tiles = 0, best_halo = 0;
-		for (int tw = 1; tw <= s.Wo && tw <= TILE_M; tw++)
-			for (int th = 1; th <= s.Ho; th++)
-			{
-				const int hw = tw + s.S - 1;
-				const int rows = (th - 1) * hw + tw;
-				const int halo = (th + s.R - 1) * hw;
-				if (rows > TILE_M)
-					break;
-				if (halo > HALO_MAX || TILE_M + (s.R - 1) * hw + s.S > LDS_PIXELS)
-					continue;
-				const int tiles = ((s.Ho + th - 1) / th) * ((s.Wo + tw - 1) / tw);
-				if (best_tiles == 0 || tiles < best_tiles || (tiles == best_tiles && halo < best_halo))
+		int th, tw, dense, tiles;
+	};
+	TileChoice choose_tile(const avhipConvShape &s, int halo_max, int lds_pixels, bool allow_dense)
+	{
+		TileChoice best = { 0, 0, 0, 0 };
+		int best_halo = 0;
+		for (int dense = 0; dense < (allow_dense ? 2 : 1); dense++)
+			for (int tw = 1; tw <= s.Wo && tw <= TILE_M; tw++)
+				for (int th = 1; th <= s.Ho; th++)
 				{
-					best_tiles = tiles;
-					best_halo = halo;
-					g.TH = th;
-					g.TW = tw;
+					const int hw = tw + s.S - 1;
+					const int rows = dense ? th * tw : (th - 1) * hw + tw;
+					const int halo = (th + s.R - 1) * hw;
+					if (rows > TILE_M)
+						break;
+					if (halo > halo_max || (!dense && TILE_M + (s.R - 1) * hw + s.S > lds_pixels))
+						continue;
+					const int tiles = ((s.Ho + th - 1) / th) * ((s.Wo + tw - 1) / tw);
+					if (best.tiles == 0 || tiles < best.tiles || (tiles == best.tiles && dense == best.dense && halo < best_halo))
+					{
+						best = { th, tw, dense, tiles };
+						best_halo = halo;
+					}
 				}
-			}
-		return best_tiles > 0;
+		return best;
 	}
 }
 
@@ -630,9 +665,39 @@ namespace avhip
 		/* per-filter constants are requested as 16-byte runs */
 		if (!aligned_to(epi.bias, 16) || !columns_aligned(epi))
 			return false;
-		TileGeom g;
-		if (!choose_tile(s, g))
+		/* two LDS layouts: the usual one (two workgroups per compute unit) and, for filters other than 3 x 3, one with a halo
+		 * large enough for 256-pixel tiles under a 5 x 5 filter (one workgroup per compute unit).  Estimated cost: rounds of
+		 * resident workgroups times (k-steps at the measured pace of a workgroup that shares its compute unit, 0.68 us, or has
+		 * it to itself, 0.47 us, plus 3.6 us of prologue and epilogue). */
+		const int64_t filter_blocks = (static_cast<int64_t>(s.K) + TILE_N - 1) / TILE_N;
+		const int64_t resident = static_cast<int64_t>(persistent_workgroups(1ll << 40));
+		const int steps = s.R * s.S * ((s.C * static_cast<int>(sizeof(TE)) + STEP_BYTES - 1) / STEP_BYTES);
+		const bool general = s.R != 3 || s.S != 3; /* the instance with the general k loop: either row order, either LDS layout */
+		TileChoice pick = choose_tile(s, HALO_SMALL, TileLds<HALO_SMALL>::pixels, general);
+		bool big = false;
+		if (general)
+		{
+			const TileChoice wide = choose_tile(s, HALO_BIG, TileLds<HALO_BIG>::pixels, true);
+			if (wide.tiles > 0)
+			{
+				const int64_t wide_groups = static_cast<int64_t>(s.N) * wide.tiles * filter_blocks, groups = static_cast<int64_t>(s.N) * pick.tiles * filter_blocks;
+				const double wide_cost = static_cast<double>((wide_groups + resident / 2 - 1) / (resident / 2)) * (steps * 0.47 + 3.6);
+				const double cost = static_cast<double>((groups + resident - 1) / resident) * (steps * (groups > resident / 2 ? 0.68 : 0.47) + 3.6);
+				/* (tiles that would be mostly padding send the layer to the gather kernel, see below: then the other layout is
+				 * the only candidate) */
+				const bool mostly_padding = pick.tiles > 0 && static_cast<double>(s.Ho) * s.Wo < 0.5 * pick.tiles * TILE_M;
+				if (pick.tiles == 0 || mostly_padding || wide_cost < 0.9 * cost)
+				{
+					pick = wide;
+					big = true;
+				}
+			}
+		}
+		if (pick.tiles == 0)
 			return false;
+		TileGeom g;
+		g.TH = pick.th;
+		g.TW = pick.tw;
 		g.H = s.H;
 		g.W = s.W;
 		g.C = s.C;
@@ -646,7 +711,9 @@ namespace avhip
 		g.flip = s.mode != 0 ? 1 : 0;
 		g.HH = g.TH + s.R - 1;
 		g.HW = g.TW + s.S - 1;
-		g.hw_magic = (1u << 20) / static_cast<unsigned int>(g.HW) + 1u; /* HW <= 300 and the dividends are below 320 */
+		g.hw_magic = (1u << 20) / static_cast<unsigned int>(g.HW) + 1u; /* HW <= 448 and the dividends are below 512 */
+		g.row_pitch = pick.dense ? g.TW : g.HW;
+		g.row_magic = (1u << 20) / static_cast<unsigned int>(g.row_pitch) + 1u; /* dividends below 256 */
 		g.tiles_h = (s.Ho + g.TH - 1) / g.TH;
 		g.tiles_w = (s.Wo + g.TW - 1) / g.TW;
 		g.slices = (s.C * static_cast<int>(sizeof(TE)) + STEP_BYTES - 1) / STEP_BYTES;
@@ -661,7 +728,6 @@ namespace avhip
 		if (static_cast<int64_t>(s.W) * s.C * static_cast<int64_t>(sizeof(TE)) >= (1 << 24))
 			return false;
 		const int64_t blocks = static_cast<int64_t>(s.N) * g.tiles_h * g.tiles_w;
-		const int64_t filter_blocks = (static_cast<int64_t>(s.K) + TILE_N - 1) / TILE_N;
 		if (blocks * filter_blocks > 0x7FFFFFFFll)
 			return false;
 		g.filter_blocks = static_cast<int>(filter_blocks);
@@ -673,6 +739,8 @@ namespace avhip
 		const dim3 grid(static_cast<unsigned int>(blocks * filter_blocks));
 		if (s.R == 3 && s.S == 3)
 			hipLaunchKernelGGL((k_conv_tile<TE, Epi, 3>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
+		else if (big)
+			hipLaunchKernelGGL((k_conv_tile<TE, Epi, 0, HALO_BIG>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
 		else
 			hipLaunchKernelGGL((k_conv_tile<TE, Epi, 0>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
 		return true;

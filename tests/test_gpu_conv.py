@@ -161,6 +161,11 @@ TILE_CASES = [
     dict(x=(2, 16, 15, 32), w=(16, 3, 3, 32), pad=(-2, -2)),              # full convolution: output larger than input
     dict(x=(2, 15, 15, 64), w=(32, 5, 5, 64), pad=(-2, -2)),              # the general k loop (not 3x3)
     dict(x=(2, 15, 14, 72), w=(24, 3, 1, 72), pad=(-1, 0), mode=1),       # three taps only, flipped
+    dict(x=(3, 32, 32, 64), w=(64, 5, 5, 64), pad=(-2, -2)),              # 8 x 32 tiles in dense row order, large-halo LDS layout
+    dict(x=(2, 37, 41, 24), w=(40, 5, 5, 24), pad=(-2, -2), mode=1),      # the same with partial tiles at both edges, flipped
+    dict(x=(2, 30, 50, 16), w=(24, 7, 7, 16), pad=(-3, -3)),              # 7 x 7
+    dict(x=(2, 19, 70, 32), w=(16, 1, 7, 32), pad=(0, -3)),               # one line of seven taps over a wide image
+    dict(x=(2, 40, 24, 32), w=(16, 5, 3, 32), pad=(-2, -1)),              # dense order in the usual LDS layout
 ]
 
 

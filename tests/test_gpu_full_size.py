@@ -148,3 +148,33 @@ def test_config5_bf16(oracle, case):
     perm = g.permutation(case["x"][0])
     again = h.conv_forward("dispatch", x[perm], w, got.shape, "bf16", bias=b, activation=cb.ACTIVATION_RELU, pad=case["pad"], stride=case["stride"])
     np.testing.assert_array_equal(again, got[perm])
+
+
+LARGE_FILTER_CASES = [
+    dict(x=(40, 37, 32, 64), w=(72, 5, 5, 64), pad=(-2, -2)),    # 5 x 5: dense 8 x 32 tiles in the large-halo layout, a partial last tile, a partial filter block
+    dict(x=(48, 30, 33, 64), w=(64, 7, 7, 64), pad=(-3, -3)),    # 7 x 7
+    dict(x=(96, 12, 70, 64), w=(64, 1, 9, 64), pad=(0, -4)),     # one line of nine taps over wide rows
+]
+
+
+@pytest.mark.parametrize("case", LARGE_FILTER_CASES, ids=["5x5", "7x7", "1x9"])
+def test_large_filters_many_images(oracle, case):
+    """Enough (image, tile) pairs that the image-tile kernel takes its layout with one workgroup per compute unit and tiles in
+    dense row order; bf16 against the oracle on sampled images, int8 -> int32 bit-exact on the same images."""
+    g = h.rng(47)
+    K = case["w"][0]
+    N = case["x"][0]
+    images = (0, N // 2, N - 1)
+    Ho, Wo = oracle.conv_output_shape(case["x"][1], case["x"][2], case["w"][1], case["w"][2], case["pad"])
+    x = h.rounded(oracle, g.standard_normal(case["x"]), "bf16")
+    w = h.rounded(oracle, he(g, case["w"]), "bf16")
+    b = g.uniform(-0.1, 0.1, K).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal((N, Ho, Wo, K)), "bf16")
+    got = h.conv_forward("implicit_gemm", x, w, (N, Ho, Wo, K), "bf16", bias=b, z=z, activation=cb.ACTIVATION_RELU, pad=case["pad"])
+    check_images(oracle, got, x, w, b, z, images, BAR["bf16"], pad=case["pad"])
+    xi = g.integers(-127, 128, case["x"], dtype=np.int8)
+    wi = g.integers(-127, 128, case["w"], dtype=np.int8)
+    bi = g.integers(-2 ** 15, 2 ** 15, K).astype(np.int32)
+    goti = h.conv_forward("implicit_gemm", xi, wi, (N, Ho, Wo, K), "i8", y_dtype="i32", bias=bi, bias_dtype="i32", activation=cb.ACTIVATION_RELU, pad=case["pad"])
+    for n in images:
+        np.testing.assert_array_equal(goti[n:n + 1], oracle.conv2d_i8(xi[n:n + 1], wi, bi, pad=case["pad"], activation=cb.ACTIVATION_RELU))
