@@ -12,7 +12,7 @@
  *   - only the weights stream: 64 filters x 128 bytes per step, fetched three steps ahead into registers (three sets) and
  *     double buffered in LDS;
  *   - the halo of the next channel slice is fetched during the third tap of the current one and held in registers.
- * Four wavefronts stack in M (64 pixels x 64 filters each, 2 x 2 MFMA tiles of 32 x 32); 61 KB of LDS and <= 256 registers
+ * Four wavefronts stack in M (64 pixels x 64 filters each, 2 x 2 MFMA tiles of 32 x 32); 72 KB of LDS and <= 256 registers
  * let two workgroups share a CU.  k order is (channel slice, tap), which sums the same products as (tap, channel).
  *
  * The 256 rows of the workgroup's GEMM tile are NOT the TH x TW output pixels in raster order: row q stands for halo
@@ -20,6 +20,9 @@
  * nobody stores.  In exchange the A operand of tap (i, j) for row q is halo pixel q + i * HW + j: the 32 rows of an MFMA
  * tile always read 32 CONSECUTIVE halo pixels, whatever the tap, and with the 144-byte pixel pitch that is free of LDS
  * bank conflicts (raster order breaks the run at every tile-row end), and no per-row division is needed for the addresses.
+ * The general instance (filters other than 3 x 3) may be launched in raster ("dense") order instead, and with an LDS layout
+ * that holds a larger halo at one workgroup per compute unit: a wide tile under a large filter does not fit 256 rows in halo
+ * order, and fewer, fuller tiles then outweigh the conflicts (see TileLds and choose_tile).
  *
  * Epilogue: the accumulators leave through LDS so that a work-item stores 16 bytes of consecutive filters of one pixel with a
  * streaming store; a table in LDS maps GEMM rows to output pixels; the residual z of the rows a work-item will store is fetched
