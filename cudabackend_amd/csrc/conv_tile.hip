@@ -675,26 +675,51 @@ namespace avhip
 		const int64_t filter_blocks = (static_cast<int64_t>(s.K) + TILE_N - 1) / TILE_N;
 		const int64_t resident = static_cast<int64_t>(persistent_workgroups(1ll << 40));
 		const int steps = s.R * s.S * ((s.C * static_cast<int>(sizeof(TE)) + STEP_BYTES - 1) / STEP_BYTES);
-		const bool general = s.R != 3 || s.S != 3; /* the instance with the general k loop: either row order, either LDS layout */
-		TileChoice pick = choose_tile(s, HALO_SMALL, TileLds<HALO_SMALL>::pixels, general);
-		bool big = false;
-		if (general)
+		auto plan = [&](TileChoice &pick, bool &big)
 		{
-			const TileChoice wide = choose_tile(s, HALO_BIG, TileLds<HALO_BIG>::pixels, true);
-			if (wide.tiles > 0)
+			const bool general = s.R != 3 || s.S != 3; /* the instance with the general k loop: either row order, either LDS layout */
+			pick = choose_tile(s, HALO_SMALL, TileLds<HALO_SMALL>::pixels, general);
+			big = false;
+			if (general)
 			{
-				const int64_t wide_groups = static_cast<int64_t>(s.N) * wide.tiles * filter_blocks, groups = static_cast<int64_t>(s.N) * pick.tiles * filter_blocks;
-				const double wide_cost = static_cast<double>((wide_groups + resident / 2 - 1) / (resident / 2)) * (steps * 0.47 + 3.6);
-				const double cost = static_cast<double>((groups + resident - 1) / resident) * (steps * (groups > resident / 2 ? 0.68 : 0.47) + 3.6);
-				/* (tiles that would be mostly padding send the layer to the gather kernel, see below: then the other layout is
-				 * the only candidate) */
-				const bool mostly_padding = pick.tiles > 0 && static_cast<double>(s.Ho) * s.Wo < 0.5 * pick.tiles * TILE_M;
-				if (pick.tiles == 0 || mostly_padding || wide_cost < 0.9 * cost)
+				const TileChoice wide = choose_tile(s, HALO_BIG, TileLds<HALO_BIG>::pixels, true);
+				if (wide.tiles > 0)
 				{
-					pick = wide;
-					big = true;
+					const int64_t wide_groups = static_cast<int64_t>(s.N) * wide.tiles * filter_blocks, groups = static_cast<int64_t>(s.N) * pick.tiles * filter_blocks;
+					const double wide_cost = static_cast<double>((wide_groups + resident / 2 - 1) / (resident / 2)) * (steps * 0.47 + 3.6);
+					const double cost = static_cast<double>((groups + resident - 1) / resident) * (steps * (groups > resident / 2 ? 0.68 : 0.47) + 3.6);
+					/* (tiles that would be mostly padding send the layer to the gather kernel, see below: then the other layout is
+					 * the only candidate) */
+					const bool mostly_padding = pick.tiles > 0 && static_cast<double>(s.Ho) * s.Wo < 0.5 * pick.tiles * TILE_M;
+					if (pick.tiles == 0 || mostly_padding || wide_cost < 0.9 * cost)
+					{
+						pick = wide;
+						big = true;
+					}
 				}
 			}
+		};
+		/* the search walks a few thousand candidate tiles: a caller that issues the same layer again (a network does nothing
+		 * else) gets the answer of the last search of its thread */
+		struct Plan
+		{
+			int N, Ho, Wo, R, S, K, C, element;
+			TileChoice pick;
+			bool big;
+		};
+		static thread_local Plan last = { 0, 0, 0, 0, 0, 0, 0, 0, { 0, 0, 0, 0 }, false };
+		TileChoice pick;
+		bool big;
+		if (last.N == s.N && last.Ho == s.Ho && last.Wo == s.Wo && last.R == s.R && last.S == s.S && last.K == s.K && last.C == s.C
+				&& last.element == static_cast<int>(sizeof(TE)))
+		{
+			pick = last.pick;
+			big = last.big;
+		}
+		else
+		{
+			plan(pick, big);
+			last = { s.N, s.Ho, s.Wo, s.R, s.S, s.K, s.C, static_cast<int>(sizeof(TE)), pick, big };
 		}
 		if (pick.tiles == 0)
 			return false;
