@@ -34,6 +34,9 @@
 #include "persistent_gemm.hpp"
 #include <type_traits>
 
+/* Instrumentation, compiled in with -DCONV_TILE_STAMPS only: wavefront 0 of every workgroup records the 100 MHz wall clock at
+ * the phase boundaries of the kernel (start, arguments read, requests out, halo in LDS, first MFMA, loop end, epilogue end), and
+ * avhip_debug_stamps() copies the records of the last launch to the host.  The phase timings quoted for this kernel come from it. */
 #ifdef CONV_TILE_STAMPS
 __device__ unsigned long long g_stamps[4096 * 8];
 #define STAMP(i) do { if (threadIdx.x == 0) g_stamps[(blockIdx.x % 4096) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
