@@ -260,7 +260,7 @@ namespace
 		{
 			/* GEMM row -> offset of its output pixel inside the image of y, in elements; -1 for rows that are not stored */
 			/* (the written-out 3 x 3 instance is launched in halo order only and spends nothing on the other one) */
-			const unsigned int pitch = FS == 0 ? static_cast<unsigned int>(g.row_pitch) : static_cast<unsigned int>(g.HW), magic = FS == 0 ? g.row_magic : g.hw_magic;
+			const unsigned int pitch = FS != 3 ? static_cast<unsigned int>(g.row_pitch) : static_cast<unsigned int>(g.HW), magic = FS != 3 ? g.row_magic : g.hw_magic;
 			const int py = static_cast<int>((static_cast<unsigned int>(tid) * magic) >> 20), px = tid - py * static_cast<int>(pitch);
 			const int oh = oh0 + py, ow = ow0 + px;
 			row_table[tid] = (py < g.TH && px < g.TW && oh < g.Ho && ow < g.Wo) ? (oh * g.Wo + ow) * g.K : -1; /* times K here, once, not in every use */
@@ -333,7 +333,7 @@ namespace
 #pragma unroll
 		for (int tm = 0; tm < 2; tm++)
 			a_off[tm] = (wave * 64 + tm * 32 + (lane & 31)) * PIXEL_PITCH + (lane >> 5) * 16;
-		if (FS == 0 && g.row_pitch != g.HW) /* (uniform) */
+		if (FS != 3 && g.row_pitch != g.HW) /* (uniform) */
 		{
 #pragma unroll
 			for (int tm = 0; tm < 2; tm++)
@@ -423,7 +423,9 @@ namespace
 			constexpr int TAPS = FS * FS;
 			constexpr int SLABS = STEP_BYTES / 32;
 			constexpr int PREFETCH_TAP = 2;
-			static_assert(TAPS % FILTER_RING == 0, "the ring phase must be the same in every channel slice");
+			/* (5 x 5: 25 taps shift the ring phase from one slice to the next, so that instance is launched for layers of a single
+			 * channel slice only) */
+			static_assert(TAPS % FILTER_RING == 0 || FS == 5, "the ring phase must be the same in every channel slice");
 			stash_filters(1, fr[1]);
 			const int row_pitch = g.HW * PIXEL_PITCH;
 			const int flip_base = g.flip ? (FS - 1) * (row_pitch + PIXEL_PITCH) : 0;
@@ -536,7 +538,7 @@ namespace
 					stash_halo(hr);
 				}
 			};
-			if (g.slices == 1)
+			if (g.slices == 1 || TAPS % FILTER_RING != 0)
 				slice_steps(0, std::true_type(), std::true_type());
 			else
 			{
@@ -770,6 +772,8 @@ namespace avhip
 		const dim3 grid(static_cast<unsigned int>(blocks * filter_blocks));
 		if (s.R == 3 && s.S == 3)
 			hipLaunchKernelGGL((k_conv_tile<TE, Epi, 3>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
+		else if (big && s.R == 5 && s.S == 5 && g.slices == 1)
+			hipLaunchKernelGGL((k_conv_tile<TE, Epi, 5, HALO_BIG>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
 		else if (big)
 			hipLaunchKernelGGL((k_conv_tile<TE, Epi, 0, HALO_BIG>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi);
 		else

@@ -178,3 +178,38 @@ def test_large_filters_many_images(oracle, case):
     goti = h.conv_forward("implicit_gemm", xi, wi, (N, Ho, Wo, K), "i8", y_dtype="i32", bias=bi, bias_dtype="i32", activation=cb.ACTIVATION_RELU, pad=case["pad"])
     for n in images:
         np.testing.assert_array_equal(goti[n:n + 1], oracle.conv2d_i8(xi[n:n + 1], wi, bi, pad=case["pad"], activation=cb.ACTIVATION_RELU))
+
+
+def test_written_out_5x5_int8_bit_exact(oracle):
+    """5 x 5 over one 128-byte channel slice (128 int8 channels) and enough images for the large-halo layout: the written-out
+    25-tap instance, int32 and requantised int8 results bit-exact on sampled images, partial tiles at the lower edge."""
+    g = h.rng(48)
+    shape, wshape, pad = (40, 37, 32, 128), (72, 5, 5, 128), (-2, -2)
+    N, K = shape[0], wshape[0]
+    x = g.integers(-127, 128, shape, dtype=np.int8)
+    w = g.integers(-127, 128, wshape, dtype=np.int8)
+    b = g.integers(-2 ** 15, 2 ** 15, K).astype(np.int32)
+    scale = g.uniform(1e-5, 1e-4, K).astype(np.float32)
+    ys = (N, 37, 32, K)
+    got = h.conv_forward("implicit_gemm", x, w, ys, "i8", y_dtype="i32", bias=b, bias_dtype="i32", activation=cb.ACTIVATION_RELU, pad=pad)
+    q = h.conv_forward("requant", x, w, ys, "i8", y_dtype="i8", bias=b, bias_dtype="i32", scale=scale, activation=cb.ACTIVATION_RELU, pad=pad)
+    for n in (0, 17, N - 1):
+        want = oracle.conv2d_i8(x[n:n + 1], w, b, pad=pad, activation=cb.ACTIVATION_RELU)
+        np.testing.assert_array_equal(got[n:n + 1], want)
+        np.testing.assert_array_equal(q[n:n + 1], oracle.requant_i8(want, scale))
+
+
+@pytest.mark.parametrize("dtype,channels", [("f32", 32), ("f16", 64), ("bf16", 48)])
+def test_written_out_5x5_floating(oracle, dtype, channels):
+    """The same instance for the floating types (one channel slice each; 48 bf16 channels leave the slice partly empty), with
+    bias, residual and ReLU, flipped filters included."""
+    g = h.rng(49)
+    shape, wshape, pad = (40, 37, 32, channels), (72, 5, 5, channels), (-2, -2)
+    N, K = shape[0], wshape[0]
+    x = h.rounded(oracle, g.standard_normal(shape), dtype)
+    w = h.rounded(oracle, he(g, wshape), dtype)
+    b = g.uniform(-0.1, 0.1, K).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal((N, 37, 32, K)), dtype)
+    for mode in (0, 1):
+        got = h.conv_forward("implicit_gemm", x, w, (N, 37, 32, K), dtype, bias=b, z=z, activation=cb.ACTIVATION_RELU, pad=pad, mode=mode)
+        check_images(oracle, got, x, w, b, z, (0, 21, N - 1), BAR[dtype], pad=pad, mode=mode)
