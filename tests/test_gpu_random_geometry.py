@@ -97,3 +97,42 @@ def test_random_geometries_int8(oracle, tiling):
             np.testing.assert_array_equal(q, oracle.requant_i8(want, scale), err_msg="requant case %d %r" % (done, c))
     finally:
         lib.avhip_set_small_problem_threshold(previous)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "i8"])
+def test_random_wide_images_and_large_filters(oracle, dtype):
+    """Stride-1 layers with wide images, many images and filters up to 7 x 7: the shapes for which the image-tile kernel picks
+    between its two row orders and its two LDS layouts.  Sampled images against the oracle; int8 -> int32 bit-exact."""
+    g = h.rng(57 if dtype == "bf16" else 58)
+    done = 0
+    while done < 24:
+        R, S = int(g.choice([1, 2, 3, 4, 5, 7])), int(g.choice([1, 2, 3, 4, 5, 7]))
+        if R * S == 1:
+            continue
+        N, H, W = int(g.integers(8, 49)), int(g.integers(8, 41)), int(g.integers(20, 73))
+        Cin, K = int(g.choice([64, 128, 192])) if dtype == "i8" else int(g.choice([32, 64, 128])), int(g.choice([16, 64, 72]))
+        pad = (-int(g.integers(0, R)), -int(g.integers(0, S)))
+        mode = int(g.integers(0, 2))
+        Ho, Wo = oracle.conv_output_shape(H, W, R, S, pad)
+        if Ho < 1 or Wo < 1:
+            continue
+        done += 1
+        images = sorted(set(int(i) for i in g.integers(0, N, 2)))
+        if dtype == "i8":
+            x = g.integers(-127, 128, (N, H, W, Cin), dtype=np.int8)
+            w = g.integers(-127, 128, (K, R, S, Cin), dtype=np.int8)
+            b = g.integers(-2 ** 15, 2 ** 15, K).astype(np.int32)
+            got = h.conv_forward("implicit_gemm", x, w, (N, Ho, Wo, K), "i8", y_dtype="i32", bias=b, bias_dtype="i32", activation=cb.ACTIVATION_RELU, pad=pad, mode=mode)
+            for n in images:
+                want = oracle.conv2d_i8(x[n:n + 1], w, b, pad=pad, mode=mode, activation=cb.ACTIVATION_RELU)
+                assert np.array_equal(got[n:n + 1], want), "case %d: N=%d %dx%d C=%d K=%d %dx%d pad=%r mode=%d image %d" % (done, N, H, W, Cin, K, R, S, pad, mode, n)
+        else:
+            x = h.rounded(oracle, g.standard_normal((N, H, W, Cin)), dtype)
+            w = h.rounded(oracle, g.standard_normal((K, R, S, Cin)) * np.sqrt(2.0 / (R * S * Cin)), dtype)
+            b = g.uniform(-0.1, 0.1, K).astype(np.float32).astype(np.float64)
+            z = h.rounded(oracle, g.standard_normal((N, Ho, Wo, K)), dtype)
+            got = h.conv_forward("dispatch", x, w, (N, Ho, Wo, K), dtype, bias=b, z=z, activation=cb.ACTIVATION_RELU, pad=pad, mode=mode)
+            for n in images:
+                want = oracle.conv2d(x[n:n + 1], w, b, z[n:n + 1], activation=oracle.RELU, pad=pad, mode=mode)
+                err = oracle.rel_l2(got[n:n + 1], want)
+                assert err < 2e-3, "case %d: N=%d %dx%d C=%d K=%d %dx%d pad=%r mode=%d image %d: rel-L2 %.3e" % (done, N, H, W, Cin, K, R, S, pad, mode, n, err)
