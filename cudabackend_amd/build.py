@@ -24,11 +24,12 @@ SOURCES = [
     "conv_tile.hip",
     "conv_small.hip",
     "conv_stem.hip",
+    "conv_thin.hip",
     "conv_pointwise.hip",
     "conv_winograd_fused.hip",
     "elementwise.hip",
 ]
-HEADERS = ["common.hpp", "mfma_core.hpp", "conv_epilogue.hpp", "conv_tile.hpp", "conv_small.hpp", "conv_stem.hpp", "conv_pointwise.hpp", "persistent_gemm.hpp", "resident_gemm.hpp", "../../include/avocado_hip_kernels.h", "../../include/avocado_hip_backend.h",
+HEADERS = ["common.hpp", "mfma_core.hpp", "conv_epilogue.hpp", "conv_tile.hpp", "conv_small.hpp", "conv_stem.hpp", "conv_thin.hpp", "conv_pointwise.hpp", "persistent_gemm.hpp", "resident_gemm.hpp", "../../include/avocado_hip_kernels.h", "../../include/avocado_hip_backend.h",
            "../../include/avocado_backend_defs.h"]
 
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

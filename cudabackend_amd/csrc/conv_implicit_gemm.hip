@@ -23,6 +23,7 @@
 #include "conv_pointwise.hpp"
 #include "conv_small.hpp"
 #include "conv_stem.hpp"
+#include "conv_thin.hpp"
 #include "conv_tile.hpp"
 #include "mfma_core.hpp"
 
@@ -527,15 +528,19 @@ namespace
 		const bool fast = fast_path_ok<TE>(s, flags, padding_value) && is_simple_activation(epi.activation) && (flags & 2) != 0;
 		/* few input channels: pack (tap, channel) into the k-steps instead of spending a step per tap */
 		const int pixel_bytes = s.C * static_cast<int>(sizeof(TE));
-		if (pixel_bytes <= STEP_BYTES / 2 && s.R * s.S > 1 && fast_path_ok<TE>(s, 1, padding_value) && is_simple_activation(epi.activation) && (flags & 2) != 0)
+		if (pixel_bytes <= STEP_BYTES / 2 && s.R * s.S > 1 && fast_path_ok<TE>(s, 1, padding_value, false) && is_simple_activation(epi.activation)
+				&& (flags & 2) != 0)
 		{
 			/* a pixel of exactly 8 bytes and a small filter: operands straight into registers, no k loop */
 			if (conv_stem_launch<TE, Epi>(st, s, x, w, epi))
 				return 0;
+			/* the image tile in LDS, the operand gathered from there: filters of any number of taps */
+			if (conv_thin_launch<TE, Epi>(st, s, x, w, epi))
+				return 0;
 			int pb = 16;
 			while (pb > 1 && (pixel_bytes % pb != 0 || !aligned_to(x, pb) || !aligned_to(w, pb)))
 				pb /= 2;
-			pb = pb < static_cast<int>(sizeof(TE)) ? 0 : pb;
+			pb = (pb < static_cast<int>(sizeof(TE)) || s.R * s.S > 32) ? 0 : pb; /* the gather kernel's tap mask has 32 bits */
 #define AVHIP_PACKED(PB) hipLaunchKernelGGL((k_conv_igemm_packed<TE, PB, Epi>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi)
 			switch (pb)
 			{

@@ -1,0 +1,439 @@
+/*
+ * conv_thin.hip -- implicit-GEMM convolution for layers whose input has few channels and whose filter may be large: the
+ * 7 x 7, stride-2 first layer of a residual network over three image planes is the type.
+ *
+ * Same arithmetic as the implicit-GEMM forward of the reference (src/conv2d_implicit_gemm.cu:152-301).  With so few
+ * channels one tap holds a handful of bytes, so k is the flattened (tap, channel) index of a filter row, R * S * C elements
+ * long, and a 16-byte MFMA operand chunk of an output pixel is put together from 16 / PB pieces of PB bytes, each from the
+ * input pixel its tap reads (PB: the largest power of two that divides the bytes of a pixel, so a piece never straddles two
+ * taps).  Gathering such pieces from global memory costs one cache-line look-up per work-item and piece; here the image
+ * tile that a workgroup's 256 output pixels read is brought into LDS once, with neighbouring work-items reading neighbouring
+ * addresses, and the pieces are gathered from LDS, which serves 32 scattered work-items per cycle.
+ *
+ * One workgroup = one tile of TH x TW = 256 output pixels of one image (TW a power of two, chosen per layer) times all the
+ * filters, 64 at a time.  In LDS:
+ *   the halo: the (TH-1)*stride + (R-1)*dilation + 1 image rows under the tile, zeros where the image ends;
+ *   a table with, for every piece of k, its byte offset from the window origin of a pixel (the same for every pixel);
+ *   the 64 filters of the current block, rows padded with zeros to whole 32-byte MFMA slabs; the accumulators leave through
+ *   the same bytes afterwards.
+ * A wavefront owns 64 pixels (two MFMA tiles) by 64 filters; per 32-byte slab of k it gathers two operand chunks from the
+ * halo, reads two filter chunks and issues four MFMAs.  No barrier inside the k loop.
+ */
+#include "conv_thin.hpp"
+#include "mfma_core.hpp"
+#include <algorithm>
+#include <type_traits>
+
+namespace
+{
+	using namespace avhip;
+
+	constexpr int THIN_FILTERS = 64; /* filters per block */
+	constexpr int THIN_LDS = 80 * 1024; /* two workgroups per compute unit */
+	constexpr int THIN_MAX_K_BYTES = 1024;
+	constexpr int THIN_MAX_PIXEL_BYTES = 64;
+	constexpr unsigned int THIN_NO_PIECE = 0xFFFFFFFFu; /* table entry of a piece past the end of k */
+
+	struct ThinGeom
+	{
+		int H, W, K, Ho, Wo, R, S;
+		int pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, flip;
+		int tw_shift; /* the tile is (256 >> tw_shift) rows of (1 << tw_shift) output pixels */
+		unsigned int tiles_x, tiles_per_image;
+		unsigned int pixel_bytes, k_bytes, kgroups; /* kgroups: 32-byte slabs of k, the last one padded */
+		unsigned int halo_pitch, halo_pieces, pieces_per_row; /* halo row = pieces_per_row pieces = halo_pitch bytes, rows back to back */
+		unsigned int step_rows, step_pieces; /* 256 pieces further on: this many rows and pieces down the halo */
+		unsigned int halo_bytes, table_bytes; /* LDS regions, multiples of 16 */
+		unsigned int w_pitch; /* LDS pitch of a padded filter row: an odd number of 16-byte units */
+		unsigned int x_bytes, w_bytes;
+		unsigned int filter_blocks;
+	};
+
+	/* A piece of PB bytes: its register type, its load from a tensor (zeros at OUT_OF_RANGE) */
+	template<int PB> struct ThinPiece;
+	template<> struct ThinPiece<16>
+	{
+		typedef u32x4_t type;
+		__device__ static inline type get(__amdgpu_buffer_rsrc_t r, unsigned int off)
+		{
+			return __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(off), 0, 0);
+		}
+	};
+	template<> struct ThinPiece<8>
+	{
+		typedef u32x2_t type;
+		__device__ static inline type get(__amdgpu_buffer_rsrc_t r, unsigned int off)
+		{
+			return __builtin_amdgcn_raw_buffer_load_b64(r, static_cast<int>(off), 0, 0);
+		}
+	};
+	template<> struct ThinPiece<4>
+	{
+		typedef unsigned int type;
+		__device__ static inline type get(__amdgpu_buffer_rsrc_t r, unsigned int off)
+		{
+			return __builtin_amdgcn_raw_buffer_load_b32(r, static_cast<int>(off), 0, 0);
+		}
+	};
+	template<> struct ThinPiece<2>
+	{
+		typedef unsigned short type;
+		__device__ static inline type get(__amdgpu_buffer_rsrc_t r, unsigned int off)
+		{
+			return __builtin_amdgcn_raw_buffer_load_b16(r, static_cast<int>(off), 0, 0);
+		}
+	};
+	template<> struct ThinPiece<1>
+	{
+		typedef unsigned char type;
+		__device__ static inline type get(__amdgpu_buffer_rsrc_t r, unsigned int off)
+		{
+			return __builtin_amdgcn_raw_buffer_load_b8(r, static_cast<int>(off), 0, 0);
+		}
+	};
+	template<int PB>
+	union ThinChunk
+	{
+		uint4 u;
+		typename ThinPiece<PB>::type piece[16 / PB];
+	};
+
+	template<typename TE, int PB, typename Epi>
+	__global__ __launch_bounds__(256, 2) void k_conv_thin(const TE *__restrict__ x, const TE *__restrict__ w, ThinGeom g, Epi epi)
+	{
+		epi.pin();
+		constexpr int NP = 16 / PB;
+		constexpr int W = Epi::wide;
+		typedef typename ThinPiece<PB>::type piece_t;
+		__shared__ __attribute__((aligned(16))) char lds[THIN_LDS];
+		const int tid = threadIdx.x;
+		const int lane = tid & 63;
+		const int wave = tid >> 6;
+		const int half = lane >> 5; /* which 16 bytes of a 32-byte slab this lane supplies */
+
+		const unsigned int n = blockIdx.x / g.tiles_per_image;
+		const unsigned int in_image = blockIdx.x - n * g.tiles_per_image;
+		const unsigned int tile_y = in_image / g.tiles_x, tile_x = in_image - tile_y * g.tiles_x;
+		const int TW = 1 << g.tw_shift;
+		const int oh0 = static_cast<int>(tile_y) * (256 >> g.tw_shift), ow0 = static_cast<int>(tile_x) * TW;
+
+		unsigned int *table = reinterpret_cast<unsigned int*>(lds + g.halo_bytes);
+		const unsigned int zero_at = g.halo_bytes + g.table_bytes; /* 16 bytes of zeros: what a piece past the end of k reads */
+		char *filters = lds + zero_at + 16;
+
+		/* the table: entry (slab, half, piece) = offset of that piece of k from the window origin of a pixel */
+		for (unsigned int idx = tid; idx < g.kgroups * 2 * NP; idx += 256)
+		{
+			const unsigned int b = (idx / NP) * 16 + (idx % NP) * PB;
+			unsigned int rel = THIN_NO_PIECE;
+			if (b < g.k_bytes)
+			{
+				const unsigned int tap = b / g.pixel_bytes, within = b - tap * g.pixel_bytes;
+				int i = static_cast<int>(tap / g.S), j = static_cast<int>(tap - (tap / g.S) * g.S);
+				if (g.flip)
+				{
+					i = g.R - 1 - i;
+					j = g.S - 1 - j;
+				}
+				rel = static_cast<unsigned int>(i * g.dil_h) * g.halo_pitch + static_cast<unsigned int>(j * g.dil_w) * g.pixel_bytes + within;
+			}
+			table[idx] = rel;
+		}
+		if (tid < 4)
+			reinterpret_cast<unsigned int*>(lds + zero_at)[tid] = 0u;
+
+		/* the halo, piece by piece: consecutive work-items read consecutive pieces of an image row */
+		{
+			const __amdgpu_buffer_rsrc_t rx = make_buffer(x, g.x_bytes);
+			const int ih_base = oh0 * g.stride_h + g.pad_h;
+			const int column_base = (ow0 * g.stride_w + g.pad_w) * static_cast<int>(g.pixel_bytes); /* byte column of the halo's first pixel */
+			const int row_bytes = g.W * static_cast<int>(g.pixel_bytes);
+			unsigned int row = tid / g.pieces_per_row, piece = tid - row * g.pieces_per_row;
+			constexpr int BATCH = 8;
+			for (unsigned int first = 0; first < g.halo_pieces; first += 256 * BATCH)
+			{
+				piece_t value[BATCH];
+#pragma unroll
+				for (int u = 0; u < BATCH; u++)
+				{
+					const unsigned int q = first + u * 256 + tid;
+					const int ih = ih_base + static_cast<int>(row);
+					const int column = column_base + static_cast<int>(piece) * PB;
+					const bool inside = (q < g.halo_pieces) & (ih >= 0) & (ih < g.H) & (column >= 0) & (column < row_bytes);
+					value[u] = ThinPiece<PB>::get(rx, inside ? static_cast<unsigned int>((static_cast<int>(n) * g.H + ih) * row_bytes + column) : OUT_OF_RANGE);
+					row += g.step_rows;
+					piece += g.step_pieces;
+					if (piece >= g.pieces_per_row)
+					{
+						piece -= g.pieces_per_row;
+						row++;
+					}
+				}
+#pragma unroll
+				for (int u = 0; u < BATCH; u++)
+				{
+					const unsigned int q = first + u * 256 + tid;
+					if (q < g.halo_pieces)
+						*reinterpret_cast<piece_t*>(lds + q * PB) = value[u];
+				}
+			}
+		}
+
+		/* window origin of this lane's two output pixels (pixel m of the tile is row m >> tw_shift, column m & (TW - 1)) */
+		unsigned int origin[2];
+#pragma unroll
+		for (int tm = 0; tm < 2; tm++)
+		{
+			const int m = wave * 64 + tm * 32 + (lane & 31);
+			origin[tm] = static_cast<unsigned int>((m >> g.tw_shift) * g.stride_h) * g.halo_pitch
+					+ static_cast<unsigned int>((m & (TW - 1)) * g.stride_w) * g.pixel_bytes;
+		}
+
+		const __amdgpu_buffer_rsrc_t rw = make_buffer(w, g.w_bytes);
+		for (unsigned int fb = 0; fb < g.filter_blocks; fb++)
+		{
+			const int f0 = static_cast<int>(fb) * THIN_FILTERS;
+			const int kcol = f0 + drain_column<1, W>();
+			typename Epi::template ColumnsT<W> columns;
+			epi.load_columns(kcol, columns);
+			__syncthreads(); /* the accumulators of the previous block have left the filter region */
+
+			/* filter rows f0 .. f0 + 63 lie back to back in w: read as aligned 16-byte chunks, written to the padded rows piece
+			 * by piece (a chunk may run over the end of a filter row) */
+			{
+				const unsigned int rows = static_cast<unsigned int>(g.K - f0 < THIN_FILTERS ? g.K - f0 : THIN_FILTERS);
+				const unsigned int total = rows * g.k_bytes, w_first = static_cast<unsigned int>(f0) * g.k_bytes;
+				const unsigned int tail_pieces = (g.kgroups * 32 - g.k_bytes) / PB;
+				for (unsigned int idx = tid; idx < THIN_FILTERS * tail_pieces; idx += 256)
+				{
+					piece_t nothing = {};
+					*reinterpret_cast<piece_t*>(filters + (idx & (THIN_FILTERS - 1)) * g.w_pitch + g.k_bytes + (idx / THIN_FILTERS) * PB) = nothing;
+				}
+				for (unsigned int off = tid * 16; off < total; off += 256 * 16)
+				{
+					ThinChunk<PB> chunk;
+					if (off + 16 <= total)
+						chunk.u = buffer_fetch(rw, w_first + off);
+					else
+					{
+#pragma unroll
+						for (int e = 0; e < NP; e++)
+							chunk.piece[e] = ThinPiece<PB>::get(rw, off + e * PB < total ? w_first + off + e * PB : OUT_OF_RANGE);
+					}
+					unsigned int row = off / g.k_bytes, column = off - row * g.k_bytes;
+#pragma unroll
+					for (int e = 0; e < NP; e++)
+					{
+						if (off + e * PB < total)
+							*reinterpret_cast<piece_t*>(filters + row * g.w_pitch + column) = chunk.piece[e];
+						column += PB;
+						if (column >= g.k_bytes)
+						{
+							column = 0;
+							row++;
+						}
+					}
+				}
+			}
+			__syncthreads();
+
+			typename Mma<TE>::acc_t acc[2][2];
+#pragma unroll
+			for (int i = 0; i < 2; i++)
+#pragma unroll
+				for (int j = 0; j < 2; j++)
+#pragma unroll
+					for (int v = 0; v < 16; v++)
+						acc[i][j][v] = 0;
+			const char *filter_row = filters + (lane & 31) * g.w_pitch + half * 16;
+			const unsigned int *table_row = table + half * NP;
+			auto slab = [&](unsigned int kg, auto last) __attribute__((always_inline))
+			{
+				unsigned int rel[NP];
+#pragma unroll
+				for (int e = 0; e < NP; e++)
+					rel[e] = table_row[kg * 2 * NP + e];
+				Chunk a[2], b[2];
+#pragma unroll
+				for (int tm = 0; tm < 2; tm++)
+				{
+					ThinChunk<PB> chunk;
+#pragma unroll
+					for (int e = 0; e < NP; e++)
+					{
+						unsigned int at = origin[tm] + rel[e];
+						if (decltype(last)::value) /* only the last slab has pieces past the end of k */
+							at = rel[e] == THIN_NO_PIECE ? zero_at : at;
+						chunk.piece[e] = *reinterpret_cast<const piece_t*>(lds + at);
+					}
+					a[tm].u = chunk.u;
+				}
+#pragma unroll
+				for (int tn = 0; tn < 2; tn++)
+					b[tn].u = *reinterpret_cast<const uint4*>(filter_row + tn * 32 * g.w_pitch + kg * 32);
+#pragma unroll
+				for (int tm = 0; tm < 2; tm++)
+#pragma unroll
+					for (int tn = 0; tn < 2; tn++)
+						Mma<TE>::run(a[tm], b[tn], acc[tm][tn]);
+			};
+			for (unsigned int kg = 0; kg + 1 < g.kgroups; kg++)
+				slab(kg, std::false_type());
+			slab(g.kgroups - 1, std::true_type());
+
+			drain_tile_private<TE, 2, W>(filters, acc, [&](int row, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
+			{
+				const int oh = oh0 + (row >> g.tw_shift), ow = ow0 + (row & (TW - 1));
+				if (oh < g.Ho && ow < g.Wo && kcol < g.K)
+					epi.template store_at<ACT_SIMPLE, true, W>((static_cast<int64_t>(static_cast<int>(n) * g.Ho + oh) * g.Wo + ow) * g.K + kcol, kcol, v, columns,
+							nullptr);
+			});
+		}
+	}
+
+	/* a workgroup stores 64 filters of a pixel: int8 results are half a cache line, which is best written through */
+	template<typename TE> FloatEpilogue<TE> for_partial_lines(const FloatEpilogue<TE> &epi)
+	{
+		return epi;
+	}
+	template<int MODE> Int8Epilogue<MODE> for_partial_lines(const Int8Epilogue<MODE> &epi)
+	{
+		Int8Epilogue<MODE> e = epi;
+		e.through = true;
+		return e;
+	}
+	unsigned int round_up(unsigned int v, unsigned int to)
+	{
+		return (v + to - 1) / to * to;
+	}
+}
+
+namespace avhip
+{
+	template<typename TE, typename Epi>
+	bool conv_thin_launch(hipStream_t stream, const avhipConvShape &s, const void *x, const void *w, const Epi &caller_epi)
+	{
+		const Epi epi = for_partial_lines(caller_epi);
+		const int pixel_bytes = s.C * static_cast<int>(sizeof(TE));
+		const int64_t k_bytes = static_cast<int64_t>(s.R) * s.S * pixel_bytes;
+		if (pixel_bytes > THIN_MAX_PIXEL_BYTES || k_bytes > THIN_MAX_K_BYTES)
+			return false;
+		int pb = 16;
+		while (pb > 1 && (pixel_bytes % pb != 0 || !aligned_to(x, pb)))
+			pb /= 2;
+		if (pb < static_cast<int>(sizeof(TE)) || !aligned_to(w, 16))
+			return false;
+		/* whole runs of Epi::wide filters leave with one vector store */
+		if (!epi.vec || s.K % Epi::wide != 0 || !aligned_to(epi.y, 16) || (epi.z != nullptr && !aligned_to(epi.z, 16)))
+			return false;
+		const int64_t x_bytes = static_cast<int64_t>(s.N) * s.H * s.W * pixel_bytes, w_bytes = static_cast<int64_t>(s.K) * k_bytes;
+		if (x_bytes >= (1ll << 31) || w_bytes >= (1ll << 31))
+			return false;
+
+		ThinGeom g;
+		g.kgroups = static_cast<unsigned int>((k_bytes + 31) / 32);
+		g.w_pitch = g.kgroups * 32 + 16;
+		g.table_bytes = round_up(g.kgroups * 2 * (16 / pb) * 4, 16);
+		const unsigned int drain_bytes = 4 * PrivateDrainRows<2, Epi::wide>::bytes;
+		const unsigned int fixed_bytes = g.table_bytes + 16 + std::max<unsigned int>(THIN_FILTERS * g.w_pitch, drain_bytes);
+		/* the tile shape: as few tiles as possible, then the smallest halo */
+		int best_shift = -1;
+		int64_t best_tiles = 0, best_halo = 0;
+		for (int shift = 0; shift <= 8; shift++)
+		{
+			const int tw = 1 << shift, th = 256 >> shift;
+			const int64_t halo_rows = static_cast<int64_t>(th - 1) * s.stride_h + static_cast<int64_t>(s.R - 1) * s.dil_h + 1;
+			const int64_t halo_columns = static_cast<int64_t>(tw - 1) * s.stride_w + static_cast<int64_t>(s.S - 1) * s.dil_w + 1;
+			const int64_t halo = halo_rows * halo_columns * pixel_bytes;
+			if (halo + 16 + fixed_bytes > THIN_LDS)
+				continue;
+			const int64_t tiles = static_cast<int64_t>((s.Ho + th - 1) / th) * ((s.Wo + tw - 1) / tw);
+			if (best_shift < 0 || tiles < best_tiles || (tiles == best_tiles && halo < best_halo))
+			{
+				best_shift = shift;
+				best_tiles = tiles;
+				best_halo = halo;
+			}
+		}
+		if (best_shift < 0)
+			return false;
+		/* images much smaller than a tile leave most of the MFMA rows empty */
+		if (static_cast<int64_t>(s.Ho) * s.Wo * 10 < best_tiles * 256 * 3)
+			return false;
+		if (best_tiles * s.N >= (1ll << 31))
+			return false;
+		const int tw = 1 << best_shift, th = 256 >> best_shift;
+		g.H = s.H;
+		g.W = s.W;
+		g.K = s.K;
+		g.Ho = s.Ho;
+		g.Wo = s.Wo;
+		g.R = s.R;
+		g.S = s.S;
+		g.pad_h = s.pad_h;
+		g.pad_w = s.pad_w;
+		g.stride_h = s.stride_h;
+		g.stride_w = s.stride_w;
+		g.dil_h = s.dil_h;
+		g.dil_w = s.dil_w;
+		g.flip = s.mode != 0 ? 1 : 0;
+		g.tw_shift = best_shift;
+		g.tiles_x = static_cast<unsigned int>((s.Wo + tw - 1) / tw);
+		g.tiles_per_image = static_cast<unsigned int>(best_tiles);
+		g.pixel_bytes = static_cast<unsigned int>(pixel_bytes);
+		g.k_bytes = static_cast<unsigned int>(k_bytes);
+		const unsigned int halo_rows = static_cast<unsigned int>((th - 1) * s.stride_h + (s.R - 1) * s.dil_h + 1);
+		const unsigned int halo_columns = static_cast<unsigned int>((tw - 1) * s.stride_w + (s.S - 1) * s.dil_w + 1);
+		g.halo_pitch = halo_columns * g.pixel_bytes;
+		g.pieces_per_row = g.halo_pitch / pb;
+		g.halo_pieces = halo_rows * g.pieces_per_row;
+		g.step_rows = 256 / g.pieces_per_row;
+		g.step_pieces = 256 % g.pieces_per_row;
+		g.halo_bytes = round_up(halo_rows * g.halo_pitch, 16);
+		g.x_bytes = static_cast<unsigned int>(x_bytes);
+		g.w_bytes = static_cast<unsigned int>(w_bytes);
+		g.filter_blocks = static_cast<unsigned int>((s.K + THIN_FILTERS - 1) / THIN_FILTERS);
+		const dim3 grid(static_cast<unsigned int>(best_tiles * s.N));
+#define AVHIP_THIN(PB) hipLaunchKernelGGL((k_conv_thin<TE, PB, Epi>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi)
+		switch (pb)
+		{
+			case 16:
+				AVHIP_THIN(16);
+				return true;
+			case 8:
+				AVHIP_THIN(8);
+				return true;
+			case 4:
+				AVHIP_THIN(4);
+				return true;
+			case 2:
+				if constexpr (sizeof(TE) <= 2)
+				{
+					AVHIP_THIN(2);
+					return true;
+				}
+				return false;
+			case 1:
+				if constexpr (sizeof(TE) == 1)
+				{
+					AVHIP_THIN(1);
+					return true;
+				}
+				return false;
+			default:
+				return false;
+		}
+#undef AVHIP_THIN
+	}
+
+#define AVHIP_INSTANTIATE(TE, EPI) template bool conv_thin_launch<TE, EPI>(hipStream_t, const avhipConvShape&, const void*, const void*, const EPI&);
+	AVHIP_INSTANTIATE(float, FloatEpilogue<float>)
+	AVHIP_INSTANTIATE(f16_t, FloatEpilogue<f16_t>)
+	AVHIP_INSTANTIATE(bf16_t, FloatEpilogue<bf16_t>)
+	AVHIP_INSTANTIATE(int8_t, Int8Epilogue<I8_EXACT>)
+	AVHIP_INSTANTIATE(int8_t, Int8Epilogue<I8_REQUANT>)
+	AVHIP_INSTANTIATE(int8_t, Int8Epilogue<I8_FLOAT_I32>)
+	AVHIP_INSTANTIATE(int8_t, Int8Epilogue<I8_FLOAT_I8>)
+	AVHIP_INSTANTIATE(int8_t, Int8Epilogue<I8_FLOAT_F32>)
+#undef AVHIP_INSTANTIATE
+}

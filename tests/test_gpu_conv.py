@@ -124,6 +124,57 @@ def test_int8_few_input_channels_bit_exact(oracle, case):
     np.testing.assert_array_equal(got, oracle.conv2d_i8(x, w, b, activation=cb.ACTIVATION_RELU, **kw))
 
 
+# ---- few input channels, images large enough for 256-pixel tiles: the kernel that gathers its operand from a tile in LDS ------
+THIN_CASES = [
+    dict(x=(2, 40, 44, 3), w=(72, 7, 7, 3), pad=(-3, -3), stride=(2, 2)),                         # a residual network's first layer; the second filter block partial
+    dict(x=(2, 33, 35, 3), w=(64, 5, 5, 3), pad=(-2, -2), mode=1),                                # flipped; partial tiles at both edges
+    dict(x=(1, 50, 20, 1), w=(16, 9, 9, 1), pad=(-4, -4)),                                        # 81 taps of one plane
+    dict(x=(2, 24, 40, 6), w=(32, 3, 5, 6), pad=(-2, -4), dilation=(2, 2)),                       # dilated
+    dict(x=(2, 30, 30, 16), w=(40, 3, 3, 16), pad=(-1, -1), stride=(1, 2)),                       # whole 16-byte pieces
+    dict(x=(3, 20, 20, 5), w=(24, 4, 4, 5), pad=(-1, -2)),                                        # odd channel count, even filter
+    dict(x=(2, 70, 9, 4), w=(136, 7, 3, 4), pad=(-3, -1), stride=(3, 1), mode=1),                 # tall images, three filter blocks
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", THIN_CASES, ids=[str(i) for i in range(len(THIN_CASES))])
+def test_thin_kernel_with_residual(oracle, dtype, case):
+    g = h.rng(28)
+    x = h.rounded(oracle, g.standard_normal(case["x"]), dtype)
+    w = he(g, case["w"], dtype, oracle)
+    ys = out_shape(oracle, case)
+    b = g.uniform(-0.1, 0.1, ys[3]).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal(ys), dtype)
+    y0 = h.rounded(oracle, g.standard_normal(ys), dtype)
+    kw = dict(pad=case["pad"], stride=case.get("stride", (1, 1)), dilation=case.get("dilation", (1, 1)), mode=case.get("mode", 0))
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, **kw)
+    want = oracle.conv2d(x, w, **kw)
+    assert got.shape == want.shape
+    assert oracle.rel_l2(got, want) < BAR[dtype]
+    # every image separately: a tile that went to the wrong place would hide in a global norm
+    assert max(oracle.rel_l2(got[i], want[i]) for i in range(ys[0])) < 2 * BAR[dtype]
+    a2, be = float(np.float32(0.7)), float(np.float32(0.3))
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, bias=b, z=z, y0=y0, alpha2=a2, beta=be, activation=cb.ACTIVATION_RELU, **kw)
+    want = oracle.conv2d(x, w, b, z, y0, alpha2=a2, beta=be, activation=oracle.RELU, **kw)
+    assert oracle.rel_l2(got, want) < BAR[dtype]
+
+
+@pytest.mark.parametrize("case", THIN_CASES, ids=[str(i) for i in range(len(THIN_CASES))])
+def test_thin_kernel_int8_bit_exact(oracle, case):
+    g = h.rng(29)
+    x = g.integers(-127, 128, case["x"], dtype=np.int8)
+    w = g.integers(-127, 128, case["w"], dtype=np.int8)
+    K = case["w"][0]
+    b = g.integers(-2 ** 15, 2 ** 15, K).astype(np.int32)
+    kw = dict(pad=case["pad"], stride=case.get("stride", (1, 1)), dilation=case.get("dilation", (1, 1)), mode=case.get("mode", 0))
+    ys = out_shape(oracle, case)
+    got = h.conv_forward("implicit_gemm", x, w, ys, "i8", y_dtype="i32", bias=b, bias_dtype="i32", activation=cb.ACTIVATION_RELU, **kw)
+    np.testing.assert_array_equal(got, oracle.conv2d_i8(x, w, b, activation=cb.ACTIVATION_RELU, **kw))
+    scale = g.uniform(1e-4, 1e-3, K).astype(np.float32)
+    got = h.conv_forward("requant", x, w, ys, "i8", y_dtype="i8", bias=b, bias_dtype="i32", scale=scale, activation=cb.ACTIVATION_LINEAR, **kw)
+    np.testing.assert_array_equal(got, oracle.requant_i8(oracle.conv2d_i8(x, w, b, **kw), scale))
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_implicit_gemm_full_epilogue(oracle, dtype):
     """alpha1, alpha2, beta, bias, residual and every activation, in the order of the reference's epilogue
