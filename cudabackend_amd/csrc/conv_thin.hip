@@ -29,7 +29,7 @@ namespace
 	using namespace avhip;
 
 	constexpr int THIN_FILTERS = 64; /* filters per block */
-	constexpr int THIN_LDS = 80 * 1024; /* two workgroups per compute unit */
+	constexpr int THIN_LDS = 64 * 1024; /* most a workgroup may ask for; it asks for what the layer needs, and two to four fit a compute unit */
 	constexpr int THIN_MAX_K_BYTES = 1024;
 	constexpr int THIN_MAX_PIXEL_BYTES = 64;
 	constexpr unsigned int THIN_NO_PIECE = 0xFFFFFFFFu; /* table entry of a piece past the end of k */
@@ -47,6 +47,7 @@ namespace
 		unsigned int w_pitch; /* LDS pitch of a padded filter row: an odd number of 16-byte units */
 		unsigned int x_bytes, w_bytes;
 		unsigned int filter_blocks;
+		int wide_halo; /* the halo is brought in as 16-byte pieces of image rows that start on 16-byte boundaries */
 	};
 
 	/* A piece of PB bytes: its register type, its load from a tensor (zeros at OUT_OF_RANGE) */
@@ -99,13 +100,13 @@ namespace
 	};
 
 	template<typename TE, int PB, typename Epi>
-	__global__ __launch_bounds__(256, 2) void k_conv_thin(const TE *__restrict__ x, const TE *__restrict__ w, ThinGeom g, Epi epi)
+	__global__ __launch_bounds__(256, 3) void k_conv_thin(const TE *__restrict__ x, const TE *__restrict__ w, ThinGeom g, Epi epi)
 	{
 		epi.pin();
 		constexpr int NP = 16 / PB;
 		constexpr int W = Epi::wide;
 		typedef typename ThinPiece<PB>::type piece_t;
-		__shared__ __attribute__((aligned(16))) char lds[THIN_LDS];
+		extern __shared__ __attribute__((aligned(16))) char lds[];
 		const int tid = threadIdx.x;
 		const int lane = tid & 63;
 		const int wave = tid >> 6;
@@ -120,6 +121,121 @@ namespace
 		unsigned int *table = reinterpret_cast<unsigned int*>(lds + g.halo_bytes);
 		const unsigned int zero_at = g.halo_bytes + g.table_bytes; /* 16 bytes of zeros: what a piece past the end of k reads */
 		char *filters = lds + zero_at + 16;
+
+		/* Filter rows f0 .. f0 + 63 lie back to back in w: read as aligned 16-byte chunks (the first FILTER_AHEAD per work-item
+		 * ahead of time, into registers), written to the padded rows piece by piece (a chunk may run over the end of a row). */
+		const __amdgpu_buffer_rsrc_t rw = make_buffer(w, g.w_bytes);
+		constexpr int FILTER_AHEAD = 6;
+		ThinChunk<PB> ahead[FILTER_AHEAD];
+		auto fetch_chunk_of = [&](unsigned int w_first, unsigned int total, unsigned int off, ThinChunk<PB> &chunk) __attribute__((always_inline))
+		{
+			chunk.u = buffer_fetch(rw, off + 16 <= total ? w_first + off : OUT_OF_RANGE);
+			if (off < total && off + 16 > total) /* the one chunk that runs over the end of w */
+			{
+#pragma unroll
+				for (int e = 0; e < NP; e++)
+					chunk.piece[e] = ThinPiece<PB>::get(rw, off + e * PB < total ? w_first + off + e * PB : OUT_OF_RANGE);
+			}
+		};
+		auto scatter_chunk = [&](unsigned int total, unsigned int off, const ThinChunk<PB> &chunk) __attribute__((always_inline))
+		{
+			if (off < total)
+			{
+				unsigned int row = off / g.k_bytes, column = off - row * g.k_bytes;
+#pragma unroll
+				for (int e = 0; e < NP; e++)
+				{
+					if (off + e * PB < total)
+						*reinterpret_cast<piece_t*>(filters + row * g.w_pitch + column) = chunk.piece[e];
+					column += PB;
+					if (column >= g.k_bytes)
+					{
+						column = 0;
+						row++;
+					}
+				}
+			}
+		};
+		auto block_bytes = [&](int f0)
+		{
+			return static_cast<unsigned int>(g.K - f0 < THIN_FILTERS ? g.K - f0 : THIN_FILTERS) * g.k_bytes;
+		};
+		auto clear_tails = [&]() __attribute__((always_inline))
+		{
+			const unsigned int tail_pieces = (g.kgroups * 32 - g.k_bytes) / PB;
+			for (unsigned int idx = tid; idx < THIN_FILTERS * tail_pieces; idx += 256)
+			{
+				piece_t nothing = {};
+				*reinterpret_cast<piece_t*>(filters + (idx & (THIN_FILTERS - 1)) * g.w_pitch + g.k_bytes + (idx / THIN_FILTERS) * PB) = nothing;
+			}
+		};
+		/* chunks `first_chunk`, `first_chunk` + 256, ... of this work-item: fetched and written one after the other */
+		auto stage_filters = [&](int f0, unsigned int first_chunk) __attribute__((always_inline))
+		{
+			const unsigned int total = block_bytes(f0), w_first = static_cast<unsigned int>(f0) * g.k_bytes;
+			for (unsigned int off = (first_chunk + tid) * 16; off < total; off += 256 * 16)
+			{
+				ThinChunk<PB> chunk;
+				fetch_chunk_of(w_first, total, off, chunk);
+				scatter_chunk(total, off, chunk);
+			}
+		};
+
+		/* The halo: the image rows under the tile, in pieces of SB bytes; consecutive work-items read consecutive pieces of a
+		 * row.  SB = 16 where every image row starts on a 16-byte boundary: the halo then starts at the boundary at or before its
+		 * first pixel (`lead` bytes earlier), and a piece lies inside an image row or outside as a whole. */
+		const int column_base = (ow0 * g.stride_w + g.pad_w) * static_cast<int>(g.pixel_bytes); /* byte column of the halo's first pixel */
+		const unsigned int lead = g.wide_halo ? static_cast<unsigned int>(column_base & 15) : 0u;
+		auto stage_halo = [&](auto piece_bytes, auto &&between) __attribute__((always_inline))
+		{
+			constexpr int SB = decltype(piece_bytes)::value;
+			typedef typename ThinPiece<SB>::type stage_t;
+			const __amdgpu_buffer_rsrc_t rx = make_buffer(x, g.x_bytes);
+			const int ih_base = oh0 * g.stride_h + g.pad_h;
+			const int column0 = column_base - static_cast<int>(lead);
+			const int row_bytes = g.W * static_cast<int>(g.pixel_bytes);
+			unsigned int row = tid / g.pieces_per_row, piece = tid - row * g.pieces_per_row;
+			constexpr int BATCH = SB == 16 ? 4 : 8;
+			for (unsigned int first = 0; first < g.halo_pieces; first += 256 * BATCH)
+			{
+				stage_t value[BATCH];
+#pragma unroll
+				for (int u = 0; u < BATCH; u++)
+				{
+					const unsigned int q = first + u * 256 + tid;
+					const int ih = ih_base + static_cast<int>(row);
+					const int column = column0 + static_cast<int>(piece) * SB;
+					const bool inside = (q < g.halo_pieces) & (ih >= 0) & (ih < g.H) & (column >= 0) & (column < row_bytes);
+					value[u] = ThinPiece<SB>::get(rx, inside ? static_cast<unsigned int>((static_cast<int>(n) * g.H + ih) * row_bytes + column) : OUT_OF_RANGE);
+					row += g.step_rows;
+					piece += g.step_pieces;
+					if (piece >= g.pieces_per_row)
+					{
+						piece -= g.pieces_per_row;
+						row++;
+					}
+				}
+				if (first == 0)
+					between(); /* the first filters are asked for before anybody waits for the halo */
+#pragma unroll
+				for (int u = 0; u < BATCH; u++)
+				{
+					const unsigned int q = first + u * 256 + tid;
+					if (q < g.halo_pieces)
+						*reinterpret_cast<stage_t*>(lds + q * SB) = value[u];
+				}
+			}
+		};
+		auto first_filters = [&]() __attribute__((always_inline))
+		{
+#pragma unroll
+			for (int u = 0; u < FILTER_AHEAD; u++)
+				fetch_chunk_of(0u, block_bytes(0), (u * 256 + tid) * 16, ahead[u]);
+		};
+		if (PB < 16 && g.wide_halo)
+			stage_halo(std::integral_constant<int, 16>(), first_filters);
+		else
+			stage_halo(std::integral_constant<int, PB>(), first_filters);
 
 		/* the table: entry (slab, half, piece) = offset of that piece of k from the window origin of a pixel */
 		for (unsigned int idx = tid; idx < g.kgroups * 2 * NP; idx += 256)
@@ -142,43 +258,6 @@ namespace
 		if (tid < 4)
 			reinterpret_cast<unsigned int*>(lds + zero_at)[tid] = 0u;
 
-		/* the halo, piece by piece: consecutive work-items read consecutive pieces of an image row */
-		{
-			const __amdgpu_buffer_rsrc_t rx = make_buffer(x, g.x_bytes);
-			const int ih_base = oh0 * g.stride_h + g.pad_h;
-			const int column_base = (ow0 * g.stride_w + g.pad_w) * static_cast<int>(g.pixel_bytes); /* byte column of the halo's first pixel */
-			const int row_bytes = g.W * static_cast<int>(g.pixel_bytes);
-			unsigned int row = tid / g.pieces_per_row, piece = tid - row * g.pieces_per_row;
-			constexpr int BATCH = 8;
-			for (unsigned int first = 0; first < g.halo_pieces; first += 256 * BATCH)
-			{
-				piece_t value[BATCH];
-#pragma unroll
-				for (int u = 0; u < BATCH; u++)
-				{
-					const unsigned int q = first + u * 256 + tid;
-					const int ih = ih_base + static_cast<int>(row);
-					const int column = column_base + static_cast<int>(piece) * PB;
-					const bool inside = (q < g.halo_pieces) & (ih >= 0) & (ih < g.H) & (column >= 0) & (column < row_bytes);
-					value[u] = ThinPiece<PB>::get(rx, inside ? static_cast<unsigned int>((static_cast<int>(n) * g.H + ih) * row_bytes + column) : OUT_OF_RANGE);
-					row += g.step_rows;
-					piece += g.step_pieces;
-					if (piece >= g.pieces_per_row)
-					{
-						piece -= g.pieces_per_row;
-						row++;
-					}
-				}
-#pragma unroll
-				for (int u = 0; u < BATCH; u++)
-				{
-					const unsigned int q = first + u * 256 + tid;
-					if (q < g.halo_pieces)
-						*reinterpret_cast<piece_t*>(lds + q * PB) = value[u];
-				}
-			}
-		}
-
 		/* window origin of this lane's two output pixels (pixel m of the tile is row m >> tw_shift, column m & (TW - 1)) */
 		unsigned int origin[2];
 #pragma unroll
@@ -186,54 +265,27 @@ namespace
 		{
 			const int m = wave * 64 + tm * 32 + (lane & 31);
 			origin[tm] = static_cast<unsigned int>((m >> g.tw_shift) * g.stride_h) * g.halo_pitch
-					+ static_cast<unsigned int>((m & (TW - 1)) * g.stride_w) * g.pixel_bytes;
+					+ static_cast<unsigned int>((m & (TW - 1)) * g.stride_w) * g.pixel_bytes + lead;
 		}
 
-		const __amdgpu_buffer_rsrc_t rw = make_buffer(w, g.w_bytes);
+		/* the first block of filters: what was fetched ahead, then the rest */
+		clear_tails();
+#pragma unroll
+		for (int u = 0; u < FILTER_AHEAD; u++)
+			scatter_chunk(block_bytes(0), (u * 256 + tid) * 16, ahead[u]);
+		stage_filters(0, FILTER_AHEAD * 256);
+
 		for (unsigned int fb = 0; fb < g.filter_blocks; fb++)
 		{
 			const int f0 = static_cast<int>(fb) * THIN_FILTERS;
 			const int kcol = f0 + drain_column<1, W>();
 			typename Epi::template ColumnsT<W> columns;
 			epi.load_columns(kcol, columns);
-			__syncthreads(); /* the accumulators of the previous block have left the filter region */
-
-			/* filter rows f0 .. f0 + 63 lie back to back in w: read as aligned 16-byte chunks, written to the padded rows piece
-			 * by piece (a chunk may run over the end of a filter row) */
+			if (fb > 0)
 			{
-				const unsigned int rows = static_cast<unsigned int>(g.K - f0 < THIN_FILTERS ? g.K - f0 : THIN_FILTERS);
-				const unsigned int total = rows * g.k_bytes, w_first = static_cast<unsigned int>(f0) * g.k_bytes;
-				const unsigned int tail_pieces = (g.kgroups * 32 - g.k_bytes) / PB;
-				for (unsigned int idx = tid; idx < THIN_FILTERS * tail_pieces; idx += 256)
-				{
-					piece_t nothing = {};
-					*reinterpret_cast<piece_t*>(filters + (idx & (THIN_FILTERS - 1)) * g.w_pitch + g.k_bytes + (idx / THIN_FILTERS) * PB) = nothing;
-				}
-				for (unsigned int off = tid * 16; off < total; off += 256 * 16)
-				{
-					ThinChunk<PB> chunk;
-					if (off + 16 <= total)
-						chunk.u = buffer_fetch(rw, w_first + off);
-					else
-					{
-#pragma unroll
-						for (int e = 0; e < NP; e++)
-							chunk.piece[e] = ThinPiece<PB>::get(rw, off + e * PB < total ? w_first + off + e * PB : OUT_OF_RANGE);
-					}
-					unsigned int row = off / g.k_bytes, column = off - row * g.k_bytes;
-#pragma unroll
-					for (int e = 0; e < NP; e++)
-					{
-						if (off + e * PB < total)
-							*reinterpret_cast<piece_t*>(filters + row * g.w_pitch + column) = chunk.piece[e];
-						column += PB;
-						if (column >= g.k_bytes)
-						{
-							column = 0;
-							row++;
-						}
-					}
-				}
+				__syncthreads(); /* the accumulators of the previous block have left the filter region */
+				clear_tails();
+				stage_filters(f0, 0u);
 			}
 			__syncthreads();
 
@@ -247,12 +299,21 @@ namespace
 						acc[i][j][v] = 0;
 			const char *filter_row = filters + (lane & 31) * g.w_pitch + half * 16;
 			const unsigned int *table_row = table + half * NP;
-			auto slab = [&](unsigned int kg, auto last) __attribute__((always_inline))
+			/* One slab: the table entries of the next slab are asked for before this slab's pieces (an LDS read that depends on
+			 * an LDS read would otherwise pay the latency twice); only the last slab has pieces past the end of k (`checked`).
+			 * Operands are not read a slab ahead: 2-byte pieces occupy a register each until they are packed, and two slabs of
+			 * them in flight do not fit the registers of three wavefronts per SIMD, which hide the latency instead. */
+			unsigned int rel[NP], rel_next[NP];
+			auto entries = [&](unsigned int kg, unsigned int (&r)[NP]) __attribute__((always_inline))
 			{
-				unsigned int rel[NP];
 #pragma unroll
 				for (int e = 0; e < NP; e++)
-					rel[e] = table_row[kg * 2 * NP + e];
+					r[e] = table_row[kg * 2 * NP + e];
+			};
+			auto slab = [&](unsigned int kg, auto checked) __attribute__((always_inline))
+			{
+				if (!decltype(checked)::value)
+					entries(kg + 1, rel_next);
 				Chunk a[2], b[2];
 #pragma unroll
 				for (int tm = 0; tm < 2; tm++)
@@ -262,7 +323,7 @@ namespace
 					for (int e = 0; e < NP; e++)
 					{
 						unsigned int at = origin[tm] + rel[e];
-						if (decltype(last)::value) /* only the last slab has pieces past the end of k */
+						if (decltype(checked)::value)
 							at = rel[e] == THIN_NO_PIECE ? zero_at : at;
 						chunk.piece[e] = *reinterpret_cast<const piece_t*>(lds + at);
 					}
@@ -276,13 +337,22 @@ namespace
 #pragma unroll
 					for (int tn = 0; tn < 2; tn++)
 						Mma<TE>::run(a[tm], b[tn], acc[tm][tn]);
+#pragma unroll
+				for (int e = 0; e < NP; e++)
+					rel[e] = rel_next[e];
 			};
-			for (unsigned int kg = 0; kg + 1 < g.kgroups; kg++)
+			const unsigned int last = g.kgroups - 1;
+			entries(0, rel);
+			for (unsigned int kg = 0; kg < last; kg++)
 				slab(kg, std::false_type());
-			slab(g.kgroups - 1, std::true_type());
+			slab(last, std::true_type());
 
-			drain_tile_private<TE, 2, W>(filters, acc, [&](int row, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
+			drain_tile_private<TE, 2, W>(filters, acc, [&](int tile_row, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
 			{
+				/* worked out here and now: hoisted out of the loop over filter blocks, the addresses of all rows would sit in
+				 * registers throughout the multiplication */
+				int row = tile_row;
+				asm volatile("" : "+v"(row));
 				const int oh = oh0 + (row >> g.tw_shift), ow = ow0 + (row & (TW - 1));
 				if (oh < g.Ho && ow < g.Wo && kcol < g.K)
 					epi.template store_at<ACT_SIMPLE, true, W>((static_cast<int64_t>(static_cast<int>(n) * g.Ho + oh) * g.Wo + ow) * g.K + kcol, kcol, v, columns,
@@ -336,15 +406,28 @@ namespace avhip
 		g.table_bytes = round_up(g.kgroups * 2 * (16 / pb) * 4, 16);
 		const unsigned int drain_bytes = 4 * PrivateDrainRows<2, Epi::wide>::bytes;
 		const unsigned int fixed_bytes = g.table_bytes + 16 + std::max<unsigned int>(THIN_FILTERS * g.w_pitch, drain_bytes);
+		/* image rows that start on 16-byte boundaries are brought in as 16-byte pieces, from the boundary at or before the first
+		 * pixel of the halo: up to 16 - pb bytes more per row */
+		g.wide_halo = (pb < 16 && (static_cast<int64_t>(s.W) * pixel_bytes) % 16 == 0 && aligned_to(x, 16)) ? 1 : 0;
+		const int stage_bytes = g.wide_halo ? 16 : pb;
+		auto halo_of = [&](int shift, unsigned int &rows, unsigned int &pitch)
+		{
+			const int tw = 1 << shift, th = 256 >> shift;
+			const int64_t r = static_cast<int64_t>(th - 1) * s.stride_h + static_cast<int64_t>(s.R - 1) * s.dil_h + 1;
+			const int64_t c = static_cast<int64_t>(tw - 1) * s.stride_w + static_cast<int64_t>(s.S - 1) * s.dil_w + 1;
+			const int64_t p = g.wide_halo ? (c * pixel_bytes + 16 - pb + 15) / 16 * 16 : c * pixel_bytes;
+			rows = static_cast<unsigned int>(std::min<int64_t>(r, 1 << 20));
+			pitch = static_cast<unsigned int>(std::min<int64_t>(p, 1 << 20));
+			return r * p;
+		};
 		/* the tile shape: as few tiles as possible, then the smallest halo */
 		int best_shift = -1;
 		int64_t best_tiles = 0, best_halo = 0;
 		for (int shift = 0; shift <= 8; shift++)
 		{
 			const int tw = 1 << shift, th = 256 >> shift;
-			const int64_t halo_rows = static_cast<int64_t>(th - 1) * s.stride_h + static_cast<int64_t>(s.R - 1) * s.dil_h + 1;
-			const int64_t halo_columns = static_cast<int64_t>(tw - 1) * s.stride_w + static_cast<int64_t>(s.S - 1) * s.dil_w + 1;
-			const int64_t halo = halo_rows * halo_columns * pixel_bytes;
+			unsigned int rows, pitch;
+			const int64_t halo = halo_of(shift, rows, pitch);
 			if (halo + 16 + fixed_bytes > THIN_LDS)
 				continue;
 			const int64_t tiles = static_cast<int64_t>((s.Ho + th - 1) / th) * ((s.Wo + tw - 1) / tw);
@@ -362,7 +445,7 @@ namespace avhip
 			return false;
 		if (best_tiles * s.N >= (1ll << 31))
 			return false;
-		const int tw = 1 << best_shift, th = 256 >> best_shift;
+		const int tw = 1 << best_shift;
 		g.H = s.H;
 		g.W = s.W;
 		g.K = s.K;
@@ -382,10 +465,9 @@ namespace avhip
 		g.tiles_per_image = static_cast<unsigned int>(best_tiles);
 		g.pixel_bytes = static_cast<unsigned int>(pixel_bytes);
 		g.k_bytes = static_cast<unsigned int>(k_bytes);
-		const unsigned int halo_rows = static_cast<unsigned int>((th - 1) * s.stride_h + (s.R - 1) * s.dil_h + 1);
-		const unsigned int halo_columns = static_cast<unsigned int>((tw - 1) * s.stride_w + (s.S - 1) * s.dil_w + 1);
-		g.halo_pitch = halo_columns * g.pixel_bytes;
-		g.pieces_per_row = g.halo_pitch / pb;
+		unsigned int halo_rows;
+		halo_of(best_shift, halo_rows, g.halo_pitch);
+		g.pieces_per_row = g.halo_pitch / stage_bytes;
 		g.halo_pieces = halo_rows * g.pieces_per_row;
 		g.step_rows = 256 / g.pieces_per_row;
 		g.step_pieces = 256 % g.pieces_per_row;
@@ -394,7 +476,8 @@ namespace avhip
 		g.w_bytes = static_cast<unsigned int>(w_bytes);
 		g.filter_blocks = static_cast<unsigned int>((s.K + THIN_FILTERS - 1) / THIN_FILTERS);
 		const dim3 grid(static_cast<unsigned int>(best_tiles * s.N));
-#define AVHIP_THIN(PB) hipLaunchKernelGGL((k_conv_thin<TE, PB, Epi>), grid, dim3(256), 0, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi)
+		const unsigned int lds_bytes = g.halo_bytes + fixed_bytes;
+#define AVHIP_THIN(PB) hipLaunchKernelGGL((k_conv_thin<TE, PB, Epi>), grid, dim3(256), lds_bytes, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi)
 		switch (pb)
 		{
 			case 16:

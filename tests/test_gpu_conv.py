@@ -126,7 +126,7 @@ def test_int8_few_input_channels_bit_exact(oracle, case):
 
 # ---- few input channels, images large enough for 256-pixel tiles: the kernel that gathers its operand from a tile in LDS ------
 THIN_CASES = [
-    dict(x=(2, 40, 44, 3), w=(72, 7, 7, 3), pad=(-3, -3), stride=(2, 2)),                         # a residual network's first layer; the second filter block partial
+    dict(x=(2, 40, 48, 3), w=(72, 7, 7, 3), pad=(-3, -3), stride=(2, 2)),                         # a residual network's first layer; the second filter block partial
     dict(x=(2, 33, 35, 3), w=(64, 5, 5, 3), pad=(-2, -2), mode=1),                                # flipped; partial tiles at both edges
     dict(x=(1, 50, 20, 1), w=(16, 9, 9, 1), pad=(-4, -4)),                                        # 81 taps of one plane
     dict(x=(2, 24, 40, 6), w=(32, 3, 5, 6), pad=(-2, -4), dilation=(2, 2)),                       # dilated
