@@ -21,15 +21,30 @@
  */
 #include "conv_thin.hpp"
 #include "mfma_core.hpp"
+#include "persistent_gemm.hpp"
 #include <algorithm>
 #include <type_traits>
+
+/* Instrumentation, compiled in with -DCONV_THIN_STAMPS only: work-item 0 of every workgroup records the 100 MHz wall clock at
+ * the phase boundaries of the kernel (start, requests out, halo in LDS, filters in LDS, first slab, last slab, accumulators
+ * gone), and avhip_debug_thin_stamps() copies the records of the last launch to the host. */
+#ifdef CONV_THIN_STAMPS
+__device__ unsigned long long g_thin_stamps[4096 * 8];
+#define THIN_STAMP(i) do { if (threadIdx.x == 0) g_thin_stamps[(blockIdx.x % 4096) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+extern "C" __attribute__((visibility("default"))) int avhip_debug_thin_stamps(void *out)
+{
+	return static_cast<int>(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_thin_stamps), sizeof(g_thin_stamps)));
+}
+#else
+#define THIN_STAMP(i) do { } while (0)
+#endif
 
 namespace
 {
 	using namespace avhip;
 
 	constexpr int THIN_FILTERS = 64; /* filters per block */
-	constexpr int THIN_LDS = 64 * 1024; /* most a workgroup may ask for; it asks for what the layer needs, and two to four fit a compute unit */
+	constexpr int THIN_LDS = 80 * 1024; /* most a workgroup may ask for (two per compute unit); it asks for what the layer needs */
 	constexpr int THIN_MAX_K_BYTES = 1024;
 	constexpr int THIN_MAX_PIXEL_BYTES = 64;
 	constexpr unsigned int THIN_NO_PIECE = 0xFFFFFFFFu; /* table entry of a piece past the end of k */
@@ -39,7 +54,7 @@ namespace
 		int H, W, K, Ho, Wo, R, S;
 		int pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, flip;
 		int tw_shift; /* the tile is (256 >> tw_shift) rows of (1 << tw_shift) output pixels */
-		unsigned int tiles_x, tiles_per_image;
+		unsigned int tiles_x, tiles_per_image, tiles, items; /* tiles: of all images; items: (filter block, tile) pairs */
 		unsigned int pixel_bytes, k_bytes, kgroups; /* kgroups: 32-byte slabs of k, the last one padded */
 		unsigned int halo_pitch, halo_pieces, pieces_per_row; /* halo row = pieces_per_row pieces = halo_pitch bytes, rows back to back */
 		unsigned int step_rows, step_pieces; /* 256 pieces further on: this many rows and pieces down the halo */
@@ -47,6 +62,7 @@ namespace
 		unsigned int w_pitch; /* LDS pitch of a padded filter row: an odd number of 16-byte units */
 		unsigned int x_bytes, w_bytes;
 		unsigned int filter_blocks;
+		int narrow_rows; /* a tile's part of y spans less than 2 GiB: 32-bit offsets from its first pixel */
 		int wide_halo; /* the halo is brought in as 16-byte pieces of image rows that start on 16-byte boundaries */
 	};
 
@@ -100,7 +116,7 @@ namespace
 	};
 
 	template<typename TE, int PB, typename Epi>
-	__global__ __launch_bounds__(256, 3) void k_conv_thin(const TE *__restrict__ x, const TE *__restrict__ w, ThinGeom g, Epi epi)
+	__global__ __launch_bounds__(256, 2) void k_conv_thin(const TE *__restrict__ x, const TE *__restrict__ w, ThinGeom g, Epi epi)
 	{
 		epi.pin();
 		constexpr int NP = 16 / PB;
@@ -111,36 +127,64 @@ namespace
 		const int lane = tid & 63;
 		const int wave = tid >> 6;
 		const int half = lane >> 5; /* which 16 bytes of a 32-byte slab this lane supplies */
-
-		const unsigned int n = blockIdx.x / g.tiles_per_image;
-		const unsigned int in_image = blockIdx.x - n * g.tiles_per_image;
-		const unsigned int tile_y = in_image / g.tiles_x, tile_x = in_image - tile_y * g.tiles_x;
-		const int TW = 1 << g.tw_shift;
-		const int oh0 = static_cast<int>(tile_y) * (256 >> g.tw_shift), ow0 = static_cast<int>(tile_x) * TW;
+		THIN_STAMP(0);
 
 		unsigned int *table = reinterpret_cast<unsigned int*>(lds + g.halo_bytes);
 		const unsigned int zero_at = g.halo_bytes + g.table_bytes; /* 16 bytes of zeros: what a piece past the end of k reads */
 		char *filters = lds + zero_at + 16;
-
-		/* Filter rows f0 .. f0 + 63 lie back to back in w: read as aligned 16-byte chunks (the first FILTER_AHEAD per work-item
-		 * ahead of time, into registers), written to the padded rows piece by piece (a chunk may run over the end of a row). */
+		char *drain = filters + THIN_FILTERS * g.w_pitch;
+		const int TW = 1 << g.tw_shift;
+		const __amdgpu_buffer_rsrc_t rx = make_buffer(x, g.x_bytes);
 		const __amdgpu_buffer_rsrc_t rw = make_buffer(w, g.w_bytes);
-		constexpr int FILTER_AHEAD = 6;
-		ThinChunk<PB> ahead[FILTER_AHEAD];
-		auto fetch_chunk_of = [&](unsigned int w_first, unsigned int total, unsigned int off, ThinChunk<PB> &chunk) __attribute__((always_inline))
+
+		/* A workgroup walks the work items (filter block, image, tile) from its own number in steps of the grid: the filters stay
+		 * in LDS while the filter block stays the same, which is nearly always. */
+		struct Item
 		{
-			chunk.u = buffer_fetch(rw, off + 16 <= total ? w_first + off : OUT_OF_RANGE);
-			if (off < total && off + 16 > total) /* the one chunk that runs over the end of w */
-			{
-#pragma unroll
-				for (int e = 0; e < NP; e++)
-					chunk.piece[e] = ThinPiece<PB>::get(rw, off + e * PB < total ? w_first + off + e * PB : OUT_OF_RANGE);
-			}
+			unsigned int fb, n;
+			int oh0, ow0; /* first output pixel of the tile */
+			int ih_base, column0; /* image row and byte column of the halo's first piece */
+			unsigned int lead; /* bytes between the halo's first piece and its first pixel */
 		};
-		auto scatter_chunk = [&](unsigned int total, unsigned int off, const ThinChunk<PB> &chunk) __attribute__((always_inline))
+		auto locate = [&](unsigned int item) __attribute__((always_inline))
 		{
-			if (off < total)
+			Item it;
+			it.fb = item / g.tiles;
+			const unsigned int t = item - it.fb * g.tiles;
+			it.n = t / g.tiles_per_image;
+			const unsigned int in_image = t - it.n * g.tiles_per_image;
+			const unsigned int tile_y = in_image / g.tiles_x, tile_x = in_image - tile_y * g.tiles_x;
+			it.oh0 = static_cast<int>(tile_y) * (256 >> g.tw_shift);
+			it.ow0 = static_cast<int>(tile_x) * TW;
+			const int column_base = (it.ow0 * g.stride_w + g.pad_w) * static_cast<int>(g.pixel_bytes);
+			it.lead = g.wide_halo ? static_cast<unsigned int>(column_base & 15) : 0u;
+			it.column0 = column_base - static_cast<int>(it.lead);
+			it.ih_base = it.oh0 * g.stride_h + g.pad_h;
+			return it;
+		};
+
+		/* Filter rows f0 .. f0 + 63 lie back to back in w: read as aligned 16-byte chunks, written to the padded rows of LDS
+		 * piece by piece (a chunk may run over the end of a filter row). */
+		auto stage_filters = [&](int f0) __attribute__((always_inline))
+		{
+			const unsigned int total = static_cast<unsigned int>(g.K - f0 < THIN_FILTERS ? g.K - f0 : THIN_FILTERS) * g.k_bytes;
+			const unsigned int w_first = static_cast<unsigned int>(f0) * g.k_bytes;
+			const unsigned int tail_pieces = (g.kgroups * 32 - g.k_bytes) / PB;
+			for (unsigned int idx = tid; idx < THIN_FILTERS * tail_pieces; idx += 256)
 			{
+				piece_t nothing = {};
+				*reinterpret_cast<piece_t*>(filters + (idx & (THIN_FILTERS - 1)) * g.w_pitch + g.k_bytes + (idx / THIN_FILTERS) * PB) = nothing;
+			}
+			for (unsigned int off = tid * 16; off < total; off += 256 * 16)
+			{
+				ThinChunk<PB> chunk;
+				chunk.u = buffer_fetch(rw, off + 16 <= total ? w_first + off : OUT_OF_RANGE);
+				if (off + 16 > total) /* the one chunk that runs over the end of w */
+				{
+#pragma unroll
+					for (int e = 0; e < NP; e++)
+						chunk.piece[e] = ThinPiece<PB>::get(rw, off + e * PB < total ? w_first + off + e * PB : OUT_OF_RANGE);
+				}
 				unsigned int row = off / g.k_bytes, column = off - row * g.k_bytes;
 #pragma unroll
 				for (int e = 0; e < NP; e++)
@@ -156,87 +200,92 @@ namespace
 				}
 			}
 		};
-		auto block_bytes = [&](int f0)
-		{
-			return static_cast<unsigned int>(g.K - f0 < THIN_FILTERS ? g.K - f0 : THIN_FILTERS) * g.k_bytes;
-		};
-		auto clear_tails = [&]() __attribute__((always_inline))
-		{
-			const unsigned int tail_pieces = (g.kgroups * 32 - g.k_bytes) / PB;
-			for (unsigned int idx = tid; idx < THIN_FILTERS * tail_pieces; idx += 256)
-			{
-				piece_t nothing = {};
-				*reinterpret_cast<piece_t*>(filters + (idx & (THIN_FILTERS - 1)) * g.w_pitch + g.k_bytes + (idx / THIN_FILTERS) * PB) = nothing;
-			}
-		};
-		/* chunks `first_chunk`, `first_chunk` + 256, ... of this work-item: fetched and written one after the other */
-		auto stage_filters = [&](int f0, unsigned int first_chunk) __attribute__((always_inline))
-		{
-			const unsigned int total = block_bytes(f0), w_first = static_cast<unsigned int>(f0) * g.k_bytes;
-			for (unsigned int off = (first_chunk + tid) * 16; off < total; off += 256 * 16)
-			{
-				ThinChunk<PB> chunk;
-				fetch_chunk_of(w_first, total, off, chunk);
-				scatter_chunk(total, off, chunk);
-			}
-		};
 
 		/* The halo: the image rows under the tile, in pieces of SB bytes; consecutive work-items read consecutive pieces of a
 		 * row.  SB = 16 where every image row starts on a 16-byte boundary: the halo then starts at the boundary at or before its
-		 * first pixel (`lead` bytes earlier), and a piece lies inside an image row or outside as a whole. */
-		const int column_base = (ow0 * g.stride_w + g.pad_w) * static_cast<int>(g.pixel_bytes); /* byte column of the halo's first pixel */
-		const unsigned int lead = g.wide_halo ? static_cast<unsigned int>(column_base & 15) : 0u;
-		auto stage_halo = [&](auto piece_bytes, auto &&between) __attribute__((always_inline))
+		 * first pixel (`lead` bytes earlier), and a piece lies inside an image row or outside as a whole.  The first pieces of a
+		 * work-item are requested early (`request`) and written to LDS later (`commit`, which also moves the rest). */
+		const unsigned int first_row = tid / g.pieces_per_row, first_piece = tid - first_row * g.pieces_per_row;
+		const int row_bytes = g.W * static_cast<int>(g.pixel_bytes);
+		struct Walk
 		{
-			constexpr int SB = decltype(piece_bytes)::value;
-			typedef typename ThinPiece<SB>::type stage_t;
-			const __amdgpu_buffer_rsrc_t rx = make_buffer(x, g.x_bytes);
-			const int ih_base = oh0 * g.stride_h + g.pad_h;
-			const int column0 = column_base - static_cast<int>(lead);
-			const int row_bytes = g.W * static_cast<int>(g.pixel_bytes);
-			unsigned int row = tid / g.pieces_per_row, piece = tid - row * g.pieces_per_row;
-			constexpr int BATCH = SB == 16 ? 4 : 8;
-			for (unsigned int first = 0; first < g.halo_pieces; first += 256 * BATCH)
+			unsigned int row, piece;
+		};
+		auto fetch_batch = [&](const Item &it, unsigned int first, Walk &at, auto &value) __attribute__((always_inline))
+		{
+			typedef typename std::remove_reference<decltype(value[0])>::type stage_t;
+			constexpr int SB = sizeof(stage_t);
+			constexpr int BATCH = sizeof(value) / SB;
+#pragma unroll
+			for (int u = 0; u < BATCH; u++)
 			{
-				stage_t value[BATCH];
-#pragma unroll
-				for (int u = 0; u < BATCH; u++)
+				const unsigned int q = first + u * 256 + tid;
+				const int ih = it.ih_base + static_cast<int>(at.row);
+				const int column = it.column0 + static_cast<int>(at.piece) * SB;
+				const bool inside = (q < g.halo_pieces) & (ih >= 0) & (ih < g.H) & (column >= 0) & (column < row_bytes);
+				value[u] = ThinPiece<SB>::get(rx, inside ? static_cast<unsigned int>((static_cast<int>(it.n) * g.H + ih) * row_bytes + column) : OUT_OF_RANGE);
+				at.row += g.step_rows;
+				at.piece += g.step_pieces;
+				if (at.piece >= g.pieces_per_row)
 				{
-					const unsigned int q = first + u * 256 + tid;
-					const int ih = ih_base + static_cast<int>(row);
-					const int column = column0 + static_cast<int>(piece) * SB;
-					const bool inside = (q < g.halo_pieces) & (ih >= 0) & (ih < g.H) & (column >= 0) & (column < row_bytes);
-					value[u] = ThinPiece<SB>::get(rx, inside ? static_cast<unsigned int>((static_cast<int>(n) * g.H + ih) * row_bytes + column) : OUT_OF_RANGE);
-					row += g.step_rows;
-					piece += g.step_pieces;
-					if (piece >= g.pieces_per_row)
-					{
-						piece -= g.pieces_per_row;
-						row++;
-					}
-				}
-				if (first == 0)
-					between(); /* the first filters are asked for before anybody waits for the halo */
-#pragma unroll
-				for (int u = 0; u < BATCH; u++)
-				{
-					const unsigned int q = first + u * 256 + tid;
-					if (q < g.halo_pieces)
-						*reinterpret_cast<stage_t*>(lds + q * SB) = value[u];
+					at.piece -= g.pieces_per_row;
+					at.row++;
 				}
 			}
 		};
-		auto first_filters = [&]() __attribute__((always_inline))
+		auto store_batch = [&](unsigned int first, const auto &value) __attribute__((always_inline))
 		{
+			typedef typename std::remove_const<typename std::remove_reference<decltype(value[0])>::type>::type stage_t;
+			constexpr int SB = sizeof(stage_t);
+			constexpr int BATCH = sizeof(value) / SB;
 #pragma unroll
-			for (int u = 0; u < FILTER_AHEAD; u++)
-				fetch_chunk_of(0u, block_bytes(0), (u * 256 + tid) * 16, ahead[u]);
+			for (int u = 0; u < BATCH; u++)
+			{
+				const unsigned int q = first + u * 256 + tid;
+				if (q < g.halo_pieces)
+					*reinterpret_cast<stage_t*>(lds + q * SB) = value[u];
+			}
 		};
-		if (PB < 16 && g.wide_halo)
-			stage_halo(std::integral_constant<int, 16>(), first_filters);
-		else
-			stage_halo(std::integral_constant<int, PB>(), first_filters);
+		constexpr int NARROW_BATCH = PB == 16 ? 4 : 8;
+		u32x4_t wide_value[4];
+		piece_t narrow_value[NARROW_BATCH];
+		Walk walk;
+		const bool wide = PB < 16 && g.wide_halo != 0;
+		auto request = [&](const Item &it) __attribute__((always_inline))
+		{
+			walk.row = first_row;
+			walk.piece = first_piece;
+			if (wide)
+				fetch_batch(it, 0u, walk, wide_value);
+			else
+				fetch_batch(it, 0u, walk, narrow_value);
+		};
+		auto commit = [&](const Item &it) __attribute__((always_inline))
+		{
+			if (wide)
+			{
+				store_batch(0u, wide_value);
+				for (unsigned int first = 256 * 4; first < g.halo_pieces; first += 256 * 4)
+				{
+					fetch_batch(it, first, walk, wide_value);
+					store_batch(first, wide_value);
+				}
+			}
+			else
+			{
+				store_batch(0u, narrow_value);
+				for (unsigned int first = 256 * NARROW_BATCH; first < g.halo_pieces; first += 256 * NARROW_BATCH)
+				{
+					fetch_batch(it, first, walk, narrow_value);
+					store_batch(first, narrow_value);
+				}
+			}
+		};
 
+		unsigned int item = blockIdx.x;
+		Item cur = locate(item);
+		request(cur);
+		THIN_STAMP(1);
 		/* the table: entry (slab, half, piece) = offset of that piece of k from the window origin of a pixel */
 		for (unsigned int idx = tid; idx < g.kgroups * 2 * NP; idx += 256)
 		{
@@ -257,37 +306,31 @@ namespace
 		}
 		if (tid < 4)
 			reinterpret_cast<unsigned int*>(lds + zero_at)[tid] = 0u;
+		stage_filters(static_cast<int>(cur.fb) * THIN_FILTERS);
+		commit(cur);
+		THIN_STAMP(2);
+		__syncthreads();
 
 		/* window origin of this lane's two output pixels (pixel m of the tile is row m >> tw_shift, column m & (TW - 1)) */
-		unsigned int origin[2];
+		unsigned int pixel_at[2];
 #pragma unroll
 		for (int tm = 0; tm < 2; tm++)
 		{
 			const int m = wave * 64 + tm * 32 + (lane & 31);
-			origin[tm] = static_cast<unsigned int>((m >> g.tw_shift) * g.stride_h) * g.halo_pitch
-					+ static_cast<unsigned int>((m & (TW - 1)) * g.stride_w) * g.pixel_bytes + lead;
+			pixel_at[tm] = static_cast<unsigned int>((m >> g.tw_shift) * g.stride_h) * g.halo_pitch
+					+ static_cast<unsigned int>((m & (TW - 1)) * g.stride_w) * g.pixel_bytes;
 		}
+		const char *filter_row = filters + (lane & 31) * g.w_pitch + half * 16;
+		const unsigned int *table_row = table + half * NP;
 
-		/* the first block of filters: what was fetched ahead, then the rest */
-		clear_tails();
-#pragma unroll
-		for (int u = 0; u < FILTER_AHEAD; u++)
-			scatter_chunk(block_bytes(0), (u * 256 + tid) * 16, ahead[u]);
-		stage_filters(0, FILTER_AHEAD * 256);
-
-		for (unsigned int fb = 0; fb < g.filter_blocks; fb++)
+		for (;;)
 		{
-			const int f0 = static_cast<int>(fb) * THIN_FILTERS;
+			THIN_STAMP(3);
+			const int f0 = static_cast<int>(cur.fb) * THIN_FILTERS;
 			const int kcol = f0 + drain_column<1, W>();
 			typename Epi::template ColumnsT<W> columns;
 			epi.load_columns(kcol, columns);
-			if (fb > 0)
-			{
-				__syncthreads(); /* the accumulators of the previous block have left the filter region */
-				clear_tails();
-				stage_filters(f0, 0u);
-			}
-			__syncthreads();
+			const unsigned int origin[2] = { pixel_at[0] + cur.lead, pixel_at[1] + cur.lead };
 
 			typename Mma<TE>::acc_t acc[2][2];
 #pragma unroll
@@ -297,12 +340,10 @@ namespace
 #pragma unroll
 					for (int v = 0; v < 16; v++)
 						acc[i][j][v] = 0;
-			const char *filter_row = filters + (lane & 31) * g.w_pitch + half * 16;
-			const unsigned int *table_row = table + half * NP;
 			/* One slab: the table entries of the next slab are asked for before this slab's pieces (an LDS read that depends on
 			 * an LDS read would otherwise pay the latency twice); only the last slab has pieces past the end of k (`checked`).
 			 * Operands are not read a slab ahead: 2-byte pieces occupy a register each until they are packed, and two slabs of
-			 * them in flight do not fit the registers of three wavefronts per SIMD, which hide the latency instead. */
+			 * them in flight take more registers than two workgroups per compute unit leave; the other wavefronts hide the latency. */
 			unsigned int rel[NP], rel_next[NP];
 			auto entries = [&](unsigned int kg, unsigned int (&r)[NP]) __attribute__((always_inline))
 			{
@@ -346,18 +387,67 @@ namespace
 			for (unsigned int kg = 0; kg < last; kg++)
 				slab(kg, std::false_type());
 			slab(last, std::true_type());
+			THIN_STAMP(4);
 
-			drain_tile_private<TE, 2, W>(filters, acc, [&](int tile_row, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
+			/* the next item's halo is asked for now and arrives while the accumulators leave */
+			const unsigned int next_item = item + gridDim.x;
+			const bool more = next_item < g.items;
+			const Item next = locate(more ? next_item : item);
+			if (more)
+				request(next);
+
+			const int oh0 = cur.oh0, ow0 = cur.ow0;
+			const unsigned int n = cur.n;
+			/* (the hand-over starts with a barrier: every wavefront is done with the halo and the filters) */
+			bool gone = false;
+			if constexpr (std::is_same<Epi, FloatEpilogue<TE>>::value && sizeof(TE) == 2)
 			{
-				/* worked out here and now: hoisted out of the loop over filter blocks, the addresses of all rows would sit in
-				 * registers throughout the multiplication */
-				int row = tile_row;
-				asm volatile("" : "+v"(row));
+				/* the usual first layer (16-bit tensors, no residual, beta = 0): no branch in the epilogue, a buffer over the tile's
+				 * part of y, rows outside the image at an out-of-range offset, runs written through as they go */
+				if (epi.z == nullptr && epi.beta == 0.0f && g.narrow_rows)
+				{
+					constexpr unsigned int SZ = sizeof(TE);
+					const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + (static_cast<int64_t>(static_cast<int>(n) * g.Ho + oh0) * g.Wo + ow0) * g.K, 0x7FFFFFF0u);
+					const int rows_left = g.Ho - oh0, columns_left = g.Wo - ow0;
+					auto leave = [&](auto relu) __attribute__((always_inline))
+					{
+						drain_tile_private<TE, 2, W>(drain, acc, [&](int row, const float (&v)[W], int) __attribute__((always_inline))
+						{
+							const int ty = row >> g.tw_shift, tx = row & (TW - 1);
+							const unsigned int offset = (ty < rows_left && tx < columns_left && kcol < g.K) ?
+									static_cast<unsigned int>((ty * g.Wo + tx) * g.K + kcol) * SZ : OUT_OF_RANGE;
+							typename Epi::template Residual<W> none;
+							epi.template store_fast<decltype(relu)::value, false, W>(v, columns, none, [&](auto words) __attribute__((always_inline))
+							{
+								buffer_put<STORE_STREAM_THROUGH>(ry, offset, words);
+							});
+						});
+					};
+					if (epi.activation == ACT_RELU)
+						leave(std::true_type());
+					else
+						leave(std::false_type());
+					gone = true;
+				}
+			}
+			if (!gone)
+				drain_tile_private<TE, 2, W>(drain, acc, [&](int row, const typename Epi::scalar_t (&v)[W], int) __attribute__((always_inline))
+			{
 				const int oh = oh0 + (row >> g.tw_shift), ow = ow0 + (row & (TW - 1));
 				if (oh < g.Ho && ow < g.Wo && kcol < g.K)
 					epi.template store_at<ACT_SIMPLE, true, W>((static_cast<int64_t>(static_cast<int>(n) * g.Ho + oh) * g.Wo + ow) * g.K + kcol, kcol, v, columns,
 							nullptr);
 			});
+			THIN_STAMP(5);
+			if (!more)
+				break;
+			commit(next);
+			if (next.fb != cur.fb)
+				stage_filters(static_cast<int>(next.fb) * THIN_FILTERS);
+			THIN_STAMP(6);
+			__syncthreads();
+			cur = next;
+			item = next_item;
 		}
 	}
 
@@ -405,7 +495,7 @@ namespace avhip
 		g.w_pitch = g.kgroups * 32 + 16;
 		g.table_bytes = round_up(g.kgroups * 2 * (16 / pb) * 4, 16);
 		const unsigned int drain_bytes = 4 * PrivateDrainRows<2, Epi::wide>::bytes;
-		const unsigned int fixed_bytes = g.table_bytes + 16 + std::max<unsigned int>(THIN_FILTERS * g.w_pitch, drain_bytes);
+		const unsigned int fixed_bytes = g.table_bytes + 16 + THIN_FILTERS * g.w_pitch + drain_bytes;
 		/* image rows that start on 16-byte boundaries are brought in as 16-byte pieces, from the boundary at or before the first
 		 * pixel of the halo: up to 16 - pb bytes more per row */
 		g.wide_halo = (pb < 16 && (static_cast<int64_t>(s.W) * pixel_bytes) % 16 == 0 && aligned_to(x, 16)) ? 1 : 0;
@@ -443,7 +533,7 @@ namespace avhip
 		/* images much smaller than a tile leave most of the MFMA rows empty */
 		if (static_cast<int64_t>(s.Ho) * s.Wo * 10 < best_tiles * 256 * 3)
 			return false;
-		if (best_tiles * s.N >= (1ll << 31))
+		if (best_tiles * s.N * ((s.K + THIN_FILTERS - 1) / THIN_FILTERS) >= (1ll << 31))
 			return false;
 		const int tw = 1 << best_shift;
 		g.H = s.H;
@@ -475,9 +565,16 @@ namespace avhip
 		g.x_bytes = static_cast<unsigned int>(x_bytes);
 		g.w_bytes = static_cast<unsigned int>(w_bytes);
 		g.filter_blocks = static_cast<unsigned int>((s.K + THIN_FILTERS - 1) / THIN_FILTERS);
-		const dim3 grid(static_cast<unsigned int>(best_tiles * s.N));
+		g.narrow_rows = (256ll * s.Wo * s.K * static_cast<int64_t>(sizeof(TE)) < (1ll << 31)) ? 1 : 0;
+		g.tiles = static_cast<unsigned int>(best_tiles * s.N);
+		g.items = g.tiles * g.filter_blocks;
 		const unsigned int lds_bytes = g.halo_bytes + fixed_bytes;
-#define AVHIP_THIN(PB) hipLaunchKernelGGL((k_conv_thin<TE, PB, Epi>), grid, dim3(256), lds_bytes, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi)
+		/* the workgroups that stay resident (two per compute unit: registers and LDS) share the work items */
+		const dim3 grid(std::min(g.items, persistent_workgroups(1 << 30)));
+#define AVHIP_THIN(PB) \
+		if (lds_bytes > 64u * 1024u) \
+			(void)hipFuncSetAttribute(reinterpret_cast<const void*>(&k_conv_thin<TE, PB, Epi>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)); \
+		hipLaunchKernelGGL((k_conv_thin<TE, PB, Epi>), grid, dim3(256), lds_bytes, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi)
 		switch (pb)
 		{
 			case 16:

@@ -153,6 +153,8 @@ def test_thin_kernel_with_residual(oracle, dtype, case):
     assert oracle.rel_l2(got, want) < BAR[dtype]
     # every image separately: a tile that went to the wrong place would hide in a global norm
     assert max(oracle.rel_l2(got[i], want[i]) for i in range(ys[0])) < 2 * BAR[dtype]
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, bias=b, activation=cb.ACTIVATION_RELU, **kw)
+    assert oracle.rel_l2(got, oracle.conv2d(x, w, b, activation=oracle.RELU, **kw)) < BAR[dtype]
     a2, be = float(np.float32(0.7)), float(np.float32(0.3))
     got = h.conv_forward("implicit_gemm", x, w, ys, dtype, bias=b, z=z, y0=y0, alpha2=a2, beta=be, activation=cb.ACTIVATION_RELU, **kw)
     want = oracle.conv2d(x, w, b, z, y0, alpha2=a2, beta=be, activation=oracle.RELU, **kw)
