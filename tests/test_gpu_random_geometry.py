@@ -136,3 +136,51 @@ def test_random_wide_images_and_large_filters(oracle, dtype):
                 want = oracle.conv2d(x[n:n + 1], w, b, z[n:n + 1], activation=oracle.RELU, pad=pad, mode=mode)
                 err = oracle.rel_l2(got[n:n + 1], want)
                 assert err < 2e-3, "case %d: N=%d %dx%d C=%d K=%d %dx%d pad=%r mode=%d image %d: rel-L2 %.3e" % (done, N, H, W, Cin, K, R, S, pad, mode, n, err)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32", "i8"])
+def test_random_few_channel_layers(oracle, dtype):
+    """First-layer shapes: 1 to 12 input planes, filters up to 9 x 9, strides, dilations, both modes, images large enough for
+    the kernel that gathers its operand from an image tile in LDS (piece sizes 1 to 16 bytes, with and without 16-byte image
+    rows, one to three filter blocks, several tiles per image).  Sampled images against the oracle; int8 -> int32 bit-exact."""
+    g = h.rng({"bf16": 61, "f32": 62, "i8": 63}[dtype])
+    bar = {"bf16": 2e-3, "f32": 1e-5}
+    done = 0
+    while done < 30:
+        R, S = int(g.integers(1, 10)), int(g.integers(1, 10))
+        Cin = int(g.integers(1, 13))
+        elem = {"bf16": 2, "f32": 4, "i8": 1}[dtype]
+        if R * S == 1 or R * S * Cin * elem > 1024:
+            continue
+        stride = (int(g.integers(1, 4)), int(g.integers(1, 4)))
+        dilation = (int(g.integers(1, 3)), int(g.integers(1, 3)))
+        N, H, W = int(g.integers(1, 6)), int(g.integers(16, 70)), int(g.integers(16, 70))
+        if g.integers(0, 2) == 1:
+            W = (W + 7) // 8 * 8  # image rows of whole 16-byte pieces
+        K = int(g.choice([8, 24, 64, 72, 136]))
+        pad = (-int(g.integers(0, (R - 1) * dilation[0] + 1)), -int(g.integers(0, (S - 1) * dilation[1] + 1)))
+        mode = int(g.integers(0, 2))
+        Ho, Wo = oracle.conv_output_shape(H, W, R, S, pad, stride, dilation)
+        if Ho < 1 or Wo < 1 or Ho * Wo < 100:
+            continue
+        done += 1
+        kw = dict(pad=pad, stride=stride, dilation=dilation, mode=mode)
+        what = "case %d: N=%d %dx%d C=%d K=%d %dx%d %r" % (done, N, H, W, Cin, K, R, S, kw)
+        images = sorted(set(int(i) for i in g.integers(0, N, 2)))
+        if dtype == "i8":
+            x = g.integers(-127, 128, (N, H, W, Cin), dtype=np.int8)
+            w = g.integers(-127, 128, (K, R, S, Cin), dtype=np.int8)
+            b = g.integers(-2 ** 15, 2 ** 15, K).astype(np.int32)
+            got = h.conv_forward("implicit_gemm", x, w, (N, Ho, Wo, K), "i8", y_dtype="i32", bias=b, bias_dtype="i32", activation=cb.ACTIVATION_RELU, **kw)
+            for n in images:
+                want = oracle.conv2d_i8(x[n:n + 1], w, b, activation=cb.ACTIVATION_RELU, **kw)
+                assert np.array_equal(got[n:n + 1], want), what + " image %d" % n
+        else:
+            x = h.rounded(oracle, g.standard_normal((N, H, W, Cin)), dtype)
+            w = h.rounded(oracle, g.standard_normal((K, R, S, Cin)) * np.sqrt(2.0 / (R * S * Cin)), dtype)
+            b = g.uniform(-0.1, 0.1, K).astype(np.float32).astype(np.float64)
+            got = h.conv_forward("implicit_gemm", x, w, (N, Ho, Wo, K), dtype, bias=b, activation=cb.ACTIVATION_RELU, **kw)
+            for n in images:
+                want = oracle.conv2d(x[n:n + 1], w, b, activation=oracle.RELU, **kw)
+                err = oracle.rel_l2(got[n:n + 1], want)
+                assert err < bar[dtype], what + " image %d: rel-L2 %.3e" % (n, err)
