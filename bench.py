@@ -427,16 +427,22 @@ def mfma_rates(hip, ctx):
     return out
 
 
-def other_configs(hip, ctx, iters):
-    """BASELINE configs 1, 3 and 5 through the dispatcher (bias + ReLU fused), one timing each."""
+BASELINE_LAYERS = [("cfg1_f32_3x3_15x15_64", "f32", (8, 15, 15, 64), (64, 3, 3, 64), -1, 1),
+                   ("cfg3_bf16_3x3_56x56_256", "bf16", (64, 56, 56, 256), (256, 3, 3, 256), -1, 1),
+                   ("cfg3_f16_3x3_56x56_256", "f16", (64, 56, 56, 256), (256, 3, 3, 256), -1, 1),
+                   ("cfg5_bf16_3x3_stride2_128_256", "bf16", (64, 56, 56, 128), (256, 3, 3, 128), -1, 2),
+                   ("cfg5_bf16_1x1_256_512", "bf16", (64, 28, 28, 256), (512, 1, 1, 256), 0, 1),
+                   ("cfg5_bf16_5x5_64_64", "bf16", (64, 32, 32, 64), (64, 5, 5, 64), -2, 1)]
+# not BASELINE configs: first layers over image planes, the shapes of the thin-channel kernel
+FIRST_LAYERS = [("bf16_7x7_stride2_3_64_224x224_N32", "bf16", (32, 224, 224, 3), (64, 7, 7, 3), -3, 2),
+                ("bf16_5x5_3_32_128x128_N32", "bf16", (32, 128, 128, 3), (32, 5, 5, 3), -2, 1),
+                ("f32_3x3_3_64_64x64_N64", "f32", (64, 64, 64, 3), (64, 3, 3, 3), -1, 1)]
+
+
+def other_configs(hip, ctx, iters, cases=BASELINE_LAYERS):
+    """Single layers through the dispatcher (bias + ReLU fused), one timing each: BASELINE configs 1, 3 and 5 by default."""
     lib = cb.load_library()
     g = np.random.default_rng(SEED + 7)
-    cases = [("cfg1_f32_3x3_15x15_64", "f32", (8, 15, 15, 64), (64, 3, 3, 64), -1, 1),
-             ("cfg3_bf16_3x3_56x56_256", "bf16", (64, 56, 56, 256), (256, 3, 3, 256), -1, 1),
-             ("cfg3_f16_3x3_56x56_256", "f16", (64, 56, 56, 256), (256, 3, 3, 256), -1, 1),
-             ("cfg5_bf16_3x3_stride2_128_256", "bf16", (64, 56, 56, 128), (256, 3, 3, 128), -1, 2),
-             ("cfg5_bf16_1x1_256_512", "bf16", (64, 28, 28, 256), (512, 1, 1, 256), 0, 1),
-             ("cfg5_bf16_5x5_64_64", "bf16", (64, 32, 32, 64), (64, 5, 5, 64), -2, 1)]
     out = {}
     for name, dtype, xs, ws, pad, stride in cases:
         d = DT[dtype]
@@ -600,6 +606,7 @@ def main():
         detail["stream_GBs_measured"] = stream_rates(hip, ctx)
         detail["mfma_rate_measured"] = mfma_rates(hip, ctx)
         detail["other_configs"] = other_configs(hip, ctx, it)
+        detail["first_layers_beyond_baseline"] = other_configs(hip, ctx, it, FIRST_LAYERS)
         cpu = None if args.no_cpu else cpu_baseline()
     ctx.close()
     peak = PEAK[args.dtype]
