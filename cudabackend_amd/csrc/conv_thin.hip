@@ -10,14 +10,16 @@
  * tile that a workgroup's 256 output pixels read is brought into LDS once, with neighbouring work-items reading neighbouring
  * addresses, and the pieces are gathered from LDS, which serves 32 scattered work-items per cycle.
  *
- * One workgroup = one tile of TH x TW = 256 output pixels of one image (TW a power of two, chosen per layer) times all the
- * filters, 64 at a time.  In LDS:
+ * A work item is one tile of TH x TW = 256 output pixels of one image (TW a power of two, chosen per layer) times one block
+ * of 64 filters; the resident workgroups (two per compute unit) walk the items in steps of the grid.  In LDS:
  *   the halo: the (TH-1)*stride + (R-1)*dilation + 1 image rows under the tile, zeros where the image ends;
  *   a table with, for every piece of k, its byte offset from the window origin of a pixel (the same for every pixel);
- *   the 64 filters of the current block, rows padded with zeros to whole 32-byte MFMA slabs; the accumulators leave through
- *   the same bytes afterwards.
+ *   the 64 filters of the current block, rows padded with zeros to whole 32-byte MFMA slabs (staged when the block changes,
+ *   which for a workgroup is nearly never);
+ *   the region through which the accumulators leave.
  * A wavefront owns 64 pixels (two MFMA tiles) by 64 filters; per 32-byte slab of k it gathers two operand chunks from the
- * halo, reads two filter chunks and issues four MFMAs.  No barrier inside the k loop.
+ * halo, reads two filter chunks and issues four MFMAs.  No barrier inside the k loop.  The next item's halo is requested
+ * before the accumulators leave and written once every wavefront is done with the current one.
  */
 #include "conv_thin.hpp"
 #include "mfma_core.hpp"
@@ -26,8 +28,9 @@
 #include <type_traits>
 
 /* Instrumentation, compiled in with -DCONV_THIN_STAMPS only: work-item 0 of every workgroup records the 100 MHz wall clock at
- * the phase boundaries of the kernel (start, requests out, halo in LDS, filters in LDS, first slab, last slab, accumulators
- * gone), and avhip_debug_thin_stamps() copies the records of the last launch to the host. */
+ * the phase boundaries of the kernel (start, first requests out, set-up done, and for its last item: first slab, last slab,
+ * accumulators gone; next halo in LDS for the item before), and avhip_debug_thin_stamps() copies the records of the last
+ * launch to the host. */
 #ifdef CONV_THIN_STAMPS
 __device__ unsigned long long g_thin_stamps[4096 * 8];
 #define THIN_STAMP(i) do { if (threadIdx.x == 0) g_thin_stamps[(blockIdx.x % 4096) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
