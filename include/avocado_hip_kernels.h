@@ -122,7 +122,9 @@ extern "C"
 
 	/* Tuning knob without a counterpart in the reference.  The implicit-GEMM launcher sends a convolution to the kernel with
 	 * one 32 x 32 tile per wavefront when its 128 x 128 tiling would yield fewer than this many workgroups (default 192 on
-	 * the 256 compute units of an MI355X; 0 never uses that kernel).  Returns the previous value.  Process-wide. */
+	 * the 256 compute units of an MI355X) and its k extent is short enough for that kernel to be the faster one by the
+	 * launcher's estimate; 0 never uses that kernel; a negative value uses it for everything it can run (tests).  Returns the
+	 * previous value.  Process-wide. */
 	AVHIP_API int avhip_set_small_problem_threshold(int workgroups);
 
 	/* Tuning knob without a counterpart in the reference.  Products with a short k (at most 512 bytes per operand row: 1x1

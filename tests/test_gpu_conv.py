@@ -14,12 +14,12 @@ BAR = {"f32": 1e-5, "f16": 2e-3, "bf16": 2e-3}
 
 @pytest.fixture(autouse=True, params=["wavefront_tiles", "workgroup_tiles"])
 def tiling(request):
-    """The shapes of this file are tiny, so the launcher would send all of them to the kernel with one 32 x 32 tile per
-    wavefront.  Every test therefore runs twice: as launched by default, and with that kernel switched off so that the
-    same geometry goes through the 128 x 128 gather kernel, the image-tile kernel or the packed-k kernel."""
+    """Every test runs twice: with the kernel that gives each wavefront one 32 x 32 tile forced for whatever it can run
+    (the launcher itself picks it for problems small in tiles and short in k), and with that kernel switched off, so that
+    the same geometry goes through the 128 x 128 gather kernel, the image-tile kernel or the few-channel kernels."""
     lib = cb.load_library()
     lib.avhip_set_small_problem_threshold.restype = int
-    previous = lib.avhip_set_small_problem_threshold(192 if request.param == "wavefront_tiles" else 0)
+    previous = lib.avhip_set_small_problem_threshold(-1 if request.param == "wavefront_tiles" else 0)
     yield request.param
     lib.avhip_set_small_problem_threshold(previous)
 

@@ -37,7 +37,7 @@ def output_shape(orc, c):
 def test_random_geometries_floating(oracle, dtype, tiling):
     lib = cb.load_library()
     lib.avhip_set_small_problem_threshold.restype = int
-    previous = lib.avhip_set_small_problem_threshold(192 if tiling == "wavefront_tiles" else 0)
+    previous = lib.avhip_set_small_problem_threshold(-1 if tiling == "wavefront_tiles" else 0)
     try:
         g = h.rng(50 + ["f32", "f16", "bf16"].index(dtype))
         done = 0
@@ -73,7 +73,7 @@ def test_random_geometries_floating(oracle, dtype, tiling):
 def test_random_geometries_int8(oracle, tiling):
     lib = cb.load_library()
     lib.avhip_set_small_problem_threshold.restype = int
-    previous = lib.avhip_set_small_problem_threshold(192 if tiling == "wavefront_tiles" else 0)
+    previous = lib.avhip_set_small_problem_threshold(-1 if tiling == "wavefront_tiles" else 0)
     try:
         g = h.rng(53)
         done = 0
