@@ -88,7 +88,7 @@ PROTOTYPES = {
 # the thin kernel layer of include/avocado_hip_kernels.h (exported, bound only for the symbol check)
 KERNEL_LAYER_SYMBOLS = ["avhip_winograd_weight_transform", "avhip_winograd_input_transform", "avhip_winograd_output_transform",
                         "avhip_winograd_gradient_transform", "avhip_winograd_update_transform", "avhip_gemm_batched",
-                        "avhip_conv2d_implicit_gemm", "avhip_conv2d_winograd_fused", "avhip_add_bias", "avhip_im2row", "avhip_change_type",
+                        "avhip_conv2d_implicit_gemm", "avhip_conv2d_implicit_gemm_split_k", "avhip_conv2d_split_k_workspace", "avhip_conv2d_winograd_fused", "avhip_add_bias", "avhip_im2row", "avhip_change_type",
                         "avhip_set_memory", "avhip_mfma_rate_probe", "avhip_set_small_problem_threshold", "avhip_set_short_k_engine",
                         "avhip_affine_forward", "avhip_batchnorm_inference", "avhip_stream_probe"]
 

@@ -15,6 +15,7 @@
  */
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstring>
@@ -794,6 +795,29 @@ namespace
 		touch(yMem);
 		const int rc = avhip_conv2d_implicit_gemm(c.ctx.stream, p.x_dtype, p.y_dtype, c.bias_dtype, &p.shape, c.x->data, c.w->data, c.bias, c.z, c.y->data,
 				padding_value_or_null(p.conv), c.alpha1, c.alpha2, c.beta, activation, requant_scale);
+		return from_launcher(rc);
+	}
+	/* Layers with few output pixels and a long k: the k range split across workgroups, partial sums in the caller's
+	 * workspace.  NOT_SUPPORTED (nothing launched) when the layer is not of that kind or the workspace does not take it. */
+	int64_t split_k_bytes(const ConvProblem &p)
+	{
+		int64_t bytes = 0;
+		if (p.y_dtype != p.x_dtype || avhip_conv2d_split_k_workspace(p.x_dtype, &p.shape, &bytes) != 0)
+			return 0;
+		return bytes;
+	}
+	avStatus_t run_split_k(const ConvCall &c, Memory *ws, avMemoryDescriptor_t workspaceMem, avMemoryDescriptor_t yMem, avActivationType_t activation)
+	{
+		const ConvProblem &p = c.problem;
+		const int64_t bytes = split_k_bytes(p);
+		if (bytes == 0 || ws == nullptr || ws->data == nullptr || ws->size < bytes || (c.bias != nullptr && c.bias_dtype != AVOCADO_DTYPE_FLOAT32))
+			return AVOCADO_STATUS_NOT_SUPPORTED;
+		const int rc = avhip_conv2d_implicit_gemm_split_k(c.ctx.stream, p.x_dtype, &p.shape, c.x->data, c.w->data, c.bias, c.z, c.y->data,
+				padding_value_or_null(p.conv), c.alpha1, c.alpha2, c.beta, activation, ws->data, ws->size);
+		if (rc == AVHIP_NOT_SUPPORTED)
+			return AVOCADO_STATUS_NOT_SUPPORTED;
+		touch(workspaceMem, 0, bytes);
+		touch(yMem);
 		return from_launcher(rc);
 	}
 	bool fused_winograd_applicable(const ConvProblem &p)
@@ -1803,6 +1827,8 @@ namespace avocado
 				return st;
 			NonFusedPlan plan;
 			result[0] = (nonfused_plan(p, plan) && (nonfused_preferred(p, plan) || !fused_winograd_applicable(p))) ? plan.total : 0;
+			/* what the split-k plan of the implicit GEMM would take, for layers that go there */
+			result[0] = std::max<av_int64>(result[0], split_k_bytes(p));
 			return AVOCADO_STATUS_SUCCESS;
 		}
 
@@ -1857,6 +1883,9 @@ namespace avocado
 				if (ns != AVOCADO_STATUS_BAD_ALLOC)
 					return ns;
 			}
+			const avStatus_t ss = run_split_k(call, ws, workspaceMem, yMem, activation);
+			if (ss != AVOCADO_STATUS_NOT_SUPPORTED)
+				return ss;
 			return run_implicit_gemm(call, yMem, activation, nullptr);
 		}
 

@@ -17,6 +17,7 @@
  *   int8 requantised : y = sat_i8(rne(float(sum + bias) * scale[k])), each step a single fp32 rounding;
  *   int8 with float scalars: the header's convention (cast to fp32, scale, cast back with rounding and saturation).
  */
+#include <algorithm>
 #include <cstring>
 
 #include "conv_epilogue.hpp"
@@ -45,6 +46,14 @@ namespace
 	struct TapCursor
 	{
 		int i = 0, j = 0, slice = 0, tap = 0;
+		/* to k-step `step` of the walk */
+		__device__ inline void seek(const ConvGeom &g, int step)
+		{
+			tap = step / g.steps_per_tap;
+			slice = step - tap * g.steps_per_tap;
+			i = tap / g.S;
+			j = tap - i * g.S;
+		}
 		__device__ inline void advance(const ConvGeom &g)
 		{
 			if (++slice == g.steps_per_tap)
@@ -192,6 +201,11 @@ namespace
 			cur.advance(g);
 			set_tap();
 		}
+		__device__ inline void seek(int step)
+		{
+			cur.seek(g, step);
+			set_tap();
+		}
 	};
 
 	/* Rows of B are output filters; a chunk is 16 bytes of channels of w[k, i, j, :]. */
@@ -258,6 +272,10 @@ namespace
 		__device__ inline void next()
 		{
 			cur.advance(g);
+		}
+		__device__ inline void seek(int step)
+		{
+			cur.seek(g, step);
 		}
 	};
 
@@ -465,6 +483,74 @@ namespace
 		});
 	}
 
+	/*
+	 * Split k: for layers with few output pixels and a long k (the last stages of a deep network at a small batch) the
+	 * 128 x 128 tiling yields a few dozen workgroups, each walking thousands of k elements alone.  Here blockIdx.z takes an
+	 * even number of k-steps of the walk and stores the raw fp32 sums of its part to partial[z][pixel][filter]; k_split_reduce
+	 * adds the parts and applies the epilogue.  Branch-free loaders only (aligned chunks, zero padding value).
+	 */
+	template<typename TE>
+	__global__ __launch_bounds__(256, 2) void k_conv_igemm_split(const TE *__restrict__ x, const TE *__restrict__ w, ConvGeom g, int steps_per_split,
+			float *__restrict__ partial)
+	{
+		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
+		unsigned int pixel_block, filter_block;
+		xcd_tile(pixel_block, filter_block);
+		const int64_t p0 = static_cast<int64_t>(pixel_block) * BLOCK_M;
+		const int k = filter_block * BLOCK_N + drain_column<2>();
+		const int total = g.R * g.S * g.steps_per_tap, first = static_cast<int>(blockIdx.z) * steps_per_split;
+		const int steps = total - first < steps_per_split ? total - first : steps_per_split;
+
+		const TE no_padding_value = TE();
+		PixelLoader<TE, true> la(x, g, no_padding_value, true, p0);
+		FilterLoader<TE, true> lb(w, g, true, filter_block * BLOCK_N);
+		la.seek(first);
+		lb.seek(first);
+		typename Mma<TE>::acc_t acc[2][2];
+		block_mma<TE>(lds, steps, la, lb, acc);
+
+		float *part = partial + static_cast<int64_t>(blockIdx.z) * g.pixels * g.K;
+		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const float (&v)[4], int) __attribute__((always_inline))
+		{
+			const int64_t p = p0 + r;
+			if (p < g.pixels && k < g.K)
+			{
+				typedef float f32x4 __attribute__((ext_vector_type(4)));
+				const f32x4 sums = { v[0], v[1], v[2], v[3] };
+				*reinterpret_cast<f32x4*>(part + p * g.K + k) = sums;
+			}
+		});
+	}
+	/* y = epilogue(sum over the parts), four filters of a pixel per work-item */
+	template<typename TE>
+	__global__ __launch_bounds__(256) void k_split_reduce(const float *__restrict__ partial, int splits, int64_t plane, FloatEpilogue<TE> epi)
+	{
+		const int64_t e = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+		if (e >= plane)
+			return;
+		typedef float f32x4 __attribute__((ext_vector_type(4)));
+		/* four parts at a time, so that their loads are in flight together; the sum runs in the order of the parts either way */
+		f32x4 sum = *reinterpret_cast<const f32x4*>(partial + e);
+		int z = 1;
+		for (; z + 4 <= splits; z += 4)
+		{
+			f32x4 part[4];
+#pragma unroll
+			for (int u = 0; u < 4; u++)
+				part[u] = *reinterpret_cast<const f32x4*>(partial + (z + u) * plane + e);
+#pragma unroll
+			for (int u = 0; u < 4; u++)
+				sum += part[u];
+		}
+		for (; z < splits; z++)
+			sum += *reinterpret_cast<const f32x4*>(partial + z * plane + e);
+		const int k = static_cast<int>(e % epi.K);
+		typename FloatEpilogue<TE>::Columns columns;
+		epi.load_columns(k, columns);
+		const float v[4] = { sum[0], sum[1], sum[2], sum[3] };
+		epi.template store_at<ACT_ANY, false, 4>(e, k, v, columns);
+	}
+
 	template<typename TE>
 	ConvGeom make_geom(const avhipConvShape &s)
 	{
@@ -654,5 +740,126 @@ extern "C" int avhip_conv2d_implicit_gemm(void *stream, int x_dtype, int y_dtype
 		}
 		default:
 			return AVHIP_UNSUPPORTED_DATATYPE;
+	}
+}
+
+namespace
+{
+	/* Whether to split k, into how many parts of how many steps, and the workspace that takes: worth it when the plain tiling
+	 * leaves most compute units idle for a long walk.  Estimates in microseconds (fitted to layers of 196 to 6272 pixels with
+	 * 1024 to 4608 elements of k): 4 + 0.7 per k-step for a workgroup of the plain gather kernel (less in the image-tile kernel); for the split, 10 for the two
+	 * launches and their prologues, 0.7 per step of a part, 0.25 per part and the parts read back at 4 TB/s in the reduction;
+	 * the one-wavefront-per-tile kernel by its own estimate where the launcher would use it. */
+	struct SplitPlan
+	{
+		int splits, steps_per_split;
+		int64_t bytes;
+	};
+	template<typename TE>
+	bool split_k_plan(const avhipConvShape &s, SplitPlan &plan)
+	{
+		constexpr int KE = STEP_BYTES / sizeof(TE);
+		const int64_t pixels = static_cast<int64_t>(s.N) * s.Ho * s.Wo;
+		const int64_t tiles = ((pixels + BLOCK_M - 1) / BLOCK_M) * ((static_cast<int64_t>(s.K) + BLOCK_N - 1) / BLOCK_N);
+		const int64_t steps = static_cast<int64_t>(s.R) * s.S * ((s.C + KE - 1) / KE);
+		/* the branch-free loaders: whole 16-byte chunks of channels, one mask bit per tap */
+		if (tiles >= 256 || steps < 8 || steps > (1 << 20) || (s.C * sizeof(TE)) % 16 != 0 || s.R * s.S > 32)
+			return false;
+		int64_t parts = std::min<int64_t>(512 / tiles, steps / 4);
+		if (parts < 2)
+			return false;
+		const int64_t per_part = ((steps + parts - 1) / parts + 1) / 2 * 2; /* even: the engine runs its steps in pairs */
+		parts = (steps + per_part - 1) / per_part;
+		if (parts < 2 || parts > 65535)
+			return false;
+		const double plane_bytes = static_cast<double>(pixels) * s.K * 4.0;
+		double other = 4.0 + 0.7 * static_cast<double>(steps);
+		if (s.stride_h == 1 && s.stride_w == 1 && s.dil_h == 1 && s.dil_w == 1 && s.R * s.S > 1 && s.Ho * s.Wo >= 128)
+		{
+			/* the image-tile kernel takes such layers: 0.47 us per step for a workgroup with a compute unit to itself, 0.68 us
+			 * when two share one, 3.6 us around the loop */
+			const int64_t workgroups = static_cast<int64_t>(s.N) * ((s.K + 63) / 64) * ((s.Ho * s.Wo + 255) / 256);
+			other = 3.6 + (workgroups <= 256 ? 0.47 : 0.68) * static_cast<double>(steps);
+		}
+		if (s.R * s.S <= 32 && conv_small_preferred(s, static_cast<int>(sizeof(TE)), tiles))
+			other = std::min(other, conv_small_estimate(s, static_cast<int>(sizeof(TE)), tiles).small_us);
+		const double split = 10.0 + 0.7 * static_cast<double>(per_part) + 0.25 * static_cast<double>(parts)
+				+ plane_bytes * static_cast<double>(parts + 1) / 4.0e6;
+		if (split > 0.85 * other)
+			return false;
+		plan.splits = static_cast<int>(parts);
+		plan.steps_per_split = static_cast<int>(per_part);
+		plan.bytes = static_cast<int64_t>(plane_bytes) * parts;
+		return true;
+	}
+	template<typename TE>
+	int launch_split(hipStream_t st, const avhipConvShape &s, const void *x, const void *w, const void *bias, const void *z, void *y, const void *padding_value,
+			double alpha1, double alpha2, double beta, int activation, void *workspace, int64_t workspace_bytes)
+	{
+		SplitPlan plan;
+		const int flags = vector_flags<TE>(s, x, w, y, z, sizeof(TE));
+		if (!split_k_plan<TE>(s, plan) || !fast_path_ok<TE>(s, flags, padding_value) || (flags & 2) == 0 || workspace == nullptr
+				|| workspace_bytes < plan.bytes || !aligned_to(workspace, 16))
+			return AVHIP_NOT_SUPPORTED;
+		const ConvGeom g = make_geom<TE>(s);
+		const dim3 grid(ceil_div(g.pixels, BLOCK_M), ceil_div(s.K, BLOCK_N), static_cast<unsigned int>(plan.splits));
+		hipLaunchKernelGGL((k_conv_igemm_split<TE>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, plan.steps_per_split,
+				static_cast<float*>(workspace));
+		const FloatEpilogue<TE> epi { static_cast<const float*>(bias), static_cast<const TE*>(z), static_cast<TE*>(y), static_cast<float>(alpha1),
+				static_cast<float>(alpha2), static_cast<float>(beta), activation, s.K, true };
+		const int64_t plane = g.pixels * s.K;
+		hipLaunchKernelGGL((k_split_reduce<TE>), dim3(ceil_div(plane / 4, 256)), dim3(256), 0, st, static_cast<const float*>(workspace), plan.splits, plane, epi);
+		return 0;
+	}
+	bool shape_ok(const avhipConvShape *shape)
+	{
+		if (shape == nullptr)
+			return false;
+		const avhipConvShape &s = *shape;
+		return s.N > 0 && s.H > 0 && s.W > 0 && s.C > 0 && s.K > 0 && s.R > 0 && s.S > 0 && s.Ho > 0 && s.Wo > 0 && s.stride_h > 0 && s.stride_w > 0 && s.dil_h > 0
+				&& s.dil_w > 0 && (static_cast<int64_t>(s.K) + BLOCK_N - 1) / BLOCK_N <= 65535;
+	}
+}
+
+extern "C" int avhip_conv2d_split_k_workspace(int x_dtype, const avhipConvShape *shape, int64_t *bytes)
+{
+	if (!shape_ok(shape) || bytes == nullptr)
+		return AVHIP_BAD_PARAM;
+	SplitPlan plan;
+	bool yes = false;
+	switch (x_dtype)
+	{
+		case DT_FLOAT32:
+			yes = split_k_plan<float>(*shape, plan);
+			break;
+		case DT_FLOAT16:
+			yes = split_k_plan<f16_t>(*shape, plan);
+			break;
+		case DT_BFLOAT16:
+			yes = split_k_plan<bf16_t>(*shape, plan);
+			break;
+		default:
+			break;
+	}
+	*bytes = yes ? plan.bytes : 0;
+	return 0;
+}
+
+extern "C" int avhip_conv2d_implicit_gemm_split_k(void *stream, int x_dtype, const avhipConvShape *shape, const void *x, const void *w, const void *bias,
+		const void *z, void *y, const void *padding_value, double alpha1, double alpha2, double beta, int activation, void *workspace, int64_t workspace_bytes)
+{
+	if (!shape_ok(shape) || x == nullptr || w == nullptr || y == nullptr)
+		return AVHIP_BAD_PARAM;
+	hipStream_t st = static_cast<hipStream_t>(stream);
+	switch (x_dtype)
+	{
+		case DT_FLOAT32:
+			return launch_split<float>(st, *shape, x, w, bias, z, y, padding_value, alpha1, alpha2, beta, activation, workspace, workspace_bytes);
+		case DT_FLOAT16:
+			return launch_split<f16_t>(st, *shape, x, w, bias, z, y, padding_value, alpha1, alpha2, beta, activation, workspace, workspace_bytes);
+		case DT_BFLOAT16:
+			return launch_split<bf16_t>(st, *shape, x, w, bias, z, y, padding_value, alpha1, alpha2, beta, activation, workspace, workspace_bytes);
+		default:
+			return AVHIP_NOT_SUPPORTED;
 	}
 }

@@ -185,34 +185,48 @@ extern "C" int avhip_set_small_problem_threshold(int workgroups)
 
 namespace avhip
 {
+	/* Small in tiles is not enough: the problem must be short in k as well.  A wavefront fetches its own operands, one 32-byte
+	 * slab of both per MFMA with no re-use inside a workgroup: measured about 0.12 us per slab, plus 0.19 us per slab and
+	 * wavefront per SIMD as the tiles crowd L2 (a 3x3 layer of 256 channels on 32 images of 14 x 14 took 59 us here and 19 us in
+	 * the image-tile kernel with half the compute units idle).  The workgroup-tile kernels take about 0.7 us per 128-byte
+	 * k-step and 4 us around the loop, per round of 512 workgroups. */
+	SmallProblemEstimate conv_small_estimate(const avhipConvShape &s, int element_bytes, int64_t big_tile_workgroups)
+	{
+		const int64_t pixels = static_cast<int64_t>(s.N) * s.Ho * s.Wo;
+		const int64_t tiles = ((pixels + SMALL_TILE - 1) / SMALL_TILE) * ((static_cast<int64_t>(s.K) + SMALL_TILE - 1) / SMALL_TILE);
+		const int slabs_per_tap = (s.C * element_bytes + 31) / 32;
+		SmallProblemEstimate e;
+		/* fewer tiles than half the 1024 SIMDs of the chip, and enough k to share: four wavefronts per tile */
+		e.split_k = tiles < 512 && static_cast<int64_t>(s.R) * s.S * slabs_per_tap >= 4 * GROUP;
+		const double wavefronts = static_cast<double>(tiles) * (e.split_k ? 4 : 1);
+		const double slabs = static_cast<double>(s.R) * s.S * slabs_per_tap / (e.split_k ? 4 : 1);
+		e.small_us = 2.5 + slabs * (0.12 + 0.19 * wavefronts / 1024.0);
+		const double k_steps = static_cast<double>(s.R) * s.S * ((s.C * element_bytes + 127) / 128);
+		e.workgroup_tiles_us = static_cast<double>((big_tile_workgroups + 511) / 512) * (0.7 * k_steps + 4.0);
+		return e;
+	}
+	bool conv_small_preferred(const avhipConvShape &s, int element_bytes, int64_t big_tile_workgroups)
+	{
+		const int64_t busy = small_problem_threshold().load(std::memory_order_relaxed);
+		if (busy < 0) /* asked for by name (tests): whatever the kernel can run */
+			return true;
+		if (big_tile_workgroups >= busy)
+			return false;
+		const SmallProblemEstimate e = conv_small_estimate(s, element_bytes, big_tile_workgroups);
+		return e.small_us <= e.workgroup_tiles_us;
+	}
+
 	template<typename TE, typename Epi>
 	bool conv_small_launch(hipStream_t stream, const avhipConvShape &s, const void *x, const void *w, const Epi &epi, int64_t big_tile_workgroups)
 	{
-		const int64_t BUSY = small_problem_threshold().load(std::memory_order_relaxed);
-		const bool always = BUSY < 0; /* asked for by name (tests): whatever the kernel can run */
 		const int64_t pixels = static_cast<int64_t>(s.N) * s.Ho * s.Wo;
-		if ((!always && big_tile_workgroups >= BUSY) || !epi.vec || s.R * s.S > 32)
+		if (!conv_small_preferred(s, static_cast<int>(sizeof(TE)), big_tile_workgroups) || !epi.vec || s.R * s.S > 32)
 			return false;
 		const int64_t tiles = (pixels + SMALL_TILE - 1) / SMALL_TILE, filter_tiles = (static_cast<int64_t>(s.K) + SMALL_TILE - 1) / SMALL_TILE;
 		if (tiles > 0x7FFFFFFFll || filter_tiles > 65535 || pixels >= (1ll << 31) - SMALL_TILE)
 			return false;
 		const int slabs_per_tap = (s.C * static_cast<int>(sizeof(TE)) + 31) / 32;
-		const bool split_k = tiles * filter_tiles < 512 && static_cast<int64_t>(s.R) * s.S * slabs_per_tap >= 4 * GROUP;
-		if (!always)
-		{
-			/* Small in tiles is not enough: the problem must be short in k as well.  A wavefront fetches its own operands, one
-			 * 32-byte slab of both per MFMA with no re-use inside a workgroup: measured about 0.12 us per slab, plus 0.19 us per
-			 * slab and wavefront per SIMD as the tiles crowd L2 (a 3x3 layer of 256 channels on 32 images of 14 x 14 took 59 us
-			 * here and 19 us in the image-tile kernel with half the compute units idle).  The workgroup-tile kernels take about
-			 * 0.7 us per 128-byte k-step and 4 us around the loop, per round of 512 workgroups. */
-			const double wavefronts = static_cast<double>(tiles * filter_tiles) * (split_k ? 4 : 1);
-			const double slabs = static_cast<double>(s.R) * s.S * slabs_per_tap / (split_k ? 4 : 1);
-			const double here = 2.5 + slabs * (0.12 + 0.19 * wavefronts / 1024.0);
-			const double k_steps = static_cast<double>(s.R) * s.S * ((s.C * static_cast<int>(sizeof(TE)) + 127) / 128);
-			const double there = static_cast<double>((big_tile_workgroups + 511) / 512) * (0.7 * k_steps + 4.0);
-			if (here > there)
-				return false;
-		}
+		const bool split_k = conv_small_estimate(s, static_cast<int>(sizeof(TE)), big_tile_workgroups).split_k;
 		SmallGeom g;
 		g.H = s.H;
 		g.W = s.W;

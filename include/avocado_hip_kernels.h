@@ -120,6 +120,20 @@ extern "C"
 	 * src/descriptors.cu:22-39. */
 	AVHIP_API int avhip_set_memory(void *stream, void *dst, int64_t bytes, const void *pattern, int pattern_size);
 
+	/* The implicit-GEMM forward with k split across workgroups, for layers with few output pixels and a long k (fewer than 256
+	 * tiles of 128 x 128 and a walk that is worth cutting, by the launcher's estimate): parts of the k range are summed in
+	 * fp32 into `workspace` ([parts][N * Ho * Wo][K] floats), a second kernel adds the parts and applies the same epilogue as
+	 * avhip_conv2d_implicit_gemm (any activation).  fp32 / fp16 / bf16 tensors, y of the type of x, fp32 bias.  Returns
+	 * AVHIP_NOT_SUPPORTED, with nothing launched, when the layer is not worth splitting, the workspace is smaller than
+	 * avhip_conv2d_split_k_workspace() reports, or the tensors are not aligned for the branch-free loaders (the caller then
+	 * uses avhip_conv2d_implicit_gemm).  No counterpart in the reference, whose prototype has one tiling
+	 * (src/conv2d_implicit_gemm.cu:303-352). */
+	AVHIP_API int avhip_conv2d_implicit_gemm_split_k(void *stream, int x_dtype, const avhipConvShape *shape, const void *x, const void *w, const void *bias,
+			const void *z, void *y, const void *padding_value, double alpha1, double alpha2, double beta, int activation, void *workspace,
+			int64_t workspace_bytes);
+	/* Bytes of workspace with which avhip_conv2d_implicit_gemm_split_k takes the layer; 0 when it would not. */
+	AVHIP_API int avhip_conv2d_split_k_workspace(int x_dtype, const avhipConvShape *shape, int64_t *bytes);
+
 	/* Tuning knob without a counterpart in the reference.  The implicit-GEMM launcher sends a convolution to the kernel with
 	 * one 32 x 32 tile per wavefront when its 128 x 128 tiling would yield fewer than this many workgroups (default 192 on
 	 * the 256 compute units of an MI355X) and its k extent is short enough for that kernel to be the faster one by the

@@ -1,6 +1,8 @@
 """GPU parity of the convolution entry points (implicit GEMM, fused Winograd, dispatcher, requantised int8) against the CPU
 oracle on identical seeded inputs, through the C API.  Bars: int8 bit-exact; fp32 implicit GEMM rel-L2 <= 1e-5; fp32 Winograd
 <= 1e-4; fp16 / bf16 <= 2e-3."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -550,3 +552,48 @@ def test_convolution_argument_errors(oracle):
     # an empty batch is refused, not skipped (the reference's launch with a zero-sized grid fails as well)
     h.conv_forward("implicit_gemm", np.zeros((0, 6, 6, 8)), w, (0, 6, 6, 4), "f32", expect=cb.STATUS_BAD_PARAM)
     h.conv_forward("winograd_fused", x, np.zeros((4, 5, 5, 8)), (2, 6, 6, 4), "f32", pad=(-2, -2), expect=cb.STATUS_NOT_SUPPORTED)
+
+
+# ---- few output pixels, long k: the dispatcher splits k across workgroups when the caller lends it a workspace -----------------
+SPLIT_CASES = [
+    dict(x=(4, 7, 7, 512), w=(512, 3, 3, 512), pad=(-1, -1)),                        # the last stage of a residual network
+    dict(x=(8, 7, 7, 2048), w=(256, 1, 1, 2048), pad=(0, 0)),                        # 1x1, thirty-two k-steps
+    dict(x=(2, 14, 14, 256), w=(256, 3, 3, 256), pad=(-1, -1), stride=(2, 2)),       # strided
+    dict(x=(3, 9, 8, 160), w=(72, 3, 3, 160), pad=(-1, -1), mode=1),                 # the last part of k shorter and odd; flipped; partial tiles
+    dict(x=(2, 6, 6, 192), w=(40, 5, 5, 192), pad=(-2, -2), dilation=(1, 2)),        # 25 taps, dilated
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", SPLIT_CASES, ids=[str(i) for i in range(len(SPLIT_CASES))])
+def test_split_k_through_the_dispatcher(oracle, tiling, dtype, case):
+    if tiling != "workgroup_tiles":
+        pytest.skip("with the one-wavefront-per-tile kernel available the plan leaves layers this small to it")
+    g = h.rng(43)
+    x = h.rounded(oracle, g.standard_normal(case["x"]), dtype)
+    w = he(g, case["w"], dtype, oracle)
+    ys = out_shape(oracle, case)
+    b = g.uniform(-0.1, 0.1, ys[3]).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal(ys), dtype)
+    y0 = h.rounded(oracle, g.standard_normal(ys), dtype)
+    kw = dict(pad=case["pad"], stride=case.get("stride", (1, 1)), dilation=case.get("dilation", (1, 1)), mode=case.get("mode", 0))
+    # the workspace query names the plan: partial sums of at least two parts
+    with h.Call() as c:
+        conv = cb.ConvolutionDescriptor(mode=kw["mode"], padding=kw["pad"], strides=kw["stride"], dilation=kw["dilation"], dtype=h.DT[dtype])
+        xt, wt = c.tensor(x, dtype), c.tensor(w, dtype)
+        need = C.c_int64(0)
+        cb.check(c.lib.cudaGetConvolutionWorkspaceSize(c.ctx.handle, conv.handle, xt.desc, wt.desc, 0, C.byref(need)), "workspace size")
+    fused_winograd = dtype == "f32" and case["w"][1:3] == (3, 3) and "stride" not in case
+    if not fused_winograd:
+        assert need.value >= 2 * 4 * ys[0] * ys[1] * ys[2] * ys[3], need.value
+    a2, be = float(np.float32(0.7)), float(np.float32(0.3))
+    for act, oact in ((cb.ACTIVATION_RELU, oracle.RELU), (cb.ACTIVATION_TANH, oracle.TANH)):
+        got = h.conv_forward("dispatch", x, w, ys, dtype, bias=b, z=z, y0=y0, alpha2=a2, beta=be, activation=act, **kw)
+        want = oracle.conv2d(x, w, b, z, y0, alpha2=a2, beta=be, activation=oact, **kw)
+        assert got.shape == want.shape
+        assert oracle.rel_l2(got, want) < BAR[dtype] * (3 if dtype == "f32" else 1)
+    # without a workspace the plain kernels take the layer: the same result to rounding
+    plain = h.conv_forward("dispatch", x, w, ys, dtype, bias=b, workspace_bytes=0, **kw)
+    split = h.conv_forward("dispatch", x, w, ys, dtype, bias=b, **kw)
+    assert oracle.rel_l2(split, plain) < BAR[dtype] * (3 if dtype == "f32" else 1)
+    assert oracle.rel_l2(split, oracle.conv2d(x, w, b, **kw)) < BAR[dtype] * (3 if dtype == "f32" else 1)
