@@ -457,12 +457,14 @@ namespace avhip
 			{
 				int t[W];
 				integer_values<W>(t, v, c);
-				/* whole runs leave as streaming vector stores: the kernel never reads y back, so the caches may drain it while
-				 * the kernel runs.  int32 results (16 bytes per work-item, whole cache lines per row) are fastest as plain
-				 * non-temporal stores; so are int8 results of a workgroup that writes whole lines (the 1x1 kernels: 7.5 us
-				 * against 9.8 us written through).  Where a workgroup's row of int8 results is part of a cache line (64 filters
-				 * of the tile kernel) they are written through as well, or the partial lines wait in L2 for the write-back at the
-				 * end of the kernel (config 4, requantised 3x3 layer: 17.0 -> 14.8 us; int32 results there: 14.6 -> 16.6 us) */
+				/* int32 results (16 bytes per work-item, whole cache lines per row) leave as non-temporal vector stores: the
+				 * kernel never reads y back, so the caches may drain it while the kernel runs.  int8 results of a workgroup that
+				 * writes whole lines (the 1x1 kernels) leave as ordinary stores, 8 bytes per work-item, which L2 puts together:
+				 * 7.7 us on config 4 (9.8 us written through, 7.6 us with the non-temporal hint), but a layer that writes 206 MB
+				 * takes 95 us this way against 221 us with the hint.  Where a workgroup's row of int8 results is part of a cache
+				 * line (64 filters of the tile kernel) they are written through, or the partial lines wait in L2 for the
+				 * write-back at the end of the kernel (config 4, requantised 3x3 layer: 17.0 -> 14.8 us; int32 results there:
+				 * 14.6 -> 16.6 us) */
 				typedef typename Words<W / 4>::type words_t; /* W int8 values as 32-bit words */
 				if (MODE == I8_EXACT)
 				{
@@ -502,7 +504,7 @@ namespace avhip
 							if (through)
 								store_through(reinterpret_cast<words_t*>(dst), o.w);
 							else
-								__builtin_nontemporal_store(o.w, reinterpret_cast<words_t*>(dst));
+								*reinterpret_cast<words_t*>(dst) = o.w;
 						}
 						else
 							__builtin_nontemporal_store(o.w, reinterpret_cast<words_t*>(dst));
