@@ -1854,6 +1854,14 @@ namespace avocado
 					* ((p.shape.K + 127) / 128);
 			NonFusedPlan plan;
 			Memory *ws = get_memory(workspaceMem);
+			/* few output pixels and a long k: where the Winograd kernels could not fill the chip either, the implicit GEMM with k
+			 * split across workgroups comes first (fp32 3x3 512->512 on 32 images of 7x7: 86 us against 340 us) */
+			if (fused_workgroups < 256)
+			{
+				const avStatus_t ss = run_split_k(call, ws, workspaceMem, yMem, activation);
+				if (ss != AVOCADO_STATUS_NOT_SUPPORTED)
+					return ss;
+			}
 			const bool nonfused_ready = nonfused_plan(p, plan) && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32 && ws != nullptr && ws->data != nullptr
 					&& ws->size >= plan.total && reinterpret_cast<uintptr_t>(ws->data) % 256 == 0;
 			/* AVOCADO_STATUS_BAD_ALLOC from a Winograd plan means that the stream is capturing and the transformed weights are not

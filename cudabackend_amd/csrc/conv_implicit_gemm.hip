@@ -776,17 +776,24 @@ namespace
 			return false;
 		const double plane_bytes = static_cast<double>(pixels) * s.K * 4.0;
 		double other = 4.0 + 0.7 * static_cast<double>(steps);
+		int64_t plain_workgroups = tiles;
 		if (s.stride_h == 1 && s.stride_w == 1 && s.dil_h == 1 && s.dil_w == 1 && s.R * s.S > 1 && s.Ho * s.Wo >= 128)
 		{
 			/* the image-tile kernel takes such layers: 0.47 us per step for a workgroup with a compute unit to itself, 0.68 us
 			 * when two share one, 3.6 us around the loop */
 			const int64_t workgroups = static_cast<int64_t>(s.N) * ((s.K + 63) / 64) * ((s.Ho * s.Wo + 255) / 256);
 			other = 3.6 + (workgroups <= 256 ? 0.47 : 0.68) * static_cast<double>(steps);
+			plain_workgroups = workgroups;
 		}
 		if (s.R * s.S <= 32 && conv_small_preferred(s, static_cast<int>(sizeof(TE)), tiles))
 			other = std::min(other, conv_small_estimate(s, static_cast<int>(sizeof(TE)), tiles).small_us);
-		const double split = 10.0 + 0.7 * static_cast<double>(per_part) + 0.25 * static_cast<double>(parts)
-				+ plane_bytes * static_cast<double>(parts + 1) / 4.0e6;
+		/* neither path is faster than the matrix cores of the compute units it occupies (what decides for fp32, whose MFMAs
+		 * take eight times as long per element): flops per microsecond of the chip as sustained on random data */
+		const double chip = sizeof(TE) == 4 ? 1.55e8 : 1.87e9;
+		const double flops = 2.0 * static_cast<double>(pixels) * s.K * s.C * s.R * s.S;
+		other = std::max(other, flops / (chip * std::min(1.0, static_cast<double>(plain_workgroups) / 256.0)));
+		const double walk = std::max(0.7 * static_cast<double>(per_part), flops / (chip * std::min(1.0, static_cast<double>(tiles * parts) / 256.0)));
+		const double split = 10.0 + walk + 0.25 * static_cast<double>(parts) + plane_bytes * static_cast<double>(parts + 1) / 4.0e6;
 		if (split > 0.85 * other)
 			return false;
 		plan.splits = static_cast<int>(parts);

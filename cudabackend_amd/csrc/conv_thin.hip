@@ -47,7 +47,7 @@ namespace
 	using namespace avhip;
 
 	constexpr int THIN_FILTERS = 64; /* filters per block */
-	constexpr int THIN_LDS = 80 * 1024; /* most a workgroup may ask for (two per compute unit); it asks for what the layer needs */
+	constexpr int THIN_LDS = 160 * 1024; /* most a workgroup may ask for: the LDS of a compute unit; it asks for what the layer needs (two fit up to 80 KB) */
 	constexpr int THIN_MAX_K_BYTES = 1024;
 	constexpr int THIN_MAX_PIXEL_BYTES = 64;
 	constexpr unsigned int THIN_NO_PIECE = 0xFFFFFFFFu; /* table entry of a piece past the end of k */
@@ -572,8 +572,10 @@ namespace avhip
 		g.tiles = static_cast<unsigned int>(best_tiles * s.N);
 		g.items = g.tiles * g.filter_blocks;
 		const unsigned int lds_bytes = g.halo_bytes + fixed_bytes;
-		/* the workgroups that stay resident (two per compute unit: registers and LDS) share the work items */
-		const dim3 grid(std::min(g.items, persistent_workgroups(1 << 30)));
+		/* the workgroups that stay resident (two per compute unit by their registers, one where LDS allows no more) share the
+		 * work items */
+		const unsigned int resident = persistent_workgroups(1 << 30) / (lds_bytes > 80u * 1024u ? 2 : 1);
+		const dim3 grid(std::min(g.items, resident));
 #define AVHIP_THIN(PB) \
 		if (lds_bytes > 64u * 1024u) \
 			(void)hipFuncSetAttribute(reinterpret_cast<const void*>(&k_conv_thin<TE, PB, Epi>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)); \
