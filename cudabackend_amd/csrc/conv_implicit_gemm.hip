@@ -785,13 +785,17 @@ namespace
 			other = 3.6 + (workgroups <= 256 ? 0.47 : 0.68) * static_cast<double>(steps);
 			plain_workgroups = workgroups;
 		}
-		if (s.R * s.S <= 32 && conv_small_preferred(s, static_cast<int>(sizeof(TE)), tiles))
-			other = std::min(other, conv_small_estimate(s, static_cast<int>(sizeof(TE)), tiles).small_us);
 		/* neither path is faster than the matrix cores of the compute units it occupies (what decides for fp32, whose MFMAs
 		 * take eight times as long per element): flops per microsecond of the chip as sustained on random data */
 		const double chip = sizeof(TE) == 4 ? 1.55e8 : 1.87e9;
 		const double flops = 2.0 * static_cast<double>(pixels) * s.K * s.C * s.R * s.S;
 		other = std::max(other, flops / (chip * std::min(1.0, static_cast<double>(plain_workgroups) / 256.0)));
+		if (s.R * s.S <= 32 && conv_small_preferred(s, static_cast<int>(sizeof(TE)), tiles))
+		{
+			const double wavefronts = static_cast<double>(((pixels + 31) / 32) * ((s.K + 31) / 32));
+			const double small = std::max(conv_small_estimate(s, static_cast<int>(sizeof(TE)), tiles).small_us, flops / (chip * std::min(1.0, wavefronts / 1024.0)));
+			other = std::min(other, small);
+		}
 		const double walk = std::max(0.7 * static_cast<double>(per_part), flops / (chip * std::min(1.0, static_cast<double>(tiles * parts) / 256.0)));
 		const double split = 10.0 + walk + 0.25 * static_cast<double>(parts) + plane_bytes * static_cast<double>(parts + 1) / 4.0e6;
 		if (split > 0.85 * other)
