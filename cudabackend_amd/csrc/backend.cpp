@@ -1854,9 +1854,15 @@ namespace avocado
 					* ((p.shape.K + 127) / 128);
 			NonFusedPlan plan;
 			Memory *ws = get_memory(workspaceMem);
-			/* few output pixels and a long k: where the Winograd kernels could not fill the chip either, the implicit GEMM with k
-			 * split across workgroups comes first (fp32 3x3 512->512 on 32 images of 7x7: 86 us against 340 us) */
-			if (fused_workgroups < 256)
+			/* few output pixels and a long k: where the fused Winograd kernel does not pay (below), the implicit GEMM with k split
+			 * across workgroups comes first (fp32 3x3 512->512 on 32 images of 7x7: 86 us against 340 us) */
+			/* the fused kernel pays where its workgroups (one per compute unit) cover most of the chip and its 16 x 16 tiles are
+			 * mostly image: at 128 workgroups it loses to the implicit GEMM (3x3 128->128 on 32 images of 28 x 28: 96 against 81 us),
+			 * at 256 it wins (77 against 146 us on 64 images); on 7 x 7 images, a fifth of a tile, it takes twice the time of the
+			 * implicit GEMM */
+			const double fused_fill = static_cast<double>(p.shape.Ho) * p.shape.Wo / (((p.shape.Ho + 15) / 16 * 16.0) * ((p.shape.Wo + 15) / 16 * 16.0));
+			const bool fused_pays = fused_workgroups >= 160 && fused_fill >= 0.5;
+			if (!fused_pays)
 			{
 				const avStatus_t ss = run_split_k(call, ws, workspaceMem, yMem, activation);
 				if (ss != AVOCADO_STATUS_NOT_SUPPORTED)
@@ -1873,7 +1879,7 @@ namespace avocado
 					return ns;
 			}
 			else if (fused_winograd_applicable(p) && p.x_dtype == AVOCADO_DTYPE_FLOAT32 && bias_fp32 && p.shape.C >= 32 && p.shape.K >= 32
-					&& p.shape.Ho == p.shape.H && p.shape.Wo == p.shape.W && fused_workgroups >= 128)
+					&& p.shape.Ho == p.shape.H && p.shape.Wo == p.shape.W && fused_pays)
 			{
 				const avStatus_t fs = run_fused_winograd(call, wMem, yMem, activation);
 				if (fs != AVOCADO_STATUS_NOT_SUPPORTED && fs != AVOCADO_STATUS_BAD_ALLOC)
