@@ -187,3 +187,44 @@ def test_descriptor_tables_survive_concurrent_callers():
     for th in threads:
         th.join()
     assert not errors, errors[0]
+
+
+class ConvShape(C.Structure):
+    """avhipConvShape of include/avocado_hip_kernels.h."""
+    _fields_ = [(n, C.c_int) for n in ("N", "H", "W", "C", "K", "R", "S", "Ho", "Wo", "pad_h", "pad_w", "stride_h", "stride_w", "dil_h", "dil_w", "mode")]
+
+
+def split_k_bytes(lib, dtype, N, H, Cin, K, R, stride=1):
+    pad = -(R // 2)
+    Ho = (H - 2 * pad - R) // stride + 1
+    s = ConvShape(N, H, H, Cin, K, R, R, Ho, Ho, pad, pad, stride, stride, 1, 1, 0)
+    out = C.c_int64(-1)
+    lib.avhip_conv2d_split_k_workspace.argtypes = [C.c_int, C.POINTER(ConvShape), C.POINTER(C.c_int64)]
+    assert lib.avhip_conv2d_split_k_workspace(dtype, C.byref(s), C.byref(out)) == 0
+    return out.value, N * Ho * Ho * K * 4
+
+
+def test_split_k_plan_is_for_few_pixels_and_a_long_k():
+    """The host-side plan of the split-k implicit GEMM (no GPU involved): partial sums of two or more parts for the last stages
+    of a deep network at a modest batch, nothing for layers that fill the chip, that are short in k, that the small-problem
+    kernel takes, or whose tensors the branch-free loaders cannot read."""
+    lib = cb.load_library()
+    bf16, f32, i8 = cb.DTYPE_BFLOAT16, cb.DTYPE_FLOAT32, cb.DTYPE_INT8
+    got, plane = split_k_bytes(lib, bf16, 32, 7, 512, 512, 3)           # 3x3 512->512 on 32 images of 7x7
+    assert got >= 2 * plane and got % plane == 0
+    got, plane = split_k_bytes(lib, bf16, 32, 14, 512, 512, 3, stride=2)
+    assert got >= 2 * plane
+    got, plane = split_k_bytes(lib, f32, 32, 14, 256, 256, 3)           # fp32: half the compute units would idle for 8x the MFMA time
+    assert got >= 2 * plane
+    assert split_k_bytes(lib, bf16, 256, 15, 128, 128, 3)[0] == 0       # BASELINE config 2: 900 tiles of 128 x 128
+    assert split_k_bytes(lib, bf16, 32, 14, 256, 256, 3)[0] == 0        # the image-tile kernel's pace is hard to beat
+    assert split_k_bytes(lib, bf16, 32, 14, 256, 1024, 1)[0] == 0       # four k-steps
+    assert split_k_bytes(lib, f32, 8, 15, 64, 64, 3)[0] == 0            # BASELINE config 1: the small-problem kernel's
+    assert split_k_bytes(lib, bf16, 4, 7, 512, 512, 3)[0] == 0          # tiny batch: the small-problem kernel's
+    assert split_k_bytes(lib, i8, 32, 7, 512, 512, 3)[0] == 0           # floating types only
+    assert split_k_bytes(lib, bf16, 32, 7, 500, 512, 3)[0] == 0         # 1000 bytes of channels: not whole 16-byte chunks
+    assert split_k_bytes(lib, bf16, 32, 7, 512, 512, 7)[0] == 0         # 49 taps: beyond the loaders' tap mask
+    s = ConvShape(0, 7, 7, 512, 512, 3, 3, 7, 7, -1, -1, 1, 1, 1, 1, 0)
+    out = C.c_int64(0)
+    assert lib.avhip_conv2d_split_k_workspace(bf16, C.byref(s), C.byref(out)) != 0      # N = 0
+    assert lib.avhip_conv2d_split_k_workspace(bf16, None, C.byref(out)) != 0
