@@ -430,8 +430,10 @@ namespace
 	};
 
 	/* One kernel for every epilogue: Epi is FloatEpilogue<TE> or Int8Epilogue<mode>.  FAST instances use the branch-free
-	 * loaders and are launched for LINEAR / RELU only; everything else runs the general instance. */
-	template<typename TE, bool FAST, typename Epi>
+	 * loaders and are launched for LINEAR / RELU only; everything else runs the general instance.  A FAST instance without
+	 * VEC is for filter counts that are not a multiple of four (21 classes, 255 = 3 x 85 box values) or unaligned y: the
+	 * loaders are what makes the general instance slow, not its element-wise stores. */
+	template<typename TE, bool FAST, typename Epi, bool VEC = FAST>
 	__global__ __launch_bounds__(256, 2) void k_conv_igemm(const TE *__restrict__ x, const TE *__restrict__ w, ConvGeom g, TE padv, int vec_ok, Epi epi)
 	{
 		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
@@ -453,7 +455,7 @@ namespace
 		{
 			const int64_t p = p0 + r;
 			if (p < g.pixels && k < g.K)
-				epi.template store<FAST ? ACT_SIMPLE : ACT_ANY, FAST>(p, k, v, columns); /* fast instances store whole 4-filter vectors */
+				epi.template store<FAST ? ACT_SIMPLE : ACT_ANY, VEC>(p, k, v, columns); /* VEC instances store whole 4-filter vectors */
 		});
 	}
 
@@ -662,6 +664,9 @@ namespace
 			return 0;
 		if (fast)
 			hipLaunchKernelGGL((k_conv_igemm<TE, true, Epi>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags, epi);
+		else if (fast_path_ok<TE>(s, flags, padding_value) && is_simple_activation(epi.activation))
+			hipLaunchKernelGGL((k_conv_igemm<TE, true, Epi, false>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags,
+					epi);
 		else
 			hipLaunchKernelGGL((k_conv_igemm<TE, false, Epi>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags, epi);
 		return 0;

@@ -126,6 +126,51 @@ def test_int8_few_input_channels_bit_exact(oracle, case):
     np.testing.assert_array_equal(got, oracle.conv2d_i8(x, w, b, activation=cb.ACTIVATION_RELU, **kw))
 
 
+# ---- filter counts that are not a multiple of four: branch-free loaders, element-wise stores -------------------------------------
+ODD_FILTER_COUNTS = [
+    dict(x=(2, 20, 21, 64), w=(21, 1, 1, 64), pad=(0, 0)),                                        # 21 classes
+    dict(x=(2, 13, 13, 128), w=(255, 1, 1, 128), pad=(0, 0)),                                     # 3 x 85 box values, two filter blocks
+    dict(x=(2, 17, 18, 64), w=(3, 3, 3, 64), pad=(-1, -1)),                                       # an image out
+    dict(x=(2, 12, 14, 96), w=(35, 3, 3, 96), pad=(-1, -1), stride=(2, 1), mode=1),
+    dict(x=(1, 10, 10, 32), w=(130, 5, 5, 32), pad=(-4, -4), dilation=(2, 2)),
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", ODD_FILTER_COUNTS, ids=[str(i) for i in range(len(ODD_FILTER_COUNTS))])
+def test_odd_filter_counts(oracle, dtype, case):
+    g = h.rng(44)
+    x = h.rounded(oracle, g.standard_normal(case["x"]), dtype)
+    w = he(g, case["w"], dtype, oracle)
+    ys = out_shape(oracle, case)
+    b = g.uniform(-0.1, 0.1, ys[3]).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal(ys), dtype)
+    kw = dict(pad=case["pad"], stride=case.get("stride", (1, 1)), dilation=case.get("dilation", (1, 1)), mode=case.get("mode", 0))
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, bias=b, z=z, activation=cb.ACTIVATION_RELU, **kw)
+    want = oracle.conv2d(x, w, b, z, activation=oracle.RELU, **kw)
+    assert got.shape == want.shape
+    assert oracle.rel_l2(got, want) < BAR[dtype]
+    # every filter separately: the last ones are the ones a vector store would get wrong
+    per_filter = [oracle.rel_l2(got[..., k], want[..., k]) for k in range(ys[3])]
+    assert max(per_filter) < 4 * BAR[dtype], int(np.argmax(per_filter))
+
+
+@pytest.mark.parametrize("case", ODD_FILTER_COUNTS, ids=[str(i) for i in range(len(ODD_FILTER_COUNTS))])
+def test_odd_filter_counts_int8_bit_exact(oracle, case):
+    g = h.rng(45)
+    x = g.integers(-127, 128, case["x"], dtype=np.int8)
+    w = g.integers(-127, 128, case["w"], dtype=np.int8)
+    K = case["w"][0]
+    b = g.integers(-2 ** 15, 2 ** 15, K).astype(np.int32)
+    kw = dict(pad=case["pad"], stride=case.get("stride", (1, 1)), dilation=case.get("dilation", (1, 1)), mode=case.get("mode", 0))
+    ys = out_shape(oracle, case)
+    got = h.conv_forward("implicit_gemm", x, w, ys, "i8", y_dtype="i32", bias=b, bias_dtype="i32", activation=cb.ACTIVATION_RELU, **kw)
+    np.testing.assert_array_equal(got, oracle.conv2d_i8(x, w, b, activation=cb.ACTIVATION_RELU, **kw))
+    scale = g.uniform(1e-4, 1e-3, K).astype(np.float32)
+    got = h.conv_forward("requant", x, w, ys, "i8", y_dtype="i8", bias=b, bias_dtype="i32", scale=scale, activation=cb.ACTIVATION_LINEAR, **kw)
+    np.testing.assert_array_equal(got, oracle.requant_i8(oracle.conv2d_i8(x, w, b, **kw), scale))
+
+
 # ---- few input channels, images large enough for 256-pixel tiles: the kernel that gathers its operand from a tile in LDS ------
 THIN_CASES = [
     dict(x=(2, 40, 48, 3), w=(72, 7, 7, 3), pad=(-3, -3), stride=(2, 2)),                         # a residual network's first layer; the second filter block partial
