@@ -19,6 +19,7 @@
  */
 #include <algorithm>
 #include <cstring>
+#include <type_traits>
 
 #include "conv_epilogue.hpp"
 #include "conv_pointwise.hpp"
@@ -431,9 +432,10 @@ namespace
 
 	/* One kernel for every epilogue: Epi is FloatEpilogue<TE> or Int8Epilogue<mode>.  FAST instances use the branch-free
 	 * loaders and are launched for LINEAR / RELU only; everything else runs the general instance.  A FAST instance without
-	 * VEC is for filter counts that are not a multiple of four (21 classes, 255 = 3 x 85 box values) or unaligned y: the
-	 * loaders are what makes the general instance slow, not its element-wise stores. */
-	template<typename TE, bool FAST, typename Epi, bool VEC = FAST>
+	 * VEC is for filter counts that are not a multiple of four (21 classes, 255 = 3 x 85 box values) or unaligned y, a FAST
+	 * instance with ACT_ANY for the seven other activations: the loaders are what makes the general instance slow, not its
+	 * element-wise stores or its switch over the activations (a 3x3 layer with a sigmoid: 139 us there). */
+	template<typename TE, bool FAST, typename Epi, bool VEC = FAST, int ACT = (FAST ? ACT_SIMPLE : ACT_ANY)>
 	__global__ __launch_bounds__(256, 2) void k_conv_igemm(const TE *__restrict__ x, const TE *__restrict__ w, ConvGeom g, TE padv, int vec_ok, Epi epi)
 	{
 		__shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
@@ -451,12 +453,18 @@ namespace
 		typename Mma<TE>::acc_t acc[2][2];
 		block_mma<TE>(lds, g.R * g.S * g.steps_per_tap, la, lb, acc);
 
-		drain_tile<TE, 2, 2>(lds, acc, [&](int r, const typename Epi::scalar_t (&v)[4], int) __attribute__((always_inline))
+		auto row_out = [&](int r, const typename Epi::scalar_t (&v)[4], int) __attribute__((always_inline))
 		{
 			const int64_t p = p0 + r;
 			if (p < g.pixels && k < g.K)
-				epi.template store<FAST ? ACT_SIMPLE : ACT_ANY, VEC>(p, k, v, columns); /* VEC instances store whole 4-filter vectors */
-		});
+				epi.template store<ACT, VEC>(p, k, v, columns); /* VEC instances store whole 4-filter vectors */
+		};
+		/* (the nine-way switch of ACT_ANY, once per row of a fully unrolled hand-over, was too much to unroll: the accumulators
+		 * then lived in scratch memory and a layer with a sigmoid took 139 us against 12 us with ReLU) */
+		if constexpr (ACT == ACT_ANY)
+			drain_tile_rolled<TE, 2>(lds, acc, row_out);
+		else
+			drain_tile<TE, 2, 2>(lds, acc, row_out);
 	}
 
 	template<typename TE, int PB, typename Epi>
@@ -605,6 +613,9 @@ namespace
 	template<typename TE, typename Epi>
 	int launch(hipStream_t st, const avhipConvShape &s, const void *x, const void *w, const void *padding_value, int flags, const Epi &epi)
 	{
+		/* (the integer epilogues are only ever asked for LINEAR and RELU) */
+		constexpr bool integer_epilogue = std::is_same<Epi, Int8Epilogue<I8_EXACT>>::value || std::is_same<Epi, Int8Epilogue<I8_REQUANT>>::value;
+		constexpr int GENERAL_ACT = integer_epilogue ? ACT_SIMPLE : ACT_ANY;
 		const ConvGeom g = make_geom<TE>(s);
 		TE padv;
 		if (padding_value != nullptr)
@@ -664,11 +675,25 @@ namespace
 			return 0;
 		if (fast)
 			hipLaunchKernelGGL((k_conv_igemm<TE, true, Epi>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags, epi);
-		else if (fast_path_ok<TE>(s, flags, padding_value) && is_simple_activation(epi.activation))
-			hipLaunchKernelGGL((k_conv_igemm<TE, true, Epi, false>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags,
-					epi);
+		else if (fast_path_ok<TE>(s, flags, padding_value))
+		{
+			/* the branch-free loaders with what the layer needs of the general epilogue */
+			const bool vec = (flags & 2) != 0;
+#define AVHIP_GATHER(VEC, ACT) hipLaunchKernelGGL((k_conv_igemm<TE, true, Epi, VEC, ACT>), grid, dim3(256), 0, st, static_cast<const TE*>(x), \
+		static_cast<const TE*>(w), g, padv, flags, epi)
+			if (is_simple_activation(epi.activation))
+				AVHIP_GATHER(false, ACT_SIMPLE);
+			else if (vec && !integer_epilogue)
+			{
+				if constexpr (!integer_epilogue)
+					AVHIP_GATHER(true, ACT_ANY);
+			}
+			else /* both at once is left to the general instance */
+				hipLaunchKernelGGL((k_conv_igemm<TE, false, Epi, false, GENERAL_ACT>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags, epi);
+#undef AVHIP_GATHER
+		}
 		else
-			hipLaunchKernelGGL((k_conv_igemm<TE, false, Epi>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags, epi);
+			hipLaunchKernelGGL((k_conv_igemm<TE, false, Epi, false, GENERAL_ACT>), grid, dim3(256), 0, st, static_cast<const TE*>(x), static_cast<const TE*>(w), g, padv, flags, epi);
 		return 0;
 	}
 	template<typename TE>

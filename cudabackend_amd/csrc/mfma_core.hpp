@@ -22,6 +22,7 @@
 #define AVHIP_MFMA_CORE_HPP_
 
 #include "common.hpp"
+#include <type_traits>
 
 namespace avhip
 {
@@ -405,6 +406,51 @@ namespace avhip
 	__device__ __forceinline__ void drain_tile(char *lds, const typename Mma<TE>::acc_t (&acc)[TM][2], const F &f)
 	{
 		drain_tile<TE, TM, WAVES_N, CPL>(lds, acc, f, [](int) {});
+	}
+	/*
+	 * The same hand-over for epilogues that are long (a switch over nine activation functions with their exponentials and
+	 * logarithms): the rows of a pass are walked by a loop that stays a loop, so the epilogue is instantiated once per pass
+	 * instead of once per row, while the passes themselves are written out, so that every index into the accumulators is
+	 * a constant.  (With one unrollable loop nest the compiler gave up unrolling at that size, the accumulator indices became
+	 * variables and the accumulators lived in scratch memory for the whole kernel.)
+	 */
+	template<typename TE, int WAVES_N, typename F>
+	__device__ __forceinline__ void drain_tile_rolled(char *lds, const typename Mma<TE>::acc_t (&acc)[2][2], const F &f)
+	{
+		typedef typename Mma<TE>::scalar_t S;
+		typedef DrainShape<WAVES_N, 4> D;
+		S *sm = reinterpret_cast<S*>(lds);
+		const int tid = threadIdx.x;
+		const int lane = tid & 63;
+		const int wave = tid >> 6;
+		const int wm = WAVES_N == 2 ? (wave >> 1) : wave;
+		const int wn = WAVES_N == 2 ? (wave & 1) : 0;
+		const int col = drain_column<WAVES_N, 4>();
+		constexpr int ROW_STEP = 256 / D::threads_per_row;
+		constexpr int ITERS = D::rows_per_pass / ROW_STEP;
+		auto pass = [&](auto which) __attribute__((always_inline))
+		{
+			constexpr int tm = decltype(which)::value;
+			__syncthreads();
+#pragma unroll
+			for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+				for (int i = 0; i < 4; i++)
+#pragma unroll
+					for (int j = 0; j < 4; j++)
+						sm[(wm * 32 + 8 * i + 4 * (lane >> 5) + j) * D::pitch + wn * 64 + tn * 32 + (lane & 31)] = acc[tm][tn][4 * i + j];
+			__syncthreads();
+#pragma unroll 1
+			for (int it = 0; it < ITERS; it++)
+			{
+				typedef S quad_t __attribute__((ext_vector_type(4)));
+				const quad_t q = *reinterpret_cast<const quad_t*>(sm + (tid / D::threads_per_row + it * ROW_STEP) * D::pitch + col);
+				const S v[4] = { q[0], q[1], q[2], q[3] };
+				f(DrainRows<2, WAVES_N, 4>::row(tm * ITERS + it), v, tm * ITERS + it);
+			}
+		};
+		pass(std::integral_constant<int, 0>());
+		pass(std::integral_constant<int, 1>());
 	}
 	/*
 	 * The same hand-over for workgroups whose four wavefronts are stacked (each owns TM 32-row tiles by 64 columns, the
