@@ -462,7 +462,7 @@ namespace
 		/* (the nine-way switch of ACT_ANY, once per row of a fully unrolled hand-over, was too much to unroll: the accumulators
 		 * then lived in scratch memory and a layer with a sigmoid took 139 us against 12 us with ReLU) */
 		if constexpr (ACT == ACT_ANY)
-			drain_tile_rolled<TE, 2>(lds, acc, row_out);
+			drain_tile_rolled<TE, 2, 2>(lds, acc, row_out);
 		else
 			drain_tile<TE, 2, 2>(lds, acc, row_out);
 	}

@@ -343,20 +343,30 @@ namespace
 
 		/* four output pixels per tile: each (a, b) plane of accumulators leaves like one GEMM tile of 64 rows x 128 columns */
 		const int64_t image_pixels = static_cast<int64_t>(image) * g.Ho * g.Wo;
-#pragma unroll
-		for (int a = 0; a < 2; a++)
-#pragma unroll
-			for (int b = 0; b < 2; b++)
+		auto leave = [&](auto row_of_four, auto column_of_four) __attribute__((always_inline))
+		{
+			constexpr int a = decltype(row_of_four)::value, b = decltype(column_of_four)::value;
+			typename Kernel::acc_t plane[1][2] = { { kn.Y[a][b][0], kn.Y[a][b][1] } };
+			auto row_out = [&](int row, const float (&v)[4], int) __attribute__((always_inline))
 			{
-				typename Kernel::acc_t plane[1][2] = { { kn.Y[a][b][0], kn.Y[a][b][1] } };
-				drain_tile<TL, 1, 2>(lds, plane, [&](int row, const float (&v)[4], int) __attribute__((always_inline))
-				{
-					const int th = TILE_BLOCK * block_h + (row >> 3), tw = TILE_BLOCK * block_w + (row & 7);
-					const int oh = 2 * th + a, ow = 2 * tw + b;
-					if (oh < g.Ho && ow < g.Wo && k < g.K)
-						epi.template store<ACT>(image_pixels + static_cast<int64_t>(oh) * g.Wo + ow, k, v, columns);
-				});
-			}
+				const int th = TILE_BLOCK * block_h + (row >> 3), tw = TILE_BLOCK * block_w + (row & 7);
+				const int oh = 2 * th + a, ow = 2 * tw + b;
+				if (oh < g.Ho && ow < g.Wo && k < g.K)
+					epi.template store<ACT>(image_pixels + static_cast<int64_t>(oh) * g.Wo + ow, k, v, columns);
+			};
+			/* the long epilogue of ACT_ANY once per plane, in a loop over its rows; unrolled per row, the four planes were no
+			 * longer unrolled themselves and the accumulators went to scratch memory */
+			if constexpr (ACT == ACT_ANY)
+				drain_tile_rolled<TL, 1, 2>(lds, plane, row_out);
+			else
+				drain_tile<TL, 1, 2>(lds, plane, row_out);
+		};
+		typedef std::integral_constant<int, 0> zero_t;
+		typedef std::integral_constant<int, 1> one_t;
+		leave(zero_t(), zero_t());
+		leave(zero_t(), one_t());
+		leave(one_t(), zero_t());
+		leave(one_t(), one_t());
 	}
 
 	template<typename TX>

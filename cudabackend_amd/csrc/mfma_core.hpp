@@ -414,9 +414,10 @@ namespace avhip
 	 * a constant.  (With one unrollable loop nest the compiler gave up unrolling at that size, the accumulator indices became
 	 * variables and the accumulators lived in scratch memory for the whole kernel.)
 	 */
-	template<typename TE, int WAVES_N, typename F>
-	__device__ __forceinline__ void drain_tile_rolled(char *lds, const typename Mma<TE>::acc_t (&acc)[2][2], const F &f)
+	template<typename TE, int TM, int WAVES_N, typename F>
+	__device__ __forceinline__ void drain_tile_rolled(char *lds, const typename Mma<TE>::acc_t (&acc)[TM][2], const F &f)
 	{
+		static_assert(TM == 1 || TM == 2, "one or two passes, written out");
 		typedef typename Mma<TE>::scalar_t S;
 		typedef DrainShape<WAVES_N, 4> D;
 		S *sm = reinterpret_cast<S*>(lds);
@@ -446,11 +447,12 @@ namespace avhip
 				typedef S quad_t __attribute__((ext_vector_type(4)));
 				const quad_t q = *reinterpret_cast<const quad_t*>(sm + (tid / D::threads_per_row + it * ROW_STEP) * D::pitch + col);
 				const S v[4] = { q[0], q[1], q[2], q[3] };
-				f(DrainRows<2, WAVES_N, 4>::row(tm * ITERS + it), v, tm * ITERS + it);
+				f(DrainRows<TM, WAVES_N, 4>::row(tm * ITERS + it), v, tm * ITERS + it);
 			}
 		};
 		pass(std::integral_constant<int, 0>());
-		pass(std::integral_constant<int, 1>());
+		if constexpr (TM == 2)
+			pass(std::integral_constant<int, 1>());
 	}
 	/*
 	 * The same hand-over for workgroups whose four wavefronts are stacked (each owns TM 32-row tiles by 64 columns, the
