@@ -90,7 +90,9 @@ KERNEL_LAYER_SYMBOLS = ["avhip_winograd_weight_transform", "avhip_winograd_input
                         "avhip_winograd_gradient_transform", "avhip_winograd_update_transform", "avhip_gemm_batched",
                         "avhip_conv2d_implicit_gemm", "avhip_conv2d_implicit_gemm_split_k", "avhip_conv2d_split_k_workspace", "avhip_conv2d_winograd_fused", "avhip_add_bias", "avhip_im2row", "avhip_change_type",
                         "avhip_set_memory", "avhip_mfma_rate_probe", "avhip_set_small_problem_threshold", "avhip_set_short_k_engine",
-                        "avhip_affine_forward", "avhip_batchnorm_inference", "avhip_stream_probe"]
+                        "avhip_affine_forward", "avhip_batchnorm_inference", "avhip_stream_probe", "avhip_conv2d_winograd_rows",
+                        "avhip_winograd_rows_weight_transform", "avhip_winograd_rows_weight_bytes", "avhip_conv2d_winograd_rows_plan",
+                        "avhip_set_winograd_rows"]
 
 _lib = None
 

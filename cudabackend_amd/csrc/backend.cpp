@@ -449,7 +449,8 @@ namespace
 	{
 		uint64_t uid;
 		av_int64 offset;
-		int K, C, dtype, mode, m; /* m: Winograd output tile, 2 = F(2x2,3x3) for the fused kernel, 4 = F(4x4,3x3) for the non-fused plan */
+		int K, C, dtype, mode, m; /* m: Winograd output tile, 2 = F(2x2,3x3) for the fused kernel, 4 = F(4x4,3x3) for the non-fused plan,
+		                           * 1 = F(2,3) along rows in the operand layout of the row-Winograd kernel */
 		bool operator<(const WeightKey &o) const
 		{
 			return std::tie(uid, offset, K, C, dtype, mode, m) < std::tie(o.uid, o.offset, o.K, o.C, o.dtype, o.mode, o.m);
@@ -567,7 +568,8 @@ namespace
 		const av_int64 w_bytes = static_cast<av_int64>(p.shape.K) * 9 * p.shape.C * size_of(p.w_dtype);
 		const WeightKey key { owner->uid, offset, p.shape.K, p.shape.C, static_cast<int>(p.w_dtype), p.shape.mode, m };
 		const int t = m + 2;
-		const size_t bytes = static_cast<size_t>(t * t) * p.shape.K * p.shape.C * size_of(mat_dtype);
+		const size_t bytes = m == 1 ? static_cast<size_t>(avhip_winograd_rows_weight_bytes(p.shape.K, p.shape.C))
+				: static_cast<size_t>(t * t) * p.shape.K * p.shape.C * size_of(mat_dtype);
 		WeightCache &cache = weight_cache();
 		std::vector<WeightEntry> victims;
 		avStatus_t status = AVOCADO_STATUS_SUCCESS;
@@ -623,7 +625,8 @@ namespace
 				WeightEntry &e = it->second;
 				/* the write number is read before the transform is enqueued: a write that slips in between is seen next time */
 				e.seen = owner->writes->current();
-				const int rc = avhip_winograd_weight_transform(ctx.stream, p.w_dtype, mat_dtype, m, 3, p.shape.mode, wm->data, e.U, p.shape.K, p.shape.C);
+				const int rc = m == 1 ? avhip_winograd_rows_weight_transform(ctx.stream, p.w_dtype, p.shape.mode, wm->data, e.U, p.shape.K, p.shape.C)
+						: avhip_winograd_weight_transform(ctx.stream, p.w_dtype, mat_dtype, m, 3, p.shape.mode, wm->data, e.U, p.shape.K, p.shape.C);
 				status = from_launcher(rc);
 				cache.transforms++;
 				if (status == AVOCADO_STATUS_SUCCESS)
@@ -841,6 +844,36 @@ namespace
 		touch(yMem);
 		const int rc = avhip_conv2d_winograd_fused(c.ctx.stream, p.x_dtype, &p.shape, c.x->data, U, c.bias, c.z, c.y->data, c.alpha1, c.alpha2, c.beta,
 				activation);
+		return from_launcher(rc);
+	}
+
+	/* Row-wise Winograd F(2,3) for 16-bit 3x3 layers whose image bands fit a compute unit's LDS (conv_winograd_rows.hip): two
+	 * thirds of the direct kernel's MFMA work.  Worth it when its workgroups (one per compute unit, 128 filters each) cover
+	 * most of the chip and most of their 128 GEMM rows are image. */
+	bool rows_winograd_pays(const ConvCall &c, avActivationType_t activation)
+	{
+		const ConvProblem &p = c.problem;
+		if (p.y_dtype != p.x_dtype || !p.conv->padding_value_is_zero() || c.beta != 0.0 || (c.bias != nullptr && c.bias_dtype != AVOCADO_DTYPE_FLOAT32))
+			return false;
+		if (activation != AVOCADO_ACTIVATION_LINEAR && activation != AVOCADO_ACTIVATION_RELU)
+			return false;
+		int workgroups = 0, rows_used = 0;
+		if (avhip_conv2d_winograd_rows_plan(p.x_dtype, &p.shape, &workgroups, &rows_used) != 0)
+			return false;
+		return avhip_set_winograd_rows(-1) == 2 || (workgroups >= 192 && rows_used >= 96);
+	}
+	avStatus_t run_rows_winograd(const ConvCall &c, avMemoryDescriptor_t wMem, avMemoryDescriptor_t yMem, avActivationType_t activation)
+	{
+		const ConvProblem &p = c.problem;
+		const void *U = nullptr;
+		const avStatus_t st = cached_winograd_weights(c.ctx, p, wMem, 1, AVOCADO_DTYPE_FLOAT16, &U);
+		if (st != AVOCADO_STATUS_SUCCESS)
+			return st;
+		const int rc = avhip_conv2d_winograd_rows(c.ctx.stream, p.x_dtype, &p.shape, c.x->data, U, c.bias, c.z, c.y->data, c.alpha1, c.alpha2, c.beta,
+				activation);
+		if (rc == AVHIP_NOT_SUPPORTED)
+			return AVOCADO_STATUS_NOT_SUPPORTED;
+		touch(yMem);
 		return from_launcher(rc);
 	}
 
@@ -1862,6 +1895,14 @@ namespace avocado
 			 * implicit GEMM */
 			const double fused_fill = static_cast<double>(p.shape.Ho) * p.shape.Wo / (((p.shape.Ho + 15) / 16 * 16.0) * ((p.shape.Wo + 15) / 16 * 16.0));
 			const bool fused_pays = fused_workgroups >= 160 && fused_fill >= 0.5;
+			/* 16-bit 3x3 layers on small images: row-wise Winograd (BAD_ALLOC: capturing with a cold cache; NOT_SUPPORTED:
+			 * alignment; either way nothing was launched and the direct kernels take over) */
+			if (rows_winograd_pays(call, activation))
+			{
+				const avStatus_t rs = run_rows_winograd(call, wMem, yMem, activation);
+				if (rs != AVOCADO_STATUS_NOT_SUPPORTED && rs != AVOCADO_STATUS_BAD_ALLOC)
+					return rs;
+			}
 			if (!fused_pays)
 			{
 				const avStatus_t ss = run_split_k(call, ws, workspaceMem, yMem, activation);

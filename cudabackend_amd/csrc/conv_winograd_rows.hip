@@ -1,0 +1,600 @@
+/*
+ * conv_winograd_rows.hip -- 3x3 stride-1 convolution of 16-bit tensors by Winograd F(2,3) applied ALONG IMAGE ROWS ONLY,
+ * in one kernel, for layers whose whole image (or a band of its rows) fits the LDS of a compute unit.
+ *
+ * Same formula as the other forward paths, y = act(alpha1 * conv(x, w) + bias + alpha2 * z) + beta * y
+ * (include/Avocado/cuda_backend.h:822 of the reference; the reference's fused prototype is src/winograd_fused.cu:590-775,
+ * launched at :789-805, and transforms in both directions).  Why one direction here: on the matrix cores of gfx950 a 16-bit
+ * 3x3 layer is bound by the number of MFMA instructions, and what a two-dimensional transform saves there (2.25x) it gives
+ * back in vector instructions, because its sixteen accumulator planes do not fit the register file and every finished plane
+ * has to be folded into the outputs inside the k loop.  With the transform along one direction,
+ *
+ *     y[h, 2t + o] = sum_p A^T[o][p] * M_p[h, t],      M_p[h, t][k] = sum_{i, c} V_p[h + i, t][c] * U_p[i][k][c],
+ *     V_p[r, t] = sum_j B^T[p][j] * x[r, 2t + j],      U_p[i]      = sum_j G[p][j] * w[k, i, j],
+ *
+ * the four planes M_0..M_3 of (output row, column pair) x filter stay in accumulator registers for the whole k loop
+ * (k = 3 filter rows x C channels), the fold is four additions per pair of outputs, done once in the epilogue, and the matrix
+ * cores issue 12 products per channel and pair of outputs instead of 18: two thirds of the direct kernel's MFMA work.
+ * B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1], G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1], A^T = [1 1 1 0; 0 1 -1 -1]
+ * (the one-dimensional factors of the F(2x2,3x3) tables of src/winograd_nonfused.cu:534-575, signs moved between B and A).
+ *
+ * Workgroup = 8 wavefronts = one band of TH output rows of one image x 128 filters; GEMM rows are (row, column pair), at most
+ * 128.  Wavefront (p, half) owns plane M_p for 64 filters: 4 x 2 MFMA tiles of 32 x 32, 128 accumulator registers.
+ *   A operand: V_p lives in LDS, [slice of 64 channels][p][pixel = row * pairs + pair][128 bytes + 16], fp16; filter row i is
+ *              a constant shift of i * pairs pixels, so a 32-row tile always reads 32 consecutive pixels (conflict-free).
+ *              V is produced in the kernel, 32 channels per phase: every work-item loads the four pixels of one
+ *              (row, pair, 8 channels), forms the four differences in packed fp16 (bf16 is converted first: exact within the
+ *              fp16 range) and writes them; the next phase is transformed while the current one is multiplied.
+ *   B operand: U_p[i] comes straight from global memory (L2) in MFMA register layout, written that way by the weight
+ *              transform below: [phase][filter row][p][tile of 32 filters][16-channel slab][lane][16 bytes], one contiguous
+ *              kilobyte per wavefront load, requested two steps ahead.  No LDS, so no barrier inside a phase.
+ *   Epilogue : the planes go through LDS (two passes of 64 rows), a work-item folds four planes into two output pixels x 8
+ *              filters, applies bias / residual / ReLU and stores 16 bytes per pixel.
+ * Limits: 16-bit tensors, 3x3, stride 1, dilation 1, zero padding value, C = 64 or 128, K a multiple of 128, beta = 0,
+ * LINEAR or RELU, image rows of at most 256 pixels that tile into bands (see choose_band), values within the fp16 range.
+ */
+#include <atomic>
+
+#include "conv_epilogue.hpp"
+#include "mfma_core.hpp"
+
+/* Instrumentation, compiled in with -DWINOGRAD_ROWS_STAMPS only: work-item 0 of every workgroup records the 100 MHz wall clock at
+ * the phase boundaries of the kernel and avhip_debug_rows_stamps() copies the records of the last launch to the host. */
+#ifdef WINOGRAD_ROWS_STAMPS
+__device__ unsigned long long g_rows_stamps[4096 * 8];
+#define STAMP(i) do { if (threadIdx.x == 0) g_rows_stamps[(blockIdx.x % 4096) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+extern "C" __attribute__((visibility("default"))) int avhip_debug_rows_stamps(void *out)
+{
+	return static_cast<int>(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_rows_stamps), sizeof(g_rows_stamps)));
+}
+#else
+#define STAMP(i) do { } while (0)
+#endif
+
+namespace
+{
+	using namespace avhip;
+
+	constexpr int ROWS_MAX = 128; /* GEMM rows of a workgroup */
+	constexpr int PIXELS_MAX = 136; /* pixels of one V plane: (TH + 2) * pairs */
+	constexpr int POSITIONS = 4;
+	constexpr int FILTER_ROWS = 3;
+	constexpr int PHASE_CHANNELS = 32; /* channels transformed and multiplied per phase: two 16-channel MFMA slabs */
+	constexpr int PHASE_SLABS = 2;
+	constexpr int PITCH = 128 + 16; /* LDS bytes per pixel of a 64-channel slice */
+	constexpr int POSITION_BYTES = PIXELS_MAX * PITCH;
+	constexpr int SLICE_BYTES = POSITIONS * POSITION_BYTES;
+	constexpr int MAX_PHASES = 4;
+	constexpr int V_BYTES = (MAX_PHASES / 2) * SLICE_BYTES;
+	constexpr int ROWS_BLOCK_N = 128; /* filters per workgroup */
+	constexpr int THREADS = 512;
+	constexpr int OPERAND_BYTES = 1024; /* one MFMA operand of a wavefront: 64 lanes x 16 bytes */
+	/* epilogue: [plane][64 rows][128 filters + 4] floats */
+	constexpr int FOLD_ROWS = 64;
+	constexpr int FOLD_PITCH = ROWS_BLOCK_N + 4;
+	static_assert(POSITIONS * FOLD_ROWS * FOLD_PITCH * 4 <= V_BYTES, "the fold reuses the LDS of V");
+	static_assert(V_BYTES <= 160 * 1024, "LDS of a compute unit");
+
+	struct RowsGeom
+	{
+		int H, W, C, K, Ho, Wo, pad_h, pad_w;
+		int TH; /* output rows per band */
+		int pairs; /* column pairs per row: ceil(Wo / 2) */
+		unsigned int pairs_magic; /* 2^20 / pairs + 1: (v * magic) >> 20 == v / pairs for v < 1024 */
+		int bands; /* per image */
+		int images;
+		int filter_tiles; /* K / 32 */
+	};
+
+	typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+
+	__device__ __forceinline__ half8_t to_half8(uint4 raw, f16_t)
+	{
+		return __builtin_bit_cast(half8_t, raw);
+	}
+	__device__ __forceinline__ half8_t to_half8(uint4 raw, bf16_t)
+	{
+		const unsigned int w[4] = { raw.x, raw.y, raw.z, raw.w };
+		half8_t r;
+#pragma unroll
+		for (int i = 0; i < 4; i++)
+		{
+			r[2 * i] = static_cast<_Float16>(__uint_as_float(w[i] << 16));
+			r[2 * i + 1] = static_cast<_Float16>(__uint_as_float(w[i] & 0xFFFF0000u));
+		}
+		return r;
+	}
+
+	/* U in MFMA operand layout.  One work-item = one lane's 16 bytes of (phase, filter row, tile of 32 filters, slab), all
+	 * four positions. */
+	template<typename TE>
+	__global__ void k_rows_weight_transform(const TE *__restrict__ w, uint4 *__restrict__ U, int K, int C, int flip, int phases, int filter_tiles)
+	{
+		const int64_t e = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+		const int64_t total = static_cast<int64_t>(phases) * FILTER_ROWS * filter_tiles * PHASE_SLABS * 64;
+		if (e >= total)
+			return;
+		const int lane = static_cast<int>(e & 63);
+		int64_t t = e >> 6;
+		const int slab = static_cast<int>(t % PHASE_SLABS);
+		t /= PHASE_SLABS;
+		const int tile = static_cast<int>(t % filter_tiles);
+		t /= filter_tiles;
+		const int i = static_cast<int>(t % FILTER_ROWS);
+		const int phase = static_cast<int>(t / FILTER_ROWS);
+		const int k = tile * 32 + (lane & 31);
+		const int c0 = phase * PHASE_CHANNELS + slab * 16 + (lane >> 5) * 8;
+		float g[3][8];
+#pragma unroll
+		for (int j = 0; j < 3; j++)
+		{
+			const int wi = flip ? 2 - i : i, wj = flip ? 2 - j : j;
+#pragma unroll
+			for (int q = 0; q < 8; q++)
+				g[j][q] = (k < K && c0 + q < C) ? Traits<TE>::load(w[((static_cast<int64_t>(k) * 3 + wi) * 3 + wj) * C + c0 + q]) : 0.0f;
+		}
+		union
+		{
+			uint4 u;
+			_Float16 h[8];
+		} out[POSITIONS];
+#pragma unroll
+		for (int q = 0; q < 8; q++)
+		{
+			out[0].h[q] = static_cast<_Float16>(g[0][q]);
+			out[1].h[q] = static_cast<_Float16>(0.5f * (g[0][q] + g[1][q] + g[2][q]));
+			out[2].h[q] = static_cast<_Float16>(0.5f * (g[0][q] - g[1][q] + g[2][q]));
+			out[3].h[q] = static_cast<_Float16>(g[2][q]);
+		}
+#pragma unroll
+		for (int p = 0; p < POSITIONS; p++)
+			U[((((static_cast<int64_t>(phase) * FILTER_ROWS + i) * POSITIONS + p) * filter_tiles + tile) * PHASE_SLABS + slab) * 64 + lane] = out[p].u;
+	}
+
+	template<typename TE, int PHASES>
+	__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_winograd_rows(const TE *__restrict__ x, const void *__restrict__ U,
+			RowsGeom g, FloatEpilogue<TE> epi)
+	{
+		constexpr int STEPS = PHASES * FILTER_ROWS;
+		constexpr unsigned int SZ = sizeof(TE);
+		__shared__ __attribute__((aligned(16))) char lds[V_BYTES];
+		STAMP(0);
+		epi.pin();
+		keep_in_sgpr(g.pairs);
+		keep_in_sgpr(g.TH);
+		keep_in_sgpr(g.Ho);
+		keep_in_sgpr(g.Wo);
+		keep_in_sgpr(g.K);
+		const int tid = threadIdx.x;
+		const int lane = tid & 63;
+		const int wave = tid >> 6;
+		const int p = wave & 3; /* plane of this wavefront */
+		const int fh = wave >> 2; /* its half of the 128 filters */
+
+		int n = static_cast<int>(blockIdx.x), band = 0;
+		if (g.bands != 1)
+		{
+			n = static_cast<int>(blockIdx.x) / g.bands;
+			band = static_cast<int>(blockIdx.x) - n * g.bands;
+		}
+		const int kb = static_cast<int>(blockIdx.y);
+		const int oh0 = band * g.TH;
+		const int ih0 = oh0 + g.pad_h; /* input row of V row 0 */
+		const int v_rows = g.TH + 2;
+		int top = -ih0 < 0 ? 0 : -ih0; /* V rows above the image */
+		top = top > v_rows ? v_rows : top;
+		int bottom = ih0 + v_rows - g.H < 0 ? 0 : ih0 + v_rows - g.H; /* V rows below it */
+		bottom = bottom > v_rows - top ? v_rows - top : bottom;
+		const int real_rows = v_rows - top - bottom;
+
+		/* B operand: this wavefront's two filter tiles of step (phase, filter row) are 4 contiguous kilobytes */
+		const unsigned int step_stride = static_cast<unsigned int>(POSITIONS * g.filter_tiles * PHASE_SLABS * OPERAND_BYTES);
+		const __amdgpu_buffer_rsrc_t ru = make_buffer(U, static_cast<unsigned int>(STEPS) * step_stride);
+		const unsigned int b_offset = static_cast<unsigned int>((p * g.filter_tiles + kb * 4 + fh * 2) * PHASE_SLABS * OPERAND_BYTES + lane * 16);
+		Chunk bq[3][PHASE_SLABS][2];
+		auto load_b = [&](int step, Chunk (&set)[PHASE_SLABS][2]) __attribute__((always_inline))
+		{
+#pragma unroll
+			for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+				for (int sl = 0; sl < PHASE_SLABS; sl++)
+				{
+					const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(ru, static_cast<int>(b_offset + (tn * PHASE_SLABS + sl) * OPERAND_BYTES),
+							static_cast<int>(step * step_stride), 0);
+					set[sl][tn].u = make_uint4(v[0], v[1], v[2], v[3]);
+				}
+		};
+
+		/* transform side: this work-item's (row, pair, 8 channels) of every phase */
+		const __amdgpu_buffer_rsrc_t rx = make_buffer(x, static_cast<unsigned int>(g.images) * g.H * g.W * g.C * SZ);
+		const int t_chunk = tid & 3;
+		const int t_pixel = tid >> 2;
+		const int t_row = static_cast<int>((static_cast<unsigned int>(t_pixel) * g.pairs_magic) >> 20);
+		const int t_pair = t_pixel - t_row * g.pairs;
+		const bool t_valid = t_row < real_rows;
+		unsigned int x_src[4];
+		{
+			const int ih = ih0 + top + t_row;
+			const unsigned int line = (static_cast<unsigned int>(n) * g.H + static_cast<unsigned int>(ih)) * g.W;
+#pragma unroll
+			for (int j = 0; j < 4; j++)
+			{
+				const int iw = 2 * t_pair + g.pad_w + j;
+				const bool inside = t_valid & (static_cast<unsigned int>(iw) < static_cast<unsigned int>(g.W));
+				x_src[j] = inside ? ((line + static_cast<unsigned int>(iw)) * g.C + t_chunk * 8) * SZ : OUT_OF_RANGE;
+			}
+		}
+		const int v_dst = ((top + t_row) * g.pairs + t_pair) * PITCH + t_chunk * 16;
+		uint4 raw[4];
+		auto load_x = [&](int phase) __attribute__((always_inline))
+		{
+#pragma unroll
+			for (int j = 0; j < 4; j++)
+				raw[j] = buffer_fetch(rx, x_src[j] == OUT_OF_RANGE ? OUT_OF_RANGE : x_src[j] + static_cast<unsigned int>(phase * PHASE_CHANNELS) * SZ);
+		};
+		auto transform = [&](int phase) __attribute__((always_inline))
+		{
+			half8_t d[4];
+#pragma unroll
+			for (int j = 0; j < 4; j++)
+				d[j] = to_half8(raw[j], TE());
+			const half8_t v[POSITIONS] = { d[0] - d[2], d[1] + d[2], d[2] - d[1], d[1] - d[3] };
+			char *dst = lds + (phase >> 1) * SLICE_BYTES + (phase & 1) * 64 + v_dst;
+			if (t_valid)
+			{
+#pragma unroll
+				for (int q = 0; q < POSITIONS; q++)
+					*reinterpret_cast<half8_t*>(dst + q * POSITION_BYTES) = v[q];
+			}
+		};
+		load_x(0); /* what the first MFMA waits for longest goes out first */
+		load_b(0, bq[0]);
+		if (STEPS > 1)
+			load_b(1, bq[1]);
+
+		/* V rows outside the image are zeros, in every plane and slice: the rows above the image are the first `top * pairs`
+		 * pixels of a plane, the rows below it its last `bottom * pairs` */
+		{
+			const int above = top * g.pairs * 8, below = bottom * g.pairs * 8; /* 16-byte chunks per plane */
+			const int skip = real_rows * g.pairs * 8;
+			for (int plane = 0; plane < POSITIONS * ((PHASES + 1) / 2); plane++)
+				for (int e = tid; e < above + below; e += THREADS)
+				{
+					const int at = e < above ? e : e + skip;
+					*reinterpret_cast<uint4*>(lds + plane * POSITION_BYTES + (at >> 3) * PITCH + (at & 7) * 16) = make_uint4(0u, 0u, 0u, 0u);
+				}
+		}
+
+		/* per-filter constants of the epilogue: a work-item always stores the same 8 filters */
+		const int kcol = kb * ROWS_BLOCK_N + (tid & 15) * 8;
+		typename FloatEpilogue<TE>::template ColumnsT<8> columns;
+		epi.request_columns(kcol, columns);
+
+		/* MFMA operand addresses: lane l supplies GEMM row (l % 32) of a 32-row tile and the 8-channel half (l / 32) of a slab;
+		 * rows past the band read pixel 0 (their sums are never stored) */
+		int a_off[4];
+		const int band_rows = g.TH * g.pairs;
+#pragma unroll
+		for (int rt = 0; rt < 4; rt++)
+		{
+			const int q = rt * 32 + (lane & 31);
+			a_off[rt] = p * POSITION_BYTES + (q < band_rows ? q : 0) * PITCH + (lane >> 5) * 16;
+		}
+		const int tap_shift = g.pairs * PITCH;
+
+		STAMP(1);
+		transform(0);
+		if (PHASES > 1)
+			load_x(1);
+		__syncthreads();
+		STAMP(2);
+
+		typename Mma<f16_t>::acc_t acc[4][2];
+		Chunk a[2][4];
+		auto read_a = [&](int phase, int i, int sl, Chunk (&dst)[4]) __attribute__((always_inline))
+		{
+			const char *base = lds + (phase >> 1) * SLICE_BYTES + (phase & 1) * 64 + sl * 32 + i * tap_shift;
+#pragma unroll
+			for (int rt = 0; rt < 4; rt++)
+				dst[rt].u = *reinterpret_cast<const uint4*>(base + a_off[rt]);
+		};
+#pragma unroll
+		for (int phase = 0; phase < PHASES; phase++)
+		{
+#pragma unroll
+			for (int i = 0; i < FILTER_ROWS; i++)
+			{
+				const int step = phase * FILTER_ROWS + i;
+				if (step + 2 < STEPS)
+				{
+					/* two steps ahead and not a moment later: left to itself the scheduler sinks these requests to just before
+					 * their use, to shorten the life of their registers */
+					__builtin_amdgcn_sched_barrier(0);
+					load_b(step + 2, bq[(step + 2) % 3]);
+					__builtin_amdgcn_sched_barrier(0);
+				}
+				if (i == 0)
+					read_a(phase, 0, 0, a[(step * PHASE_SLABS) & 1]); /* behind the barrier of the phase: nothing could be read ahead */
+#pragma unroll
+				for (int sl = 0; sl < PHASE_SLABS; sl++)
+				{
+					const int s = step * PHASE_SLABS + sl;
+					if (sl + 1 < PHASE_SLABS)
+						read_a(phase, i, sl + 1, a[(s + 1) & 1]);
+					else if (i + 1 < FILTER_ROWS)
+						read_a(phase, i + 1, 0, a[(s + 1) & 1]);
+#pragma unroll
+					for (int rt = 0; rt < 4; rt++)
+#pragma unroll
+						for (int tn = 0; tn < 2; tn++)
+						{
+							/* filters as the rows of the MFMA tile, pixels as its columns: a lane then holds runs of four
+							 * consecutive filters of one pixel, which the fold can move as 16-byte vectors */
+							if (s == 0)
+								Mma<f16_t>::start(bq[step % 3][sl][tn], a[s & 1][rt], acc[rt][tn]);
+							else
+								Mma<f16_t>::run(bq[step % 3][sl][tn], a[s & 1][rt], acc[rt][tn]);
+						}
+				}
+				/* the next phase's V, from pixels requested a phase ago, while the matrix cores work on this one */
+				if (i == 1 && phase + 1 < PHASES)
+				{
+					transform(phase + 1);
+					if (phase + 2 < PHASES)
+					{
+						load_x(phase + 2);
+						__builtin_amdgcn_sched_barrier(0);
+					}
+				}
+			}
+			if (phase + 1 < PHASES)
+				__syncthreads();
+		}
+
+		STAMP(3);
+		/* fold and store: two passes of 64 GEMM rows; a work-item takes (row, 8 filters) twice per pass */
+		float *sm = reinterpret_cast<float*>(lds);
+		const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
+		__amdgpu_buffer_rsrc_t rz = make_buffer(nullptr, 0);
+		if (epi.z != nullptr)
+			rz = make_buffer(epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
+		const bool relu = epi.activation == ACT_RELU, has_z = epi.z != nullptr;
+#pragma unroll
+		for (int pass = 0; pass < 2; pass++)
+		{
+			/* where this work-item's two rows of the pass go, and their residual */
+			unsigned int y_off[2][2];
+			typename FloatEpilogue<TE>::template Residual<8> residual[2][2];
+#pragma unroll
+			for (int it = 0; it < 2; it++)
+			{
+				const int q = pass * FOLD_ROWS + (tid >> 4) + it * (THREADS / 16);
+				const int r = static_cast<int>((static_cast<unsigned int>(q) * g.pairs_magic) >> 20);
+				const int pair = q - r * g.pairs;
+				const int oh = oh0 + r;
+				const bool row_ok = (q < band_rows) & (oh < g.Ho) & (kcol < g.K);
+#pragma unroll
+				for (int o = 0; o < 2; o++)
+				{
+					const int ow = 2 * pair + o;
+					y_off[it][o] = (row_ok & (ow < g.Wo)) ? static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ : OUT_OF_RANGE;
+					union
+					{
+						uint4 u;
+						decltype(residual[0][0].raw) r8;
+					} cast;
+					cast.u = buffer_fetch<2>(rz, y_off[it][o]);
+					residual[it][o].raw = cast.r8;
+				}
+			}
+			__syncthreads(); /* pass 0: everyone is done with V; pass 1: with the planes of pass 0 */
+			/* A row of the fold buffer holds the 128 filters of a pixel as [first halves | second halves] of the 16 runs of 8
+			 * filters a work-item stores: run g, half h sits at word h * 64 + g * 4, so that sixteen lanes reading the same half of
+			 * sixteen runs touch 64 consecutive words (every bank once).  This lane's accumulator registers 4i..4i+3 are filters
+			 * fh * 64 + tn * 32 + 8i + 4 * (lane / 32) + 0..3 of pixel (lane % 32): run fh * 8 + tn * 4 + i, half (lane / 32). */
+			typedef float quad_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+			for (int rt = 0; rt < 2; rt++)
+#pragma unroll
+				for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+					for (int i = 0; i < 4; i++)
+					{
+						const typename Mma<f16_t>::acc_t &t = acc[pass * 2 + rt][tn];
+						const quad_t run = { t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3] };
+						*reinterpret_cast<quad_t*>(sm + (p * FOLD_ROWS + rt * 32 + (lane & 31)) * FOLD_PITCH + (lane >> 5) * 64 + (fh * 8 + tn * 4 + i) * 4) = run;
+					}
+			__syncthreads();
+			quad_t m[2][POSITIONS][2];
+#pragma unroll
+			for (int it = 0; it < 2; it++)
+#pragma unroll
+				for (int q = 0; q < POSITIONS; q++)
+#pragma unroll
+					for (int part = 0; part < 2; part++)
+						m[it][q][part] = *reinterpret_cast<const quad_t*>(sm + (q * FOLD_ROWS + (tid >> 4) + it * (THREADS / 16)) * FOLD_PITCH + part * 64 + (tid & 15) * 4);
+			auto leave = [&](auto with_relu, auto with_z) __attribute__((always_inline))
+			{
+#pragma unroll
+				for (int it = 0; it < 2; it++)
+				{
+					float out[2][8];
+#pragma unroll
+					for (int c = 0; c < 8; c++)
+					{
+						const float m0 = m[it][0][c >> 2][c & 3], m1 = m[it][1][c >> 2][c & 3], m2 = m[it][2][c >> 2][c & 3], m3 = m[it][3][c >> 2][c & 3];
+						out[0][c] = m0 + m1 + m2;
+						out[1][c] = m1 - m2 - m3;
+					}
+#pragma unroll
+					for (int o = 0; o < 2; o++)
+					{
+						const unsigned int offset = y_off[it][o];
+						epi.template store_fast<decltype(with_relu)::value, decltype(with_z)::value, 8>(out[o], columns, residual[it][o], [&](auto words) __attribute__((always_inline))
+						{
+							buffer_put<STORE_STREAM_THROUGH>(ry, offset, words);
+						});
+					}
+				}
+			};
+			if (relu && has_z)
+				leave(std::true_type(), std::true_type());
+			else if (relu)
+				leave(std::true_type(), std::false_type());
+			else if (has_z)
+				leave(std::false_type(), std::true_type());
+			else
+				leave(std::false_type(), std::false_type());
+		}
+		STAMP(4);
+	}
+
+	/* Rows per band: as many as fit 128 GEMM rows, the V plane and one transform item per work-item and phase
+	 * (rows inside the image x pairs <= 128).  0 when no band height does. */
+	int choose_band(const avhipConvShape &s, int pairs)
+	{
+		for (int th = s.Ho < ROWS_MAX ? s.Ho : ROWS_MAX; th >= 1; th--)
+		{
+			if (th * pairs > ROWS_MAX || (th + 2) * pairs > PIXELS_MAX)
+				continue;
+			bool fits = true;
+			for (int oh0 = 0; oh0 < s.Ho && fits; oh0 += th)
+			{
+				const int first = oh0 + s.pad_h, last = first + th + 2; /* input rows [first, last) */
+				const int lo = first < 0 ? 0 : first, hi = last > s.H ? s.H : last;
+				if (hi > lo && (hi - lo) * pairs > ROWS_MAX)
+					fits = false;
+			}
+			if (fits)
+				return th;
+		}
+		return 0;
+	}
+
+	template<typename TE>
+	int launch_rows(hipStream_t st, const avhipConvShape &s, const void *x, const void *U, const void *bias, const void *z, void *y, double alpha1,
+			double alpha2, int activation)
+	{
+		if ((s.C != 64 && s.C != 128) || s.K % ROWS_BLOCK_N != 0)
+			return AVHIP_NOT_SUPPORTED;
+		if (!aligned_to(x, 16) || !aligned_to(U, 16) || !aligned_to(y, 16) || (z != nullptr && !aligned_to(z, 16)) || (bias != nullptr && !aligned_to(bias, 16)))
+			return AVHIP_NOT_SUPPORTED;
+		if (static_cast<int64_t>(s.N) * s.H * s.W * s.C * sizeof(TE) >= (1ll << 31) || static_cast<int64_t>(s.Ho) * s.Wo * s.K * sizeof(TE) >= (1ll << 31))
+			return AVHIP_NOT_SUPPORTED;
+		const int pairs = (s.Wo + 1) / 2;
+		if (pairs > ROWS_MAX)
+			return AVHIP_NOT_SUPPORTED;
+		RowsGeom g;
+		g.TH = choose_band(s, pairs);
+		if (g.TH == 0)
+			return AVHIP_NOT_SUPPORTED;
+		g.H = s.H;
+		g.W = s.W;
+		g.C = s.C;
+		g.K = s.K;
+		g.Ho = s.Ho;
+		g.Wo = s.Wo;
+		g.pad_h = s.pad_h;
+		g.pad_w = s.pad_w;
+		g.pairs = pairs;
+		g.pairs_magic = (1u << 20) / static_cast<unsigned int>(pairs) + 1u;
+		g.bands = (s.Ho + g.TH - 1) / g.TH;
+		g.images = s.N;
+		g.filter_tiles = s.K / 32;
+		const int64_t items = static_cast<int64_t>(s.N) * g.bands;
+		if (items >= (1ll << 31) || s.K / ROWS_BLOCK_N > 65535)
+			return AVHIP_NOT_SUPPORTED;
+		const FloatEpilogue<TE> epi { static_cast<const float*>(bias), static_cast<const TE*>(z), static_cast<TE*>(y), static_cast<float>(alpha1),
+				static_cast<float>(alpha2), 0.0f, activation, s.K, true };
+		const dim3 grid(static_cast<unsigned int>(items), static_cast<unsigned int>(s.K / ROWS_BLOCK_N));
+		if (s.C == 128)
+			hipLaunchKernelGGL((k_winograd_rows<TE, 4>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+		else
+			hipLaunchKernelGGL((k_winograd_rows<TE, 2>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+		return 0;
+	}
+}
+
+namespace
+{
+	std::atomic<int> rows_mode { 1 };
+}
+extern "C" int avhip_set_winograd_rows(int mode)
+{
+	return mode < 0 ? rows_mode.load() : rows_mode.exchange(mode);
+}
+extern "C" int avhip_conv2d_winograd_rows_plan(int dtype, const avhipConvShape *shape, int *workgroups, int *rows_used)
+{
+	if (shape == nullptr)
+		return AVHIP_BAD_PARAM;
+	const avhipConvShape &s = *shape;
+	if (rows_mode.load() == 0 || (dtype != DT_FLOAT16 && dtype != DT_BFLOAT16))
+		return AVHIP_NOT_SUPPORTED;
+	if (s.R != 3 || s.S != 3 || s.stride_h != 1 || s.stride_w != 1 || s.dil_h != 1 || s.dil_w != 1 || (s.C != 64 && s.C != 128) || s.K % ROWS_BLOCK_N != 0
+			|| s.N <= 0 || s.Ho <= 0 || s.Wo <= 0)
+		return AVHIP_NOT_SUPPORTED;
+	const int pairs = (s.Wo + 1) / 2;
+	if (pairs > ROWS_MAX)
+		return AVHIP_NOT_SUPPORTED;
+	const int th = choose_band(s, pairs);
+	if (th == 0)
+		return AVHIP_NOT_SUPPORTED;
+	const int64_t groups = static_cast<int64_t>(s.N) * ((s.Ho + th - 1) / th) * (s.K / ROWS_BLOCK_N);
+	if (workgroups != nullptr)
+		workgroups[0] = groups > 0x7FFFFFFF ? 0x7FFFFFFF : static_cast<int>(groups);
+	if (rows_used != nullptr)
+		rows_used[0] = th * pairs;
+	return 0;
+}
+
+extern "C" int64_t avhip_winograd_rows_weight_bytes(int K, int C)
+{
+	if (K <= 0 || C <= 0)
+		return 0;
+	const int64_t phases = (C + PHASE_CHANNELS - 1) / PHASE_CHANNELS, tiles = (K + 31) / 32;
+	return phases * FILTER_ROWS * POSITIONS * tiles * PHASE_SLABS * OPERAND_BYTES;
+}
+
+extern "C" int avhip_winograd_rows_weight_transform(void *stream, int dtype, int invert, const void *w, void *U, int K, int C)
+{
+	if (w == nullptr || U == nullptr || K <= 0 || C <= 0)
+		return AVHIP_BAD_PARAM;
+	const int phases = (C + PHASE_CHANNELS - 1) / PHASE_CHANNELS, tiles = (K + 31) / 32;
+	const int64_t total = static_cast<int64_t>(phases) * FILTER_ROWS * tiles * PHASE_SLABS * 64;
+	const dim3 grid(ceil_div(total, 256));
+	hipStream_t st = static_cast<hipStream_t>(stream);
+	switch (dtype)
+	{
+		case DT_FLOAT16:
+			hipLaunchKernelGGL((k_rows_weight_transform<f16_t>), grid, dim3(256), 0, st, static_cast<const f16_t*>(w), static_cast<uint4*>(U), K, C, invert, phases, tiles);
+			return 0;
+		case DT_BFLOAT16:
+			hipLaunchKernelGGL((k_rows_weight_transform<bf16_t>), grid, dim3(256), 0, st, static_cast<const bf16_t*>(w), static_cast<uint4*>(U), K, C, invert, phases,
+					tiles);
+			return 0;
+		default:
+			return AVHIP_UNSUPPORTED_DATATYPE;
+	}
+}
+
+extern "C" int avhip_conv2d_winograd_rows(void *stream, int dtype, const avhipConvShape *shape, const void *x, const void *U, const void *bias, const void *z,
+		void *y, double alpha1, double alpha2, double beta, int activation)
+{
+	if (shape == nullptr || x == nullptr || U == nullptr || y == nullptr)
+		return AVHIP_BAD_PARAM;
+	const avhipConvShape &s = *shape;
+	if (s.N <= 0 || s.H <= 0 || s.W <= 0 || s.C <= 0 || s.K <= 0 || s.Ho <= 0 || s.Wo <= 0)
+		return AVHIP_BAD_PARAM;
+	if (s.R != 3 || s.S != 3 || s.stride_h != 1 || s.stride_w != 1 || s.dil_h != 1 || s.dil_w != 1 || beta != 0.0 || !is_simple_activation(activation))
+		return AVHIP_NOT_SUPPORTED;
+	hipStream_t st = static_cast<hipStream_t>(stream);
+	switch (dtype)
+	{
+		case DT_FLOAT16:
+			return launch_rows<f16_t>(st, s, x, U, bias, z, y, alpha1, alpha2, activation);
+		case DT_BFLOAT16:
+			return launch_rows<bf16_t>(st, s, x, U, bias, z, y, alpha1, alpha2, activation);
+		default:
+			return AVHIP_UNSUPPORTED_DATATYPE;
+	}
+}

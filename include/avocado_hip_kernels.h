@@ -93,6 +93,27 @@ extern "C"
 	AVHIP_API int avhip_conv2d_winograd_fused(void *stream, int dtype, const avhipConvShape *shape, const void *x, const void *U, const void *bias, const void *z,
 			void *y, double alpha1, double alpha2, double beta, int activation);
 
+	/* The same formula for 16-bit tensors by Winograd F(2,3) along image rows only, in one kernel (3x3, stride 1, dilation 1,
+	 * zero padding value, C = 64 or 128, K a multiple of 128, beta = 0, LINEAR or RELU; AVHIP_NOT_SUPPORTED otherwise, with
+	 * nothing launched).  The four planes of the transformed domain stay in accumulator registers for the whole k loop, so
+	 * the matrix cores do two thirds of the direct kernel's work and the output transform is paid once per output.  Stands
+	 * where the reference has its fused prototype, cuda_winogradFusedForward, src/winograd_fused.cu:789 (which transforms in
+	 * both directions).  U is what avhip_winograd_rows_weight_transform wrote: avhip_winograd_rows_weight_bytes(K, C) bytes
+	 * of fp16 in the register layout of the kernel's MFMA operand, [C / 32][3][4][K / 32][2][64 lanes][8]. */
+	AVHIP_API int avhip_conv2d_winograd_rows(void *stream, int dtype, const avhipConvShape *shape, const void *x, const void *U, const void *bias, const void *z,
+			void *y, double alpha1, double alpha2, double beta, int activation);
+	/* U_p[i] = sum_j G[p][j] * w[k, i, j] for the kernel above (taps reversed when `invert`), w of `dtype` (FLOAT16 / BFLOAT16).
+	 * Stands where the reference has kernel_winograd_weight_transform, src/winograd_nonfused.cu:257. */
+	AVHIP_API int avhip_winograd_rows_weight_transform(void *stream, int dtype, int invert, const void *w, void *U, int K, int C);
+	AVHIP_API int64_t avhip_winograd_rows_weight_bytes(int K, int C);
+	/* Whether avhip_conv2d_winograd_rows takes the layer (0) or not (AVHIP_NOT_SUPPORTED), the number of workgroups it would
+	 * launch and how many of a workgroup's 128 GEMM rows are output pixels pairs of the image: what a dispatcher weighs. */
+	AVHIP_API int avhip_conv2d_winograd_rows_plan(int dtype, const avhipConvShape *shape, int *workgroups, int *rows_used);
+	/* Tuning knob without a counterpart in the reference: 0 makes the plan above decline every layer (the dispatcher then uses
+	 * the direct kernels), 1 (default) lets the dispatcher weigh it, 2 makes the dispatcher take it for every layer it can run
+	 * (tests); a negative value changes nothing.  Returns the previous value. */
+	AVHIP_API int avhip_set_winograd_rows(int mode);
+
 	/* y = alpha1 * act(alpha2 * x + b + beta1 * z) + beta2 * z + beta3 * y.  Replaces kernel_add_bias,
 	 * src/tensor_op.cu:199-228.  x, y, z have `dtype`; b is fp32 (fp64 for fp64 tensors). */
 	AVHIP_API int avhip_add_bias(void *stream, int dtype, const void *x, const void *b, const void *z, void *y, int64_t first, int last, double alpha1,
