@@ -51,6 +51,10 @@ extern "C" __attribute__((visibility("default"))) int avhip_debug_rows_stamps(vo
 #define STAMP(i) do { } while (0)
 #endif
 
+#ifndef ROWS_STORE_POLICY
+#define ROWS_STORE_POLICY 17 /* sc0 sc1: written through as the kernel runs, no streaming hint */
+#endif
+
 namespace
 {
 	using namespace avhip;
@@ -62,7 +66,7 @@ namespace
 	constexpr int PHASE_CHANNELS = 32; /* channels transformed and multiplied per phase: two 16-channel MFMA slabs */
 	constexpr int PHASE_SLABS = 2;
 	constexpr int PITCH = 128 + 16; /* LDS bytes per pixel of a 64-channel slice */
-	constexpr int POSITION_BYTES = PIXELS_MAX * PITCH;
+	constexpr int POSITION_BYTES = (PIXELS_MAX + 1) * PITCH; /* one spare pixel behind every plane */
 	constexpr int SLICE_BYTES = POSITIONS * POSITION_BYTES;
 	constexpr int MAX_PHASES = 4;
 	constexpr int V_BYTES = (MAX_PHASES / 2) * SLICE_BYTES;
@@ -86,21 +90,35 @@ namespace
 		int filter_tiles; /* K / 32 */
 	};
 
-	typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-
-	__device__ __forceinline__ half8_t to_half8(uint4 raw, f16_t)
+	/* Eight fp16 values as four packed pairs: arithmetic on a pair is one packed instruction */
+	typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+	typedef float float2_t __attribute__((ext_vector_type(2)));
+	struct Half8
 	{
-		return __builtin_bit_cast(half8_t, raw);
+		half2_t h[4];
+	};
+	/* a - b on both halves with one instruction (the compiler takes a packed fp16 subtraction apart into two scalar ones and a
+	 * pack; a packed add with the negate modifiers on its second operand is the same operation) */
+	__device__ __forceinline__ half2_t pk_sub(half2_t a, half2_t b)
+	{
+		half2_t r;
+		asm("v_pk_add_f16 %0, %1, %2 neg_lo:[0,1] neg_hi:[0,1]" : "=v"(r) : "v"(a), "v"(b));
+		return r;
 	}
-	__device__ __forceinline__ half8_t to_half8(uint4 raw, bf16_t)
+	__device__ __forceinline__ Half8 to_half8(uint4 raw, f16_t)
+	{
+		return __builtin_bit_cast(Half8, raw);
+	}
+	/* bf16 -> fp16 through fp32, two values per conversion instruction (exact inside the fp16 range) */
+	__device__ __forceinline__ Half8 to_half8(uint4 raw, bf16_t)
 	{
 		const unsigned int w[4] = { raw.x, raw.y, raw.z, raw.w };
-		half8_t r;
+		Half8 r;
 #pragma unroll
 		for (int i = 0; i < 4; i++)
 		{
-			r[2 * i] = static_cast<_Float16>(__uint_as_float(w[i] << 16));
-			r[2 * i + 1] = static_cast<_Float16>(__uint_as_float(w[i] & 0xFFFF0000u));
+			const float2_t f = { __uint_as_float(w[i] << 16), __uint_as_float(w[i] & 0xFFFF0000u) };
+			r.h[i] = __builtin_convertvector(f, half2_t);
 		}
 		return r;
 	}
@@ -224,28 +242,39 @@ namespace
 				x_src[j] = inside ? ((line + static_cast<unsigned int>(iw)) * g.C + t_chunk * 8) * SZ : OUT_OF_RANGE;
 			}
 		}
-		const int v_dst = ((top + t_row) * g.pairs + t_pair) * PITCH + t_chunk * 16;
+		const int v_dst = (t_valid ? (top + t_row) * g.pairs + t_pair : PIXELS_MAX) * PITCH + t_chunk * 16;
 		uint4 raw[4];
 		auto load_x = [&](int phase) __attribute__((always_inline))
 		{
+			/* (an out-of-range offset stays out of range with the phase added: tensors here are below 2 GiB) */
 #pragma unroll
 			for (int j = 0; j < 4; j++)
-				raw[j] = buffer_fetch(rx, x_src[j] == OUT_OF_RANGE ? OUT_OF_RANGE : x_src[j] + static_cast<unsigned int>(phase * PHASE_CHANNELS) * SZ);
+			{
+				const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rx, static_cast<int>(x_src[j]), phase * PHASE_CHANNELS * static_cast<int>(SZ), 0);
+				raw[j] = make_uint4(v[0], v[1], v[2], v[3]);
+			}
 		};
+		/* B^T d for this work-item's pixels; work-items without a (row, pair) of the band write to a spare pixel, so that the
+		 * transform is straight-line code the scheduler can spread among the MFMAs */
 		auto transform = [&](int phase) __attribute__((always_inline))
 		{
-			half8_t d[4];
+			Half8 d[4];
 #pragma unroll
 			for (int j = 0; j < 4; j++)
 				d[j] = to_half8(raw[j], TE());
-			const half8_t v[POSITIONS] = { d[0] - d[2], d[1] + d[2], d[2] - d[1], d[1] - d[3] };
-			char *dst = lds + (phase >> 1) * SLICE_BYTES + (phase & 1) * 64 + v_dst;
-			if (t_valid)
-			{
+			Half8 v[POSITIONS];
 #pragma unroll
-				for (int q = 0; q < POSITIONS; q++)
-					*reinterpret_cast<half8_t*>(dst + q * POSITION_BYTES) = v[q];
+			for (int q = 0; q < 4; q++)
+			{
+				v[0].h[q] = pk_sub(d[0].h[q], d[2].h[q]);
+				v[1].h[q] = d[1].h[q] + d[2].h[q];
+				v[2].h[q] = pk_sub(d[2].h[q], d[1].h[q]);
+				v[3].h[q] = pk_sub(d[1].h[q], d[3].h[q]);
 			}
+			char *dst = lds + (phase >> 1) * SLICE_BYTES + (phase & 1) * 64 + v_dst;
+#pragma unroll
+			for (int q = 0; q < POSITIONS; q++)
+				*reinterpret_cast<uint4*>(dst + q * POSITION_BYTES) = __builtin_bit_cast(uint4, v[q]);
 		};
 		load_x(0); /* what the first MFMA waits for longest goes out first */
 		load_b(0, bq[0]);
@@ -315,6 +344,10 @@ namespace
 				}
 				if (i == 0)
 					read_a(phase, 0, 0, a[(step * PHASE_SLABS) & 1]); /* behind the barrier of the phase: nothing could be read ahead */
+				/* the next phase's V, from pixels requested a phase ago, spread among the MFMAs of this step */
+				const bool transform_here = i == FILTER_ROWS - 1 && phase + 1 < PHASES;
+				if (transform_here)
+					transform(phase + 1);
 #pragma unroll
 				for (int sl = 0; sl < PHASE_SLABS; sl++)
 				{
@@ -336,10 +369,16 @@ namespace
 								Mma<f16_t>::run(bq[step % 3][sl][tn], a[s & 1][rt], acc[rt][tn]);
 						}
 				}
-				/* the next phase's V, from pixels requested a phase ago, while the matrix cores work on this one */
-				if (i == 1 && phase + 1 < PHASES)
+				if (transform_here)
 				{
-					transform(phase + 1);
+					/* four vector instructions of the transform behind every MFMA: they issue while the matrix pipeline works */
+#pragma unroll
+					for (int k = 0; k < 4 * 2 * PHASE_SLABS; k++)
+					{
+						__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+						__builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+					}
+					__builtin_amdgcn_sched_barrier(0);
 					if (phase + 2 < PHASES)
 					{
 						load_x(phase + 2);
@@ -388,11 +427,12 @@ namespace
 				}
 			}
 			__syncthreads(); /* pass 0: everyone is done with V; pass 1: with the planes of pass 0 */
+			typedef float quad_t __attribute__((ext_vector_type(4)));
+#ifndef ROWS_KNOCK_LDS
 			/* A row of the fold buffer holds the 128 filters of a pixel as [first halves | second halves] of the 16 runs of 8
 			 * filters a work-item stores: run g, half h sits at word h * 64 + g * 4, so that sixteen lanes reading the same half of
 			 * sixteen runs touch 64 consecutive words (every bank once).  This lane's accumulator registers 4i..4i+3 are filters
 			 * fh * 64 + tn * 32 + 8i + 4 * (lane / 32) + 0..3 of pixel (lane % 32): run fh * 8 + tn * 4 + i, half (lane / 32). */
-			typedef float quad_t __attribute__((ext_vector_type(4)));
 #pragma unroll
 			for (int rt = 0; rt < 2; rt++)
 #pragma unroll
@@ -405,6 +445,7 @@ namespace
 						*reinterpret_cast<quad_t*>(sm + (p * FOLD_ROWS + rt * 32 + (lane & 31)) * FOLD_PITCH + (lane >> 5) * 64 + (fh * 8 + tn * 4 + i) * 4) = run;
 					}
 			__syncthreads();
+#endif
 			quad_t m[2][POSITIONS][2];
 #pragma unroll
 			for (int it = 0; it < 2; it++)
@@ -412,7 +453,14 @@ namespace
 				for (int q = 0; q < POSITIONS; q++)
 #pragma unroll
 					for (int part = 0; part < 2; part++)
+#ifndef ROWS_KNOCK_LDS
 						m[it][q][part] = *reinterpret_cast<const quad_t*>(sm + (q * FOLD_ROWS + (tid >> 4) + it * (THREADS / 16)) * FOLD_PITCH + part * 64 + (tid & 15) * 4);
+#else
+					{
+						const typename Mma<f16_t>::acc_t &t = acc[pass * 2 + it][part];
+						m[it][q][part] = quad_t { t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3] };
+					}
+#endif
 			auto leave = [&](auto with_relu, auto with_z) __attribute__((always_inline))
 			{
 #pragma unroll
@@ -432,7 +480,12 @@ namespace
 						const unsigned int offset = y_off[it][o];
 						epi.template store_fast<decltype(with_relu)::value, decltype(with_z)::value, 8>(out[o], columns, residual[it][o], [&](auto words) __attribute__((always_inline))
 						{
-							buffer_put<STORE_STREAM_THROUGH>(ry, offset, words);
+#ifndef ROWS_KNOCK_STORES
+							buffer_put<ROWS_STORE_POLICY>(ry, offset, words);
+#else
+							if (offset == 12345u)
+								buffer_put<STORE_STREAM_THROUGH>(ry, offset, words);
+#endif
 						});
 					}
 				}

@@ -158,7 +158,10 @@ namespace avhip
 	 * a store at OUT_OF_RANGE is dropped by the hardware, so "this row does not exist" needs no branch around the store. */
 	typedef __attribute__((__vector_size__(2 * sizeof(unsigned int)))) unsigned int u32x2_t;
 	constexpr int STORE_STREAM = 2; /* nt */
-	constexpr int STORE_STREAM_THROUGH = 19; /* sc0 sc1 nt: written through to memory as it goes; measured 1-3 % faster than nt alone in
+#ifndef AVHIP_STREAM_THROUGH_POLICY
+#define AVHIP_STREAM_THROUGH_POLICY 19
+#endif
+	constexpr int STORE_STREAM_THROUGH = AVHIP_STREAM_THROUGH_POLICY; /* sc0 sc1 nt: written through to memory as it goes; measured 1-3 % faster than nt alone in
 	                                          * the 3x3 tile kernel and the persistent 1x1 / GEMM kernels */
 	template<int POLICY = STORE_STREAM>
 	__device__ inline void buffer_put(__amdgpu_buffer_rsrc_t rsrc, unsigned int byte_offset, unsigned int __attribute__((ext_vector_type(4))) words)
