@@ -9,7 +9,7 @@ the context's stream and by device synchronisation.
 
 Prints ONE JSON line.  `value` is direct-convolution-equivalent TFLOP/s (2*N*Ho*Wo*K*C*R*S per convolution) of the whole tower
 in the headline dtype (bf16).  `roofline` is for the dominant kernel (the 128->128 body convolution), its duration measured
-with HIP events around each of its launches inside the timed region.  `cpu_baseline` is the restated CPU direct convolution
+with HIP events over the timed region ((pass - stem) / 20); `ms_per_step` is the median of five timings of `--steps` passes each.  `cpu_baseline` is the restated CPU direct convolution
 (oracle/cpu_baseline.c, "port") timed on the host cores on a batch slice of the same body convolution.  `detail` carries the
 other dtypes and the per-stage figures of the non-fused Winograd path.
 """
@@ -110,6 +110,12 @@ class Hip:
         self.rt.hipEventDestroy(e1)
         return ms / replays
 
+    def time_graph_groups(self, exe, stream, replays, warmup=2, groups=5):
+        """`groups` timings of `replays` replays each, every one between its own pair of events on an idle stream.  Returns the
+        per-replay durations of the groups, sorted: one group of 20 passes is 7-9 ms and the clocks of a box drift by several
+        per cent over such spans, so a single sample would carry that drift straight into the reported figure."""
+        return sorted(self.time_graph(exe, stream, replays, warmup if g == 0 else 1) for g in range(groups))
+
 
 def conv_flops(N, Ho, Wo, K, Cin, R, S):
     return 2.0 * N * Ho * Wo * K * Cin * R * S
@@ -195,7 +201,8 @@ def time_tower(hip, ctx, dtype, steps, warmup, check=True):
     full = hip.capture(stream, lambda: final.append(tower.step()))
     stem = hip.capture(stream, lambda: [tower.stem() for _ in range(10)])
     hip.sync()
-    ms_step = hip.time_graph(full, stream, steps, warmup)
+    groups = hip.time_graph_groups(full, stream, steps, warmup)  # five timings of exactly `steps` passes each
+    ms_step = groups[len(groups) // 2]
     ctx.synchronize()
     checked = self_check(tower, final[0]) if check else {"checked": False}  # what the timed replays left behind, against the CPU oracle
     t0 = time.perf_counter()
@@ -203,15 +210,24 @@ def time_tower(hip, ctx, dtype, steps, warmup, check=True):
         tower.step()  # the same pass as 21 eager calls: launch and host cost of the API included
     ctx.synchronize()
     ms_eager = (time.perf_counter() - t0) * 1e3 / steps
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        tower.step()
-    host_us_per_call = (time.perf_counter() - t0) * 1e6 / (steps * (1 + 2 * tower.blocks))  # enqueue only: the stream runs behind
+    # host time of one call (descriptor checks, dispatch, launch) on an idle stream: a loop that only enqueues soon runs into the
+    # back-pressure of the queue and then measures the kernels, not the host
+    host = []
+
+    def one_call_at_a_time(layer, x, z, y):
+        host.append(time.perf_counter())
+        ctx.synchronize()
+        host.append(time.perf_counter())
+    host.append(time.perf_counter())
+    tower.step(after=one_call_at_a_time)
+    calls = 1 + 2 * tower.blocks
+    host_us_per_call = sorted((host[2 * i + 1] - host[2 * i]) * 1e6 for i in range(calls))[calls // 2]
     ctx.synchronize()
-    ms_stem = hip.time_graph(stem, stream, max(steps, 10), warmup) / 10
+    ms_stem = hip.time_graph_groups(stem, stream, max(steps, 10), warmup, groups=3)[1] / 10
     ctx.synchronize()
     body_us = (ms_step - ms_stem) * 1e3 / (2 * tower.blocks)
-    out = {"ms_per_step": ms_step, "tflops": tower.flops_step / (ms_step * 1e-3) / 1e12, "stem_conv_us": ms_stem * 1e3,
+    out = {"ms_per_step": ms_step, "ms_per_step_groups": {"timings": len(groups), "passes_each": steps, "min": groups[0], "max": groups[-1]},
+           "tflops": tower.flops_step / (ms_step * 1e-3) / 1e12, "stem_conv_us": ms_stem * 1e3,
            "body_conv_us": body_us, "body_conv_tflops": tower.flops_body / (body_us * 1e-6) / 1e12, "workspace_bytes": tower.workspace_bytes,
            "ms_per_step_eager_calls": ms_eager, "host_us_per_call": host_us_per_call, "self_check": checked}
     hip.rt.hipGraphExecDestroy(full)
@@ -626,7 +642,9 @@ def main():
         "config": {"workload": "BASELINE config 2: residual tower N=256 15x15 128ch, stem 4->128 + 10 blocks (21 3x3 convs), NHWC, bias+ReLU+residual fused",
                    "global_batch": 256, "entry": "cudaConvolutionBiasActivationForward"},
         "roofline": {"bound": "mfma", "achieved": head["body_conv_tflops"], "peak": peak, "unit": "TFLOP/s", "frac": head["body_conv_tflops"] / peak,
-                     "traffic": COUNTED_TRAFFIC_BYTES.get(args.dtype), "kernel": "body 3x3 conv 128->128: direct-equivalent flops / ((graph-replayed pass - stem) / 20) by HIP events"},
+                     "traffic": COUNTED_TRAFFIC_BYTES.get(args.dtype),
+                     "kernel": "body 3x3 conv 128->128 (k_winograd_rows for 16-bit tensors: F(2,3) along rows, 12.885 GFLOP issued to the matrix cores "
+                               "for the 16.987 GFLOP of the direct form): direct-equivalent flops / ((graph-replayed pass - stem) / 20) by HIP events"},
         "cpu_baseline": cpu,
         "detail": detail,
     }

@@ -342,12 +342,16 @@ namespace
 					load_b(step + 2, bq[(step + 2) % 3]);
 					__builtin_amdgcn_sched_barrier(0);
 				}
-				if (i == 0)
-					read_a(phase, 0, 0, a[(step * PHASE_SLABS) & 1]); /* behind the barrier of the phase: nothing could be read ahead */
-				/* the next phase's V, from pixels requested a phase ago, spread among the MFMAs of this step */
-				const bool transform_here = i == FILTER_ROWS - 1 && phase + 1 < PHASES;
+				if (step == 0)
+					read_a(0, 0, 0, a[0]); /* behind the first barrier: nothing could be read ahead */
+				/* The next phase's V, from pixels requested a phase ago, is formed among the MFMAs of the middle step and made
+				 * visible by a barrier before the last one, so that the last step can read the first operands of the next phase
+				 * ahead like any other: no phase starts with a barrier and a bare LDS latency. */
+				const bool transform_here = i == 1 && phase + 1 < PHASES;
 				if (transform_here)
 					transform(phase + 1);
+				if (i == 2 && phase + 1 < PHASES)
+					__syncthreads();
 #pragma unroll
 				for (int sl = 0; sl < PHASE_SLABS; sl++)
 				{
@@ -356,6 +360,8 @@ namespace
 						read_a(phase, i, sl + 1, a[(s + 1) & 1]);
 					else if (i + 1 < FILTER_ROWS)
 						read_a(phase, i + 1, 0, a[(s + 1) & 1]);
+					else if (phase + 1 < PHASES)
+						read_a(phase + 1, 0, 0, a[(s + 1) & 1]);
 #pragma unroll
 					for (int rt = 0; rt < 4; rt++)
 #pragma unroll
@@ -386,8 +392,6 @@ namespace
 					}
 				}
 			}
-			if (phase + 1 < PHASES)
-				__syncthreads();
 		}
 
 		STAMP(3);
@@ -398,12 +402,11 @@ namespace
 		if (epi.z != nullptr)
 			rz = make_buffer(epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
 		const bool relu = epi.activation == ACT_RELU, has_z = epi.z != nullptr;
+		/* where this work-item's two rows of either pass go, and their residual, requested before the planes go through LDS */
+		unsigned int y_off[2][2][2];
+		typename FloatEpilogue<TE>::template Residual<8> residual[2][2][2];
 #pragma unroll
 		for (int pass = 0; pass < 2; pass++)
-		{
-			/* where this work-item's two rows of the pass go, and their residual */
-			unsigned int y_off[2][2];
-			typename FloatEpilogue<TE>::template Residual<8> residual[2][2];
 #pragma unroll
 			for (int it = 0; it < 2; it++)
 			{
@@ -416,16 +419,19 @@ namespace
 				for (int o = 0; o < 2; o++)
 				{
 					const int ow = 2 * pair + o;
-					y_off[it][o] = (row_ok & (ow < g.Wo)) ? static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ : OUT_OF_RANGE;
+					y_off[pass][it][o] = (row_ok & (ow < g.Wo)) ? static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ : OUT_OF_RANGE;
 					union
 					{
 						uint4 u;
-						decltype(residual[0][0].raw) r8;
+						decltype(residual[0][0][0].raw) r8;
 					} cast;
-					cast.u = buffer_fetch<2>(rz, y_off[it][o]);
-					residual[it][o].raw = cast.r8;
+					cast.u = buffer_fetch<2>(rz, y_off[pass][it][o]);
+					residual[pass][it][o].raw = cast.r8;
 				}
 			}
+#pragma unroll
+		for (int pass = 0; pass < 2; pass++)
+		{
 			__syncthreads(); /* pass 0: everyone is done with V; pass 1: with the planes of pass 0 */
 			typedef float quad_t __attribute__((ext_vector_type(4)));
 #ifndef ROWS_KNOCK_LDS
@@ -477,8 +483,8 @@ namespace
 #pragma unroll
 					for (int o = 0; o < 2; o++)
 					{
-						const unsigned int offset = y_off[it][o];
-						epi.template store_fast<decltype(with_relu)::value, decltype(with_z)::value, 8>(out[o], columns, residual[it][o], [&](auto words) __attribute__((always_inline))
+						const unsigned int offset = y_off[pass][it][o];
+						epi.template store_fast<decltype(with_relu)::value, decltype(with_z)::value, 8>(out[o], columns, residual[pass][it][o], [&](auto words) __attribute__((always_inline))
 						{
 #ifndef ROWS_KNOCK_STORES
 							buffer_put<ROWS_STORE_POLICY>(ry, offset, words);
