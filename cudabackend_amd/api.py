@@ -84,6 +84,8 @@ PROTOTYPES = {
     "avhipGetMemoryPointer": (i32, [i64, C.POINTER(vp)]),
     "avhipInvalidateCaches": (i32, []),
     "avhipGetWeightCacheState": (i32, [C.POINTER(i64), C.POINTER(i64), C.POINTER(i64)]),
+    "avhipSetWeightCacheBudget": (i32, [i64, C.POINTER(i64)]),
+    "avhipWeightCachePolicyProbe": (i32, [i32, C.POINTER(i64), C.POINTER(i64), C.POINTER(i32), i64, i64, C.POINTER(i32)]),
 }
 # the thin kernel layer of include/avocado_hip_kernels.h (exported, bound only for the symbol check)
 KERNEL_LAYER_SYMBOLS = ["avhip_winograd_weight_transform", "avhip_winograd_input_transform", "avhip_winograd_output_transform",

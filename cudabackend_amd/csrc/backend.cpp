@@ -61,29 +61,55 @@ namespace
 		hipStream_t stream = nullptr;
 		bool is_default = false;
 	};
-	/* The last writes to an owning block through the API: write number v covers bytes [lo, hi) and sits in slot v % LOG. */
+	/* The byte ranges of an owning block written through the API, each with the number of its last write.  A write of a
+	 * range that is already listed renews that entry (an arena that holds weights, activations and workspace sees the same few
+	 * ranges over and over: every layer of a network writes one of two or three activation buffers), a new range takes the slot
+	 * of the range written longest ago, and `lost` remembers the newest write whose range was dropped that way. */
 	struct WriteLog
 	{
 		static constexpr int LOG = 64;
 		std::mutex mutex;
 		uint64_t version = 0; /* number of writes so far */
+		uint64_t lost = 0; /* writes up to this number may have left the log */
+		int used = 0;
 		av_int64 lo[LOG], hi[LOG];
+		uint64_t when[LOG];
 		void record(av_int64 first, av_int64 last)
 		{
 			std::lock_guard<std::mutex> lock(mutex);
 			version++;
-			lo[version % LOG] = first;
-			hi[version % LOG] = last;
+			int oldest = 0;
+			for (int i = 0; i < used; i++)
+			{
+				if (lo[i] == first && last == hi[i])
+				{
+					when[i] = version;
+					return;
+				}
+				if (when[i] < when[oldest])
+					oldest = i;
+			}
+			int slot = used;
+			if (used < LOG)
+				used++;
+			else
+			{
+				slot = oldest;
+				lost = std::max(lost, when[slot]);
+			}
+			lo[slot] = first;
+			hi[slot] = last;
+			when[slot] = version;
 		}
 		/* Whether bytes [first, last) were written after write number `seen`; `seen` moves up to the current number when not.
 		 * Writes that have left the log count as hits. */
 		bool written_since(uint64_t &seen, av_int64 first, av_int64 last)
 		{
 			std::lock_guard<std::mutex> lock(mutex);
-			if (version - seen > static_cast<uint64_t>(LOG))
+			if (seen < lost)
 				return true;
-			for (uint64_t v = seen + 1; v <= version; v++)
-				if (lo[v % LOG] < last && first < hi[v % LOG])
+			for (int i = 0; i < used; i++)
+				if (when[i] > seen && lo[i] < last && first < hi[i])
 					return true;
 			seen = version;
 			return false;
@@ -439,7 +465,12 @@ namespace
 	 *    reading them also orders the rewrite of the matrices, and a captured graph that holds the buffer's address keeps
 	 *    reading valid memory.  Nothing is freed on that path.
 	 *  - Buffers are freed only by avhipInvalidateCaches, by the destruction of the weight block, or when the cache outgrows
-	 *    its budget at the insertion of a new tensor, then after a device synchronisation and outside the cache's mutex.
+	 *    its budget at the insertion of a new tensor, then after a synchronisation of the entry's device and outside the
+	 *    cache's mutex.  The budget never takes an entry that a capturing stream was handed (a graph holds its address and may
+	 *    be replayed at any time: such entries are pinned until avhipInvalidateCaches or the destruction of the weight block,
+	 *    which are the two events that invalidate graphs) nor one that a caller was handed and has not yet enqueued its
+	 *    kernel for (the lease returned with the matrices counts those; the device synchronisation only covers kernels that
+	 *    are already enqueued).
 	 *  - A stream that is capturing never changes the cache: no allocation, no transform, no event.  It may use an entry that
 	 *    is up to date and whose transform ran on the same stream or is known to be complete; otherwise the lookup reports
 	 *    AVOCADO_STATUS_BAD_ALLOC ("cannot allocate here": call once outside capture first) and the dispatcher takes the
@@ -466,10 +497,12 @@ namespace
 		bool complete = false; /* the event has been seen complete */
 		uint64_t seen = 0; /* write number of the weight block the matrices are known to be current for */
 		uint64_t last_use = 0;
+		bool pinned = false; /* handed to a capturing stream: a graph holds the address */
+		int in_use = 0; /* callers that hold the address and have not enqueued their kernel yet */
 	};
 	struct WeightCache
 	{
-		static constexpr size_t BUDGET = static_cast<size_t>(4) << 30; /* bytes of matrices kept before the least recently used go */
+		size_t budget = static_cast<size_t>(4) << 30; /* bytes of matrices kept before the least recently used go */
 		std::mutex mutex;
 		std::map<WeightKey, WeightEntry> entries;
 		size_t total = 0;
@@ -479,14 +512,25 @@ namespace
 		{
 			if (victims.empty())
 				return;
-			/* kernels on any stream may still read the matrices */
-			(void) hipDeviceSynchronize();
+			/* Kernels already enqueued on any stream of an entry's device may still read its matrices: that device is
+			 * synchronised before the buffer goes.  Another thread may be capturing a stream in the global mode, under which
+			 * a synchronisation or a free from any thread would break its capture: this thread says that it knows. */
+			int previous_device = 0;
+			(void) hipGetDevice(&previous_device);
+			hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+			(void) hipThreadExchangeStreamCaptureMode(&mode);
 			for (WeightEntry &e : victims)
 			{
+				if (e.U == nullptr)
+					continue; /* (entries of the policy probe own nothing) */
 				(void) hipSetDevice(e.device);
+				(void) hipDeviceSynchronize();
 				(void) hipFree(e.U);
 				(void) hipEventDestroy(e.ready);
 			}
+			(void) hipSetDevice(previous_device);
+			(void) hipThreadExchangeStreamCaptureMode(&mode);
+			(void) hipGetLastError();
 			victims.clear();
 		}
 		void clear()
@@ -518,15 +562,18 @@ namespace
 			}
 			release(victims);
 		}
-		/* with the mutex held: moves least recently used entries out until `incoming` more bytes fit the budget */
+		/* with the mutex held: moves least recently used entries out until `incoming` more bytes fit the budget; entries that
+		 * a graph or a caller still holds stay, whatever the budget says */
 		void make_room(size_t incoming, std::vector<WeightEntry> &victims)
 		{
-			while (!entries.empty() && total + incoming > BUDGET)
+			while (total + incoming > budget)
 			{
-				auto oldest = entries.begin();
+				auto oldest = entries.end();
 				for (auto it = entries.begin(); it != entries.end(); ++it)
-					if (it->second.last_use < oldest->second.last_use)
+					if (!it->second.pinned && it->second.in_use == 0 && (oldest == entries.end() || it->second.last_use < oldest->second.last_use))
 						oldest = it;
+				if (oldest == entries.end())
+					break;
 				victims.push_back(oldest->second);
 				total -= oldest->second.bytes;
 				entries.erase(oldest);
@@ -556,9 +603,38 @@ namespace
 		return status != hipStreamCaptureStatusNone;
 	}
 
+	/* Held by a caller from the lookup of transformed weights until its kernel is enqueued: keeps the budget from freeing the
+	 * matrices in between. */
+	struct WeightLease
+	{
+		WeightKey key;
+		bool held = false;
+		WeightLease() = default;
+		WeightLease(const WeightLease&) = delete;
+		WeightLease& operator=(const WeightLease&) = delete;
+		void take(const WeightKey &k, WeightEntry &e)
+		{
+			key = k;
+			held = true;
+			e.in_use++;
+		}
+		~WeightLease()
+		{
+			if (!held)
+				return;
+			WeightCache &cache = weight_cache();
+			std::lock_guard<std::mutex> lock(cache.mutex);
+			auto it = cache.entries.find(key);
+			if (it != cache.entries.end() && it->second.in_use > 0)
+				it->second.in_use--;
+		}
+	};
+
 	/* Returns the [t*t, K, C] Winograd weight matrices F(m x m, 3x3) of a weight tensor in `mat_dtype`, (re)transforming on the
-	 * context's stream when the cache has none or the weight bytes were written since. */
-	avStatus_t cached_winograd_weights(const Context &ctx, const ConvProblem &p, avMemoryDescriptor_t wMem, int m, avDataType_t mat_dtype, const void **U)
+	 * context's stream when the cache has none or the weight bytes were written since.  The caller keeps `lease` alive until
+	 * the kernel that reads the matrices is enqueued. */
+	avStatus_t cached_winograd_weights(const Context &ctx, const ConvProblem &p, avMemoryDescriptor_t wMem, int m, avDataType_t mat_dtype, const void **U,
+			WeightLease &lease)
 	{
 		Memory *wm = get_memory(wMem);
 		Memory *owner = owner_of(wm);
@@ -583,17 +659,27 @@ namespace
 				WeightEntry &e = it->second;
 				e.last_use = ++cache.clock;
 				U[0] = e.U;
+				const bool capturing = !e.pinned && is_capturing(ctx.stream); /* (a pinned entry need not ask again) */
 				if (e.complete || e.stream == ctx.stream)
-					return AVOCADO_STATUS_SUCCESS; /* stream order, or nothing left to wait for */
-				if (is_capturing(ctx.stream))
+				{
+					/* stream order, or nothing left to wait for.  Under capture the graph keeps the address: pinned from now on */
+					e.pinned = e.pinned || capturing;
+					lease.take(key, e);
+					return AVOCADO_STATUS_SUCCESS;
+				}
+				if (capturing || (e.pinned && is_capturing(ctx.stream)))
 					return AVOCADO_STATUS_BAD_ALLOC; /* an event from outside must not enter the capture */
 				if (hipEventQuery(e.ready) == hipSuccess)
 				{
 					e.complete = true;
+					lease.take(key, e);
 					return AVOCADO_STATUS_SUCCESS;
 				}
 				(void) hipGetLastError(); /* hipErrorNotReady is not an error here */
-				return from_hip(hipStreamWaitEvent(ctx.stream, e.ready, 0));
+				const avStatus_t waiting = from_hip(hipStreamWaitEvent(ctx.stream, e.ready, 0));
+				if (waiting == AVOCADO_STATUS_SUCCESS)
+					lease.take(key, e);
+				return waiting;
 			}
 			if (is_capturing(ctx.stream))
 				return AVOCADO_STATUS_BAD_ALLOC;
@@ -637,6 +723,7 @@ namespace
 					e.complete = false;
 					e.last_use = ++cache.clock;
 					U[0] = e.U;
+					lease.take(key, e);
 				}
 				else
 				{
@@ -651,10 +738,10 @@ namespace
 		return status;
 	}
 	/* [16, K, C] for the fused kernel: fp16 matrices for 16-bit tensors, fp32 for fp32 */
-	avStatus_t fused_weights(const Context &ctx, const ConvProblem &p, avMemoryDescriptor_t wMem, const void **U)
+	avStatus_t fused_weights(const Context &ctx, const ConvProblem &p, avMemoryDescriptor_t wMem, const void **U, WeightLease &lease)
 	{
 		const avDataType_t mat_dtype = (p.w_dtype == AVOCADO_DTYPE_FLOAT32) ? AVOCADO_DTYPE_FLOAT32 : AVOCADO_DTYPE_FLOAT16;
-		return cached_winograd_weights(ctx, p, wMem, 2, mat_dtype, U);
+		return cached_winograd_weights(ctx, p, wMem, 2, mat_dtype, U, lease);
 	}
 
 	bool winograd_supported(int r, int m)
@@ -838,7 +925,8 @@ namespace
 		if (c.bias != nullptr && c.bias_dtype != AVOCADO_DTYPE_FLOAT32)
 			return AVOCADO_STATUS_UNSUPPORTED_DATATYPE;
 		const void *U = nullptr;
-		const avStatus_t st = fused_weights(c.ctx, p, wMem, &U);
+		WeightLease lease;
+		const avStatus_t st = fused_weights(c.ctx, p, wMem, &U, lease);
 		if (st != AVOCADO_STATUS_SUCCESS)
 			return st;
 		touch(yMem);
@@ -866,7 +954,8 @@ namespace
 	{
 		const ConvProblem &p = c.problem;
 		const void *U = nullptr;
-		const avStatus_t st = cached_winograd_weights(c.ctx, p, wMem, 1, AVOCADO_DTYPE_FLOAT16, &U);
+		WeightLease lease;
+		const avStatus_t st = cached_winograd_weights(c.ctx, p, wMem, 1, AVOCADO_DTYPE_FLOAT16, &U, lease);
 		if (st != AVOCADO_STATUS_SUCCESS)
 			return st;
 		const int rc = avhip_conv2d_winograd_rows(c.ctx.stream, p.x_dtype, &p.shape, c.x->data, U, c.bias, c.z, c.y->data, c.alpha1, c.alpha2, c.beta,
@@ -916,7 +1005,8 @@ namespace
 		char *V = ws->data, *Mx = V + plan.v_bytes;
 		void *st = c.ctx.stream;
 		const void *U = nullptr;
-		const avStatus_t ws_status = cached_winograd_weights(c.ctx, c.problem, wMem, 4, plan.mat_dtype, &U);
+		WeightLease lease;
+		const avStatus_t ws_status = cached_winograd_weights(c.ctx, c.problem, wMem, 4, plan.mat_dtype, &U, lease);
 		if (ws_status != AVOCADO_STATUS_SUCCESS)
 			return ws_status;
 		touch(wsMem, 0, plan.total);
@@ -1974,6 +2064,40 @@ namespace avocado
 			if (hipDeviceSynchronize() != hipSuccess)
 				return AVOCADO_STATUS_EXECUTION_FAILED;
 			weight_cache().clear();
+			return AVOCADO_STATUS_SUCCESS;
+		}
+		avStatus_t avhipSetWeightCacheBudget(av_int64 bytes, av_int64 *previous)
+		{
+			if (bytes < 0)
+				return AVOCADO_STATUS_BAD_PARAM;
+			WeightCache &cache = weight_cache();
+			std::lock_guard<std::mutex> lock(cache.mutex);
+			if (previous != nullptr)
+				previous[0] = static_cast<av_int64>(cache.budget);
+			cache.budget = static_cast<size_t>(bytes);
+			return AVOCADO_STATUS_SUCCESS;
+		}
+		avStatus_t avhipWeightCachePolicyProbe(int count, const av_int64 *bytes, const av_int64 *last_use, const int *flags, av_int64 budget, av_int64 incoming,
+				int *evicted)
+		{
+			if (count < 0 || bytes == nullptr || last_use == nullptr || flags == nullptr || evicted == nullptr || budget < 0 || incoming < 0)
+				return AVOCADO_STATUS_BAD_PARAM;
+			WeightCache model; /* the same object the library keeps, filled with entries that own nothing */
+			model.budget = static_cast<size_t>(budget);
+			for (int i = 0; i < count; i++)
+			{
+				WeightEntry e;
+				e.bytes = static_cast<size_t>(bytes[i]);
+				e.last_use = static_cast<uint64_t>(last_use[i]);
+				e.pinned = (flags[i] & 1) != 0;
+				e.in_use = (flags[i] & 2) != 0 ? 1 : 0;
+				model.entries.emplace(WeightKey { static_cast<uint64_t>(i), 0, 0, 0, 0, 0, 0 }, e);
+				model.total += e.bytes;
+			}
+			std::vector<WeightEntry> victims;
+			model.make_room(static_cast<size_t>(incoming), victims);
+			for (int i = 0; i < count; i++)
+				evicted[i] = model.entries.count(WeightKey { static_cast<uint64_t>(i), 0, 0, 0, 0, 0, 0 }) == 0 ? 1 : 0;
 			return AVOCADO_STATUS_SUCCESS;
 		}
 		avStatus_t avhipGetWeightCacheState(av_int64 *entries, av_int64 *bytes, av_int64 *transforms)

@@ -161,6 +161,16 @@ namespace avhip
 		else
 			asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" : : "v"(dst), "v"(value) : "memory");
 	}
+	/* The same written through without the streaming hint ("sc0 sc1") */
+	template<typename V>
+	__device__ __forceinline__ void store_through_plain(V *dst, const V &value)
+	{
+		static_assert(sizeof(V) == 8 || sizeof(V) == 16, "one dwordx2 or dwordx4 store");
+		if constexpr (sizeof(V) == 8)
+			asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" : : "v"(dst), "v"(value) : "memory");
+		else
+			asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" : : "v"(dst), "v"(value) : "memory");
+	}
 
 	/* Makes a wavefront-uniform 32-bit value live in a scalar register from here on.  Kernel arguments sit in memory and the
 	 * compiler is free to re-load them wherever they are used; in fully unrolled epilogues that puts a scalar load and a

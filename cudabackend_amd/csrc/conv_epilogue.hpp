@@ -502,7 +502,7 @@ namespace avhip
 						if constexpr (sizeof(words_t) >= 8)
 						{
 							if (through)
-								store_through(reinterpret_cast<words_t*>(dst), o.w);
+								store_through_plain(reinterpret_cast<words_t*>(dst), o.w); /* (13.4-13.6 us on config 4 against 13.8 with the streaming hint as well) */
 							else
 								*reinterpret_cast<words_t*>(dst) = o.w;
 						}

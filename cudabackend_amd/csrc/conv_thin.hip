@@ -25,7 +25,9 @@
 #include "mfma_core.hpp"
 #include "persistent_gemm.hpp"
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
+#include <vector>
 
 /* Instrumentation, compiled in with -DCONV_THIN_STAMPS only: work-item 0 of every workgroup records the 100 MHz wall clock at
  * the phase boundaries of the kernel (start, first requests out, set-up done, and for its last item: first slab, last slab,
@@ -471,6 +473,38 @@ namespace
 	}
 }
 
+namespace
+{
+	/* Whether `kernel` may be launched with up to THIN_LDS bytes of dynamic LDS on the current device: asked of the runtime once
+	 * per kernel instance and device, remembered afterwards. */
+	bool large_lds_allowed(const void *kernel)
+	{
+		struct Answer
+		{
+			const void *kernel;
+			int device;
+			bool allowed;
+		};
+		static std::mutex mutex;
+		static std::vector<Answer> answers;
+		int device = 0;
+		if (hipGetDevice(&device) != hipSuccess)
+		{
+			(void) hipGetLastError();
+			return false;
+		}
+		std::lock_guard<std::mutex> lock(mutex);
+		for (const Answer &a : answers)
+			if (a.kernel == kernel && a.device == device)
+				return a.allowed;
+		const bool allowed = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, THIN_LDS) == hipSuccess;
+		if (!allowed)
+			(void) hipGetLastError();
+		answers.push_back({ kernel, device, allowed });
+		return allowed;
+	}
+}
+
 namespace avhip
 {
 	template<typename TE, typename Epi>
@@ -576,9 +610,11 @@ namespace avhip
 		 * work items */
 		const unsigned int resident = persistent_workgroups(1 << 30) / (lds_bytes > 80u * 1024u ? 2 : 1);
 		const dim3 grid(std::min(g.items, resident));
+		/* more than 64 KB of dynamic LDS needs the kernel's say-so, given once per instance and device; where that fails nothing
+		 * is launched and the caller's other kernels take the layer */
 #define AVHIP_THIN(PB) \
-		if (lds_bytes > 64u * 1024u) \
-			(void)hipFuncSetAttribute(reinterpret_cast<const void*>(&k_conv_thin<TE, PB, Epi>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)); \
+		if (lds_bytes > 64u * 1024u && !large_lds_allowed(reinterpret_cast<const void*>(&k_conv_thin<TE, PB, Epi>))) \
+			return false; \
 		hipLaunchKernelGGL((k_conv_thin<TE, PB, Epi>), grid, dim3(256), lds_bytes, stream, static_cast<const TE*>(x), static_cast<const TE*>(w), g, epi)
 		switch (pb)
 		{

@@ -233,7 +233,8 @@ namespace avocado
 			 * calling stream, when the weight bytes were written through this API since.  What callers must know:
 			 *  - writes the library cannot see (through the raw address, or by a replayed graph): call avhipInvalidateCaches
 			 *    afterwards.  It synchronises the device and frees every buffer, so no captured graph that contains a Winograd
-			 *    call may be replayed after it; capture again.
+			 *    call may be replayed after it; capture again.  The same holds after the weight block of such a call is destroyed.
+			 *    Nothing else frees a buffer that a graph holds (see avhipSetWeightCacheBudget).
 			 *  - under stream capture the library neither allocates nor transforms: a Winograd entry whose weights are not cached
 			 *    and up to date returns AVOCADO_STATUS_BAD_ALLOC without launching anything (run the call once outside capture,
 			 *    or use the NoAlloc entry); the dispatcher takes its implicit-GEMM plan instead.
@@ -242,6 +243,18 @@ namespace avocado
 			 * (any pointer may be null). */
 			DLL_PUBLIC avStatus_t avhipInvalidateCaches(void);
 			DLL_PUBLIC avStatus_t avhipGetWeightCacheState(av_int64 *entries, av_int64 *bytes, av_int64 *transforms);
+			/* The cache keeps at most `bytes` of matrices (default 4 GiB): inserting a new tensor beyond that frees the least
+			 * recently used buffers first, except those a captured graph holds (a buffer handed to a capturing stream stays until
+			 * avhipInvalidateCaches or the destruction of its weight block: only those two invalidate graphs) and those a call on
+			 * another thread has looked up and not yet launched its kernel for.  `previous`, when not null, receives the old limit.
+			 * No counterpart in the reference, which has no such cache. */
+			DLL_PUBLIC avStatus_t avhipSetWeightCacheBudget(av_int64 bytes, av_int64 *previous);
+			/* The eviction rule of that cache applied to a made-up set of `count` buffers, without touching a device: buffer i has
+			 * bytes[i] bytes, was last used at time last_use[i] and carries flags[i] (1: held by a graph, 2: looked up by a call
+			 * that has not launched yet).  evicted[i] is set to 1 for every buffer the rule frees to make room for `incoming` more
+			 * bytes under `budget`, 0 otherwise.  For host-side tests of the policy. */
+			DLL_PUBLIC avStatus_t avhipWeightCachePolicyProbe(int count, const av_int64 *bytes, const av_int64 *last_use, const int *flags, av_int64 budget,
+					av_int64 incoming, int *evicted);
 
 #ifdef __cplusplus
 		} /* extern "C" */

@@ -642,3 +642,46 @@ def test_split_k_through_the_dispatcher(oracle, tiling, dtype, case):
     split = h.conv_forward("dispatch", x, w, ys, dtype, bias=b, **kw)
     assert oracle.rel_l2(split, plain) < BAR[dtype] * (3 if dtype == "f32" else 1)
     assert oracle.rel_l2(split, oracle.conv2d(x, w, b, **kw)) < BAR[dtype] * (3 if dtype == "f32" else 1)
+
+
+class _Shape(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("N", "H", "W", "C", "K", "R", "S", "Ho", "Wo", "pad_h", "pad_w", "stride_h", "stride_w", "dil_h", "dil_w",
+                                       "mode")]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("case", SPLIT_CASES, ids=[str(i) for i in range(len(SPLIT_CASES))])
+def test_split_k_kernel_layer_entry(oracle, tiling, dtype, case):
+    """avhip_conv2d_implicit_gemm_split_k called directly: it must TAKE every one of these layers (return 0: the two split kernels ran,
+    which the dispatcher test cannot tell from its fallback), and decline a workspace that is short or not aligned with nothing launched."""
+    if tiling != "workgroup_tiles":
+        pytest.skip("with the one-wavefront-per-tile kernel available the plan leaves layers this small to it")
+    lib = cb.load_library()
+    g = h.rng(44)
+    x = h.rounded(oracle, g.standard_normal(case["x"]), dtype)
+    w = he(g, case["w"], dtype, oracle)
+    ys = out_shape(oracle, case)
+    b = g.uniform(-0.1, 0.1, ys[3]).astype(np.float32).astype(np.float64)
+    z = h.rounded(oracle, g.standard_normal(ys), dtype)
+    kw = dict(pad=case["pad"], stride=case.get("stride", (1, 1)), dilation=case.get("dilation", (1, 1)), mode=case.get("mode", 0))
+    xs, ws = case["x"], case["w"]
+    s = _Shape(xs[0], xs[1], xs[2], xs[3], ws[0], ws[1], ws[2], ys[1], ys[2], kw["pad"][0], kw["pad"][1], kw["stride"][0], kw["stride"][1],
+               kw["dilation"][0], kw["dilation"][1], kw["mode"])
+    need = C.c_int64(0)
+    assert lib.avhip_conv2d_split_k_workspace(h.DT[dtype], C.byref(s), C.byref(need)) == 0
+    assert need.value >= 2 * 4 * ys[0] * ys[1] * ys[2] * ys[3], "partial sums of at least two parts"
+    lib.avhip_conv2d_implicit_gemm_split_k.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                                       C.c_double, C.c_double, C.c_double, C.c_int, C.c_void_p, C.c_int64]
+    with h.Call() as c:
+        xt, wt, zt, bt = c.tensor(x, dtype), c.tensor(w, dtype), c.tensor(z, dtype), c.tensor(b, "f32")
+        y = c.empty(ys, dtype)
+        space = c.empty((need.value + 256,), cb.DTYPE_UINT8)
+        stream = C.c_void_p(c.ctx.stream())
+        args = (stream, h.DT[dtype], C.addressof(s), xt.pointer(), wt.pointer(), bt.pointer(), zt.pointer(), y.pointer(), None, 1.0, 0.7, 0.0, cb.ACTIVATION_RELU)
+        assert lib.avhip_conv2d_implicit_gemm_split_k(*args, space.pointer(), need.value) == 0
+        c.finish()
+        got = y.download()
+        assert lib.avhip_conv2d_implicit_gemm_split_k(*args, space.pointer(), need.value - 1) == -1, "short workspace"
+        assert lib.avhip_conv2d_implicit_gemm_split_k(*args, space.pointer() + 4, need.value) == -1, "workspace not aligned for 16-byte accesses"
+    want = oracle.conv2d(x, w, b, z, alpha2=float(np.float32(0.7)), activation=oracle.RELU, **kw)
+    assert oracle.rel_l2(got, want) < BAR[dtype] * (3 if dtype == "f32" else 1)

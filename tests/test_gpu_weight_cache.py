@@ -133,10 +133,20 @@ def test_weights_in_an_arena_survive_writes_elsewhere_in_it(oracle):
         cb.check(lib.cudaCopyMemoryFromHost(ctx.handle, arena.value, int(offs[0]), raw.ctypes.data, raw.nbytes), "upload through the owner")
         assert oracle.rel_l2(run(), oracle.conv2d(x2, w, b, activation=oracle.RELU)) < TOL
         assert _state(lib)[2] == t0 + 3
-        # more writes elsewhere than the write log holds: the lookup turns conservative (transforms again), results stay right
-        for _ in range(70):
+        # many more writes of the same few ranges than the write log has slots (what a deep network does to an arena: every layer
+        # writes one of two or three activation buffers): a range that is written again renews its slot, the weights stay cached
+        for i in range(200):
             upload(xv, x2)
+            upload(yv, want)
         assert oracle.rel_l2(run(), oracle.conv2d(x2, w, b, activation=oracle.RELU)) < TOL
+        assert _state(lib)[2] == t0 + 3, "repeated writes of the same ranges must not push the weight's history out of the log"
+        # more DISTINCT ranges written elsewhere than the log holds: the lookup turns conservative (transforms again), results stay right
+        piece = np.ascontiguousarray(x2.reshape(-1)[:4], dtype=np.float32)
+        for i in range(70):
+            cb.check(lib.cudaCopyMemoryFromHost(ctx.handle, xv, 16 * i, piece.ctypes.data, piece.nbytes), "upload of a piece")
+        x3 = x2.copy()
+        x3.reshape(-1)[:4 * 70] = np.tile(piece.astype(np.float64), 70)
+        assert oracle.rel_l2(run(), oracle.conv2d(x3, w, b, activation=oracle.RELU)) < TOL
         assert _state(lib)[2] == t0 + 4
     for v in views:
         lib.cudaDestroyMemoryDescriptor(v)
@@ -219,4 +229,43 @@ def test_capture_with_a_cold_cache_allocates_nothing(oracle):
         hip.rt.hipGraphExecDestroy(exe)
         ws.close()
     for t in (xt, wt, bt, y):
+        t.close()
+
+
+def test_budget_never_frees_what_a_graph_holds(oracle):
+    """With a budget that every insertion exceeds, the cache frees the least recently used matrices, but never those a captured graph
+    was handed: the graph replays on valid memory after other weight tensors have gone through the cache."""
+    lib = cb.load_library()
+    hip = bench.Hip()
+    cb.check(lib.avhipInvalidateCaches(), "avhipInvalidateCaches")
+    previous = C.c_int64(0)
+    cb.check(lib.avhipSetWeightCacheBudget(1, C.byref(previous)), "avhipSetWeightCacheBudget")
+    g = h.rng(95)
+    x, w, b = _problem(oracle, g)
+    want = oracle.conv2d(x, w, b, activation=oracle.RELU)
+    conv = cb.ConvolutionDescriptor(padding=(-1, -1))
+    xt, wt, bt = cb.DeviceTensor.from_numpy(x, cb.DTYPE_FLOAT32), cb.DeviceTensor.from_numpy(w, cb.DTYPE_FLOAT32), cb.DeviceTensor.from_numpy(b, cb.DTYPE_FLOAT32)
+    y = cb.DeviceTensor(want.shape, cb.DTYPE_FLOAT32)
+    others = [cb.DeviceTensor.from_numpy(oracle.round_to(g.standard_normal(w.shape) * 0.05, "f32"), cb.DTYPE_FLOAT32) for _ in range(3)]
+    y2 = cb.DeviceTensor(want.shape, cb.DTYPE_FLOAT32)
+    try:
+        with cb.Context(0) as ctx:
+            _fused(lib, ctx, conv, xt, wt, bt, y)  # warm: the matrices of w are in the cache
+            ctx.synchronize()
+            assert _state(lib)[0] == 1
+            exe = hip.capture(ctx.stream(), lambda: _fused(lib, ctx, conv, xt, wt, bt, y))
+            per_entry = _state(lib)[1]
+            for i, other in enumerate(others):  # every insertion is over the budget: the previous `other` goes, the graph's entry stays
+                _fused(lib, ctx, conv, xt, other, bt, y2)
+                ctx.synchronize()
+                assert _state(lib)[:2] == (2, 2 * per_entry), "one pinned entry and the newest one"
+            cb.check(lib.cudaSetMemory(ctx.handle, y.mem, 0, y.nbytes, None, 0), "clear y")
+            hip.launch(exe, ctx.stream())
+            ctx.synchronize()
+            assert oracle.rel_l2(y.download(), want) < TOL
+            hip.rt.hipGraphExecDestroy(exe)
+    finally:
+        cb.check(lib.avhipSetWeightCacheBudget(previous.value, None), "avhipSetWeightCacheBudget")
+        cb.check(lib.avhipInvalidateCaches(), "avhipInvalidateCaches")
+    for t in [xt, wt, bt, y, y2] + others:
         t.close()

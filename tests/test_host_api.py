@@ -228,3 +228,31 @@ def test_split_k_plan_is_for_few_pixels_and_a_long_k():
     out = C.c_int64(0)
     assert lib.avhip_conv2d_split_k_workspace(bf16, C.byref(s), C.byref(out)) != 0      # N = 0
     assert lib.avhip_conv2d_split_k_workspace(bf16, None, C.byref(out)) != 0
+
+
+def test_weight_cache_eviction_policy():
+    """The rule by which the cache of transformed weights makes room, on made-up buffers (no device involved): least recently used
+    first, never a buffer that a captured graph holds (flag 1) or that a call has looked up and not yet launched for (flag 2), and no
+    more than needed."""
+    import ctypes as C
+    lib = cb.load_library()
+
+    def probe(sizes, last_use, flags, budget, incoming):
+        n = len(sizes)
+        evicted = (C.c_int32 * n)()
+        st = lib.avhipWeightCachePolicyProbe(n, (C.c_int64 * n)(*sizes), (C.c_int64 * n)(*last_use), (C.c_int32 * n)(*flags), budget, incoming, evicted)
+        assert st == cb.STATUS_SUCCESS
+        return list(evicted)
+    # everything fits: nothing goes
+    assert probe([10, 10, 10], [1, 2, 3], [0, 0, 0], 100, 10) == [0, 0, 0]
+    # 10 more bytes need one buffer gone: the one used longest ago
+    assert probe([10, 10, 10], [5, 2, 9], [0, 0, 0], 30, 10) == [0, 1, 0]
+    # 25 more need all three
+    assert probe([10, 10, 10], [5, 2, 9], [0, 0, 0], 30, 25) == [1, 1, 1]
+    # the oldest is held by a graph, the next by a call in flight: the third goes although it is the most recent, and then the rule stops
+    assert probe([10, 10, 10], [1, 2, 9], [1, 2, 0], 30, 25) == [0, 0, 1]
+    # nothing can go: the rule leaves everything (the cache then exceeds its budget rather than free memory in use)
+    assert probe([10, 10], [1, 2], [1, 3], 5, 100) == [0, 0]
+    # a budget of zero empties the cache of what is free to go
+    assert probe([10, 10, 10, 10], [4, 3, 2, 1], [0, 1, 0, 2], 0, 0) == [1, 0, 1, 0]
+    assert lib.avhipWeightCachePolicyProbe(1, None, None, None, 1, 1, None) == cb.STATUS_BAD_PARAM
