@@ -344,7 +344,7 @@ def int8_leg(hip, ctx, iters):
     return out
 
 
-def nonfused_stages(hip, ctx, dtype, mat_dtype, m, iters, shape=(256, 15, 128), acc_dtype="f32"):
+def nonfused_stages(hip, ctx, dtype, mat_dtype, m, iters, shape=(256, 15, 128), acc_dtype="f32", rates=None):
     """The four-call non-fused Winograd sequence F(m x m, 3x3) on one layer, one timing per stage.  shape = (N, H = W, C = K):
     the body convolution of config 2 by default, (64, 56, 256) for config 3.  mat_dtype: U and V, acc_dtype: M.
     Algorithmic bytes per stage: input x + V; GEMM V + U + M; output M + y + bias (weight transform w + U).  The GEMM stage is
@@ -377,6 +377,8 @@ def nonfused_stages(hip, ctx, dtype, mat_dtype, m, iters, shape=(256, 15, 128), 
     alg_bytes = {"weight_transform": ch * 9 * ch * esz + t * t * ch * ch * msz, "input_transform": xbytes + t * t * tiles * ch * msz,
                  "gemm": t * t * tiles * ch * msz + t * t * ch * ch * msz + t * t * tiles * ch * asz,
                  "output_transform": t * t * tiles * ch * asz + xbytes + 4 * ch}
+    written = {"weight_transform": t * t * ch * ch * msz, "input_transform": t * t * tiles * ch * msz, "gemm": t * t * tiles * ch * asz,
+               "output_transform": xbytes}
     gemm_flops = 2.0 * t * t * tiles * ch * ch
     out = {"shape": {"N": N, "HW": HW, "channels": ch, "tiles": tiles}, "matrices": mat_dtype, "M": acc_dtype}
     total = 0.0
@@ -384,6 +386,11 @@ def nonfused_stages(hip, ctx, dtype, mat_dtype, m, iters, shape=(256, 15, 128), 
         ms = time_calls(hip, ctx, fn, iters)
         rec = {"us": ms * 1e3, "MB": alg_bytes[name] / 1e6, "GBs": alg_bytes[name] / (ms * 1e-3) / 1e9,
                "hbm_frac": alg_bytes[name] / (ms * 1e-3) / 1e9 / PEAK["hbm_GBs"]}
+        if rates is not None:
+            # the time a kernel that streams the same bytes at the read-only and write-only rates measured on this box in this run
+            # (avhip_stream_probe, 1 GiB) would take, reads and writes one after the other, over the stage's time
+            floor_ms = ((alg_bytes[name] - written[name]) / rates["read"] + written[name] / rates["write"]) / 1e6
+            rec["frac_of_measured_stream_rates"] = floor_ms / ms
         if name == "gemm":
             rec["gflop"] = gemm_flops / 1e9
             rec["tflops"] = gemm_flops / (ms * 1e-3) / 1e12
@@ -615,20 +622,20 @@ def main():
                 detail["tower_" + other] = time_tower(hip, ctx, other, max(3, args.steps // 2), 2, check=not args.no_cpu)
         detail["caller_level_two_chains_of_128"] = two_half_batch_chains(hip, args.dtype, args.steps)
         detail["int8_config4"] = int8_leg(hip, ctx, it)
-        detail["nonfused_winograd_f32_F4"] = nonfused_stages(hip, ctx, "f32", "f32", 4, it)
-        detail["nonfused_winograd_bf16_F2_fp16mat"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it)
-        detail["nonfused_winograd_f16_F2_fp16mat_fp16M"] = nonfused_stages(hip, ctx, "f16", "f16", 2, it, acc_dtype="f16")
-        detail["nonfused_winograd_bf16_F2_fp16mat_fp16M"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it, acc_dtype="f16")
+        detail["copy_GBs_measured"] = copy_bandwidth(hip, ctx)
+        rates = detail["stream_GBs_measured"] = stream_rates(hip, ctx)
+        detail["nonfused_winograd_f32_F4"] = nonfused_stages(hip, ctx, "f32", "f32", 4, it, rates=rates)
+        detail["nonfused_winograd_bf16_F2_fp16mat"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it, rates=rates)
+        detail["nonfused_winograd_f16_F2_fp16mat_fp16M"] = nonfused_stages(hip, ctx, "f16", "f16", 2, it, acc_dtype="f16", rates=rates)
+        detail["nonfused_winograd_bf16_F2_fp16mat_fp16M"] = nonfused_stages(hip, ctx, "bf16", "f16", 2, it, acc_dtype="f16", rates=rates)
         cfg3 = (64, 56, 256)
         detail["config3_nonfused_winograd"] = {
-            "bf16_F2_fp16mat": nonfused_stages(hip, ctx, "bf16", "f16", 2, it, shape=cfg3),
-            "f16_F2_fp16mat_fp16M": nonfused_stages(hip, ctx, "f16", "f16", 2, it, shape=cfg3, acc_dtype="f16"),
-            "bf16_F2_fp16mat_fp16M": nonfused_stages(hip, ctx, "bf16", "f16", 2, it, shape=cfg3, acc_dtype="f16"),
-            "bf16_F4_fp32mat": nonfused_stages(hip, ctx, "bf16", "f32", 4, it, shape=cfg3),
-            "f16_F4_fp32mat": nonfused_stages(hip, ctx, "f16", "f32", 4, it, shape=cfg3),
+            "bf16_F2_fp16mat": nonfused_stages(hip, ctx, "bf16", "f16", 2, it, shape=cfg3, rates=rates),
+            "f16_F2_fp16mat_fp16M": nonfused_stages(hip, ctx, "f16", "f16", 2, it, shape=cfg3, acc_dtype="f16", rates=rates),
+            "bf16_F2_fp16mat_fp16M": nonfused_stages(hip, ctx, "bf16", "f16", 2, it, shape=cfg3, acc_dtype="f16", rates=rates),
+            "bf16_F4_fp32mat": nonfused_stages(hip, ctx, "bf16", "f32", 4, it, shape=cfg3, rates=rates),
+            "f16_F4_fp32mat": nonfused_stages(hip, ctx, "f16", "f32", 4, it, shape=cfg3, rates=rates),
         }
-        detail["copy_GBs_measured"] = copy_bandwidth(hip, ctx)
-        detail["stream_GBs_measured"] = stream_rates(hip, ctx)
         detail["mfma_rate_measured"] = mfma_rates(hip, ctx)
         detail["other_configs"] = other_configs(hip, ctx, it)
         detail["first_layers_beyond_baseline"] = other_configs(hip, ctx, it, FIRST_LAYERS)
