@@ -69,7 +69,8 @@ namespace
 	constexpr int POSITION_BYTES = (PIXELS_MAX + 1) * PITCH; /* one spare pixel behind every plane */
 	constexpr int SLICE_BYTES = POSITIONS * POSITION_BYTES;
 	constexpr int MAX_PHASES = 4;
-	constexpr int V_BYTES = (MAX_PHASES / 2) * SLICE_BYTES;
+	constexpr int V_SLACK = 8 * PITCH; /* what an MFMA row past the tile's last may read behind the last plane */
+	constexpr int V_BYTES = (MAX_PHASES / 2) * SLICE_BYTES + V_SLACK;
 	constexpr int ROWS_BLOCK_N = 128; /* filters per workgroup */
 	constexpr int THREADS = 512;
 	constexpr int OPERAND_BYTES = 1024; /* one MFMA operand of a wavefront: 64 lanes x 16 bytes */
@@ -82,10 +83,10 @@ namespace
 	struct RowsGeom
 	{
 		int H, W, C, K, Ho, Wo, pad_h, pad_w;
-		int TH; /* output rows per band */
-		int pairs; /* column pairs per row: ceil(Wo / 2) */
+		int TH; /* output rows of a tile */
+		int pairs; /* column pairs of a tile: a tile is TH rows by 2 * pairs output pixels */
 		unsigned int pairs_magic; /* 2^20 / pairs + 1: (v * magic) >> 20 == v / pairs for v < 1024 */
-		int bands; /* per image */
+		int bands, segments; /* tiles down and across an image */
 		int images;
 		int filter_tiles; /* K / 32 */
 	};
@@ -175,6 +176,10 @@ namespace
 	{
 		constexpr int STEPS = PHASES * FILTER_ROWS;
 		constexpr unsigned int SZ = sizeof(TE);
+		/* V of four phases (128 channels) fits LDS; layers with more channels reuse the slot of phase - 4.  Phase ph + 1 is written
+		 * during the middle step of phase ph, by wavefronts that have passed the barrier of phase ph - 1, which nobody reaches
+		 * before it is done with phase ph - 2: the slot's last readers (phase ph - 3) are long gone. */
+		constexpr int RING = MAX_PHASES;
 		__shared__ __attribute__((aligned(16))) char lds[V_BYTES];
 		STAMP(0);
 		epi.pin();
@@ -189,14 +194,19 @@ namespace
 		const int p = wave & 3; /* plane of this wavefront */
 		const int fh = wave >> 2; /* its half of the 128 filters */
 
-		int n = static_cast<int>(blockIdx.x), band = 0;
-		if (g.bands != 1)
+		/* (image, band, segment): the tiles of an image are neighbours in the grid; the filter block is the slow index */
+		int n = static_cast<int>(blockIdx.x), band = 0, segment = 0;
+		if (g.bands * g.segments != 1)
 		{
-			n = static_cast<int>(blockIdx.x) / g.bands;
-			band = static_cast<int>(blockIdx.x) - n * g.bands;
+			const int per_image = g.bands * g.segments;
+			n = static_cast<int>(blockIdx.x) / per_image;
+			const int tile = static_cast<int>(blockIdx.x) - n * per_image;
+			band = tile / g.segments;
+			segment = tile - band * g.segments;
 		}
 		const int kb = static_cast<int>(blockIdx.y);
 		const int oh0 = band * g.TH;
+		const int ow0 = segment * 2 * g.pairs;
 		const int ih0 = oh0 + g.pad_h; /* input row of V row 0 */
 		const int v_rows = g.TH + 2;
 		int top = -ih0 < 0 ? 0 : -ih0; /* V rows above the image */
@@ -209,7 +219,11 @@ namespace
 		const unsigned int step_stride = static_cast<unsigned int>(POSITIONS * g.filter_tiles * PHASE_SLABS * OPERAND_BYTES);
 		const __amdgpu_buffer_rsrc_t ru = make_buffer(U, static_cast<unsigned int>(STEPS) * step_stride);
 		const unsigned int b_offset = static_cast<unsigned int>((p * g.filter_tiles + kb * 4 + fh * 2) * PHASE_SLABS * OPERAND_BYTES + lane * 16);
-		Chunk bq[3][PHASE_SLABS][2];
+		/* filters are requested two steps ahead where the kernel is written out, one step ahead where it loops: the sixteen registers
+		 * of a third set do not fit there (three registers spilled cost more, 198 against 192 us on 64 x 56 x 56 x 256 -> 256, than
+		 * the shorter way ahead) */
+		constexpr int AHEAD = PHASES <= MAX_PHASES ? 2 : 1;
+		Chunk bq[AHEAD + 1][PHASE_SLABS][2];
 		auto load_b = [&](int step, Chunk (&set)[PHASE_SLABS][2]) __attribute__((always_inline))
 		{
 #pragma unroll
@@ -237,7 +251,7 @@ namespace
 #pragma unroll
 			for (int j = 0; j < 4; j++)
 			{
-				const int iw = 2 * t_pair + g.pad_w + j;
+				const int iw = ow0 + 2 * t_pair + g.pad_w + j;
 				const bool inside = t_valid & (static_cast<unsigned int>(iw) < static_cast<unsigned int>(g.W));
 				x_src[j] = inside ? ((line + static_cast<unsigned int>(iw)) * g.C + t_chunk * 8) * SZ : OUT_OF_RANGE;
 			}
@@ -256,7 +270,7 @@ namespace
 		};
 		/* B^T d for this work-item's pixels; work-items without a (row, pair) of the band write to a spare pixel, so that the
 		 * transform is straight-line code the scheduler can spread among the MFMAs */
-		auto transform = [&](int phase) __attribute__((always_inline))
+		auto transform = [&](int slot) __attribute__((always_inline))
 		{
 			Half8 d[4];
 #pragma unroll
@@ -271,14 +285,14 @@ namespace
 				v[2].h[q] = pk_sub(d[2].h[q], d[1].h[q]);
 				v[3].h[q] = pk_sub(d[1].h[q], d[3].h[q]);
 			}
-			char *dst = lds + (phase >> 1) * SLICE_BYTES + (phase & 1) * 64 + v_dst;
+			char *dst = lds + (slot >> 1) * SLICE_BYTES + (slot & 1) * 64 + v_dst;
 #pragma unroll
 			for (int q = 0; q < POSITIONS; q++)
 				*reinterpret_cast<uint4*>(dst + q * POSITION_BYTES) = __builtin_bit_cast(uint4, v[q]);
 		};
 		load_x(0); /* what the first MFMA waits for longest goes out first */
 		load_b(0, bq[0]);
-		if (STEPS > 1)
+		if (AHEAD > 1)
 			load_b(1, bq[1]);
 
 		/* V rows outside the image are zeros, in every plane and slice: the rows above the image are the first `top * pairs`
@@ -286,7 +300,7 @@ namespace
 		{
 			const int above = top * g.pairs * 8, below = bottom * g.pairs * 8; /* 16-byte chunks per plane */
 			const int skip = real_rows * g.pairs * 8;
-			for (int plane = 0; plane < POSITIONS * ((PHASES + 1) / 2); plane++)
+			for (int plane = 0; plane < POSITIONS * ((PHASES < RING ? PHASES : RING) + 1) / 2; plane++)
 				for (int e = tid; e < above + below; e += THREADS)
 				{
 					const int at = e < above ? e : e + skip;
@@ -294,21 +308,13 @@ namespace
 				}
 		}
 
-		/* per-filter constants of the epilogue: a work-item always stores the same 8 filters */
-		const int kcol = kb * ROWS_BLOCK_N + (tid & 15) * 8;
-		typename FloatEpilogue<TE>::template ColumnsT<8> columns;
-		epi.request_columns(kcol, columns);
+		const int kcol = kb * ROWS_BLOCK_N + (tid & 15) * 8; /* a work-item always stores the same 8 filters */
 
-		/* MFMA operand addresses: lane l supplies GEMM row (l % 32) of a 32-row tile and the 8-channel half (l / 32) of a slab;
-		 * rows past the band read pixel 0 (their sums are never stored) */
-		int a_off[4];
+		/* MFMA operand address: lane l supplies GEMM row (l % 32) of a 32-row tile and the 8-channel half (l / 32) of a slab.  Rows
+		 * past the tile's last read whatever follows in LDS (at most 127 + 2 * pairs pixels into a plane of 137: the next plane, or
+		 * the slack behind the last one); their sums are never stored. */
 		const int band_rows = g.TH * g.pairs;
-#pragma unroll
-		for (int rt = 0; rt < 4; rt++)
-		{
-			const int q = rt * 32 + (lane & 31);
-			a_off[rt] = p * POSITION_BYTES + (q < band_rows ? q : 0) * PITCH + (lane >> 5) * 16;
-		}
+		const int a_off = p * POSITION_BYTES + (lane & 31) * PITCH + (lane >> 5) * 16;
 		const int tap_shift = g.pairs * PITCH;
 
 		STAMP(1);
@@ -319,79 +325,118 @@ namespace
 		STAMP(2);
 
 		typename Mma<f16_t>::acc_t acc[4][2];
-		Chunk a[2][4];
-		auto read_a = [&](int phase, int i, int sl, Chunk (&dst)[4]) __attribute__((always_inline))
+		/* A operands go through a ring of six register sets: the chunk four ahead of the one being multiplied is requested from LDS,
+		 * chunk = (phase, filter row, slab, 32-row tile) in the order of use */
+		constexpr int A_RING = 6, A_AHEAD = 4, STEP_CHUNKS_A = PHASE_SLABS * 4;
+		Chunk a[A_RING];
+		/* (slot: which of the ring's places in LDS holds the phase) */
+		auto read_a = [&](int slot, int i, int sl, int rt, Chunk &dst) __attribute__((always_inline))
 		{
-			const char *base = lds + (phase >> 1) * SLICE_BYTES + (phase & 1) * 64 + sl * 32 + i * tap_shift;
-#pragma unroll
-			for (int rt = 0; rt < 4; rt++)
-				dst[rt].u = *reinterpret_cast<const uint4*>(base + a_off[rt]);
+			dst.u = *reinterpret_cast<const uint4*>(lds + (slot >> 1) * SLICE_BYTES + (slot & 1) * 64 + sl * 32 + i * tap_shift + rt * 32 * PITCH + a_off);
 		};
-#pragma unroll
-		for (int phase = 0; phase < PHASES; phase++)
+		/*
+		 * The phases of one trip: all PHASES of them when they fit the ring (LOOPED false: written out once, the last phase without
+		 * the work for a next one), else RING of them per trip of a loop that stays a loop (LOOPED: the same code for every trip, which
+		 * keeps the registers of a layer with 256 channels where those of one with 128 are; after the last phase it requests, transforms
+		 * and reads ahead for a phase that does not exist: it asks for the last phase again, and the slot it writes is one that nobody
+		 * reads any more).  `first`: global number of the trip's first phase.
+		 */
+		auto run_phases = [&](auto looped, int first) __attribute__((always_inline))
 		{
+			constexpr bool LOOPED = decltype(looped)::value;
+			constexpr int COUNT = LOOPED ? RING : PHASES;
+			constexpr int CHUNKS = COUNT * FILTER_ROWS * STEP_CHUNKS_A;
 #pragma unroll
-			for (int i = 0; i < FILTER_ROWS; i++)
+			for (int phase = 0; phase < COUNT; phase++)
 			{
-				const int step = phase * FILTER_ROWS + i;
-				if (step + 2 < STEPS)
+				const bool more = LOOPED || phase + 1 < COUNT; /* another phase follows */
+#pragma unroll
+				for (int i = 0; i < FILTER_ROWS; i++)
 				{
-					/* two steps ahead and not a moment later: left to itself the scheduler sinks these requests to just before
-					 * their use, to shorten the life of their registers */
-					__builtin_amdgcn_sched_barrier(0);
-					load_b(step + 2, bq[(step + 2) % 3]);
-					__builtin_amdgcn_sched_barrier(0);
-				}
-				if (step == 0)
-					read_a(0, 0, 0, a[0]); /* behind the first barrier: nothing could be read ahead */
-				/* The next phase's V, from pixels requested a phase ago, is formed among the MFMAs of the middle step and made
-				 * visible by a barrier before the last one, so that the last step can read the first operands of the next phase
-				 * ahead like any other: no phase starts with a barrier and a bare LDS latency. */
-				const bool transform_here = i == 1 && phase + 1 < PHASES;
-				if (transform_here)
-					transform(phase + 1);
-				if (i == 2 && phase + 1 < PHASES)
-					__syncthreads();
-#pragma unroll
-				for (int sl = 0; sl < PHASE_SLABS; sl++)
-				{
-					const int s = step * PHASE_SLABS + sl;
-					if (sl + 1 < PHASE_SLABS)
-						read_a(phase, i, sl + 1, a[(s + 1) & 1]);
-					else if (i + 1 < FILTER_ROWS)
-						read_a(phase, i + 1, 0, a[(s + 1) & 1]);
-					else if (phase + 1 < PHASES)
-						read_a(phase + 1, 0, 0, a[(s + 1) & 1]);
-#pragma unroll
-					for (int rt = 0; rt < 4; rt++)
-#pragma unroll
-						for (int tn = 0; tn < 2; tn++)
-						{
-							/* filters as the rows of the MFMA tile, pixels as its columns: a lane then holds runs of four
-							 * consecutive filters of one pixel, which the fold can move as 16-byte vectors */
-							if (s == 0)
-								Mma<f16_t>::start(bq[step % 3][sl][tn], a[s & 1][rt], acc[rt][tn]);
-							else
-								Mma<f16_t>::run(bq[step % 3][sl][tn], a[s & 1][rt], acc[rt][tn]);
-						}
-				}
-				if (transform_here)
-				{
-					/* four vector instructions of the transform behind every MFMA: they issue while the matrix pipeline works */
-#pragma unroll
-					for (int k = 0; k < 4 * 2 * PHASE_SLABS; k++)
+					const int step = phase * FILTER_ROWS + i;
+					if (LOOPED || step + AHEAD < STEPS)
 					{
-						__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-						__builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-					}
-					__builtin_amdgcn_sched_barrier(0);
-					if (phase + 2 < PHASES)
-					{
-						load_x(phase + 2);
+						/* ahead by that many steps and not a moment later: left to itself the scheduler sinks these requests to just
+						 * before their use, to shorten the life of their registers */
 						__builtin_amdgcn_sched_barrier(0);
+						/* (a scalar offset is not part of a buffer's bounds check: steps past the last ask for the last again) */
+						const int ahead = first * FILTER_ROWS + step + AHEAD;
+						load_b(LOOPED ? (ahead < STEPS ? ahead : STEPS - 1) : ahead, bq[(step + AHEAD) % (AHEAD + 1)]);
+						__builtin_amdgcn_sched_barrier(0);
+					}
+					/* The next phase's V, from pixels requested a phase ago, is formed among the MFMAs of the middle step and made
+					 * visible by a barrier before the last one, so that the last step can read the first operands of the next phase
+					 * ahead like any other: no phase starts with a barrier and a bare LDS latency. */
+					const bool transform_here = i == 1 && more;
+					if (transform_here)
+						transform((phase + 1) % RING);
+					if (i == 2 && more)
+						__syncthreads();
+#pragma unroll
+					for (int sl = 0; sl < PHASE_SLABS; sl++)
+#pragma unroll
+						for (int rt = 0; rt < 4; rt++)
+						{
+							const int c = (step * PHASE_SLABS + sl) * 4 + rt;
+							const int cn = c + A_AHEAD; /* the chunk to request now */
+							if (cn < CHUNKS || LOOPED)
+							{
+								const int nstep = (cn / STEP_CHUNKS_A) % (COUNT * FILTER_ROWS), nphase = cn < CHUNKS ? nstep / FILTER_ROWS : COUNT;
+								read_a(nphase % RING, cn < CHUNKS ? nstep % FILTER_ROWS : 0, (cn / 4) % PHASE_SLABS, cn % 4, a[cn % A_RING]);
+							}
+#pragma unroll
+							for (int tn = 0; tn < 2; tn++)
+							{
+								/* filters as the rows of the MFMA tile, pixels as its columns: a lane then holds runs of four
+								 * consecutive filters of one pixel, which the fold can move as 16-byte vectors */
+								if (!LOOPED && step == 0 && sl == 0)
+									Mma<f16_t>::start(bq[step % (AHEAD + 1)][sl][tn], a[c % A_RING], acc[rt][tn]);
+								else
+									Mma<f16_t>::run(bq[step % (AHEAD + 1)][sl][tn], a[c % A_RING], acc[rt][tn]);
+							}
+						}
+					if (transform_here)
+					{
+						/* six vector instructions of the transform behind every MFMA: they issue while the matrix pipeline works */
+#pragma unroll
+						for (int k = 0; k < 4 * 2 * PHASE_SLABS; k++)
+						{
+							__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+							__builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+							if (k % 3 == 2)
+								__builtin_amdgcn_sched_group_barrier(0x200, 1, 0); /* a finished plane leaves for LDS at once */
+						}
+						__builtin_amdgcn_sched_barrier(0);
+						if (LOOPED || phase + 2 < COUNT)
+						{
+							const int next = first + phase + 2;
+							load_x(LOOPED ? (next < PHASES ? next : PHASES - 1) : next);
+							__builtin_amdgcn_sched_barrier(0);
+						}
 					}
 				}
 			}
+		};
+		/* behind the first barrier: nothing could be read ahead */
+#pragma unroll
+		for (int c = 0; c < A_AHEAD; c++)
+			read_a(0, 0, c / 4, c % 4, a[c]);
+		if constexpr (PHASES <= RING)
+			run_phases(std::false_type(), 0);
+		else
+		{
+			static_assert(PHASES % RING == 0 && (RING * FILTER_ROWS) % (AHEAD + 1) == 0 && (RING * FILTER_ROWS * STEP_CHUNKS_A) % A_RING == 0,
+					"whole trips, and the operand rings in the same position at the start of each");
+#pragma unroll
+			for (int rt = 0; rt < 4; rt++)
+#pragma unroll
+				for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+					for (int v = 0; v < 16; v++)
+						acc[rt][tn][v] = 0.0f;
+#pragma unroll 1
+			for (int first = 0; first < PHASES; first += RING)
+				run_phases(std::true_type(), first);
 		}
 
 		STAMP(3);
@@ -402,6 +447,10 @@ namespace
 		if (epi.z != nullptr)
 			rz = make_buffer(epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
 		const bool relu = epi.activation == ACT_RELU, has_z = epi.z != nullptr;
+		/* per-filter constants of the epilogue (requested here and not before the k loop, where eight more live registers are eight
+		 * too many; the fold through LDS hides the latency) */
+		typename FloatEpilogue<TE>::template ColumnsT<8> columns;
+		epi.request_columns(kcol, columns);
 		/* where this work-item's two rows of either pass go, and their residual, requested before the planes go through LDS */
 		unsigned int y_off[2][2][2];
 		typename FloatEpilogue<TE>::template Residual<8> residual[2][2][2];
@@ -418,7 +467,7 @@ namespace
 #pragma unroll
 				for (int o = 0; o < 2; o++)
 				{
-					const int ow = 2 * pair + o;
+					const int ow = ow0 + 2 * pair + o;
 					y_off[pass][it][o] = (row_ok & (ow < g.Wo)) ? static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ : OUT_OF_RANGE;
 					union
 					{
@@ -508,45 +557,61 @@ namespace
 		STAMP(4);
 	}
 
-	/* Rows per band: as many as fit 128 GEMM rows, the V plane and one transform item per work-item and phase
-	 * (rows inside the image x pairs <= 128).  0 when no band height does. */
-	int choose_band(const avhipConvShape &s, int pairs)
+	/* The tile (TH output rows by `pairs` column pairs) of a layer: what fits 128 GEMM rows, the V plane and one transform item per
+	 * work-item and phase (rows of the tile's input inside the image x pairs <= 128), with the fewest tiles per image and, among
+	 * those, the fewest halo rows.  th = 0 when nothing fits. */
+	struct RowsTile
 	{
-		for (int th = s.Ho < ROWS_MAX ? s.Ho : ROWS_MAX; th >= 1; th--)
+		int th, pairs, bands, segments;
+	};
+	RowsTile choose_tile(const avhipConvShape &s)
+	{
+		RowsTile best = { 0, 0, 0, 0 };
+		const int all_pairs = (s.Wo + 1) / 2;
+		for (int pairs = 1; pairs <= all_pairs && pairs <= ROWS_MAX; pairs++)
 		{
-			if (th * pairs > ROWS_MAX || (th + 2) * pairs > PIXELS_MAX)
-				continue;
-			bool fits = true;
-			for (int oh0 = 0; oh0 < s.Ho && fits; oh0 += th)
+			const int segments = (all_pairs + pairs - 1) / pairs;
+			if (pairs > 1 && (all_pairs + pairs - 2) / (pairs - 1) == segments)
+				continue; /* a narrower tile gives the same number of segments: handled at that width, with more rows per tile */
+			for (int th = s.Ho < ROWS_MAX ? s.Ho : ROWS_MAX; th >= 1; th--)
 			{
-				const int first = oh0 + s.pad_h, last = first + th + 2; /* input rows [first, last) */
-				const int lo = first < 0 ? 0 : first, hi = last > s.H ? s.H : last;
-				if (hi > lo && (hi - lo) * pairs > ROWS_MAX)
-					fits = false;
+				if (th * pairs > ROWS_MAX || (th + 2) * pairs > PIXELS_MAX)
+					continue;
+				bool fits = true;
+				for (int oh0 = 0; oh0 < s.Ho && fits; oh0 += th)
+				{
+					const int first = oh0 + s.pad_h, last = first + th + 2; /* input rows [first, last) */
+					const int lo = first < 0 ? 0 : first, hi = last > s.H ? s.H : last;
+					if (hi > lo && (hi - lo) * pairs > ROWS_MAX)
+						fits = false;
+				}
+				if (!fits)
+					continue;
+				const int bands = (s.Ho + th - 1) / th;
+				if (best.th == 0 || bands * segments < best.bands * best.segments || (bands * segments == best.bands * best.segments && bands < best.bands))
+					best = { th, pairs, bands, segments };
+				break; /* smaller th only adds tiles */
 			}
-			if (fits)
-				return th;
 		}
-		return 0;
+		return best;
 	}
 
 	template<typename TE>
 	int launch_rows(hipStream_t st, const avhipConvShape &s, const void *x, const void *U, const void *bias, const void *z, void *y, double alpha1,
 			double alpha2, int activation)
 	{
-		if ((s.C != 64 && s.C != 128) || s.K % ROWS_BLOCK_N != 0)
+		if ((s.C != 64 && s.C != 128 && s.C != 256) || s.K % ROWS_BLOCK_N != 0)
 			return AVHIP_NOT_SUPPORTED;
 		if (!aligned_to(x, 16) || !aligned_to(U, 16) || !aligned_to(y, 16) || (z != nullptr && !aligned_to(z, 16)) || (bias != nullptr && !aligned_to(bias, 16)))
 			return AVHIP_NOT_SUPPORTED;
 		if (static_cast<int64_t>(s.N) * s.H * s.W * s.C * sizeof(TE) >= (1ll << 31) || static_cast<int64_t>(s.Ho) * s.Wo * s.K * sizeof(TE) >= (1ll << 31))
 			return AVHIP_NOT_SUPPORTED;
-		const int pairs = (s.Wo + 1) / 2;
-		if (pairs > ROWS_MAX)
+		const RowsTile tile = choose_tile(s);
+		if (tile.th == 0)
 			return AVHIP_NOT_SUPPORTED;
+		const int pairs = tile.pairs;
 		RowsGeom g;
-		g.TH = choose_band(s, pairs);
-		if (g.TH == 0)
-			return AVHIP_NOT_SUPPORTED;
+		g.TH = tile.th;
 		g.H = s.H;
 		g.W = s.W;
 		g.C = s.C;
@@ -557,16 +622,19 @@ namespace
 		g.pad_w = s.pad_w;
 		g.pairs = pairs;
 		g.pairs_magic = (1u << 20) / static_cast<unsigned int>(pairs) + 1u;
-		g.bands = (s.Ho + g.TH - 1) / g.TH;
+		g.bands = tile.bands;
+		g.segments = tile.segments;
 		g.images = s.N;
 		g.filter_tiles = s.K / 32;
-		const int64_t items = static_cast<int64_t>(s.N) * g.bands;
+		const int64_t items = static_cast<int64_t>(s.N) * g.bands * g.segments;
 		if (items >= (1ll << 31) || s.K / ROWS_BLOCK_N > 65535)
 			return AVHIP_NOT_SUPPORTED;
 		const FloatEpilogue<TE> epi { static_cast<const float*>(bias), static_cast<const TE*>(z), static_cast<TE*>(y), static_cast<float>(alpha1),
 				static_cast<float>(alpha2), 0.0f, activation, s.K, true };
 		const dim3 grid(static_cast<unsigned int>(items), static_cast<unsigned int>(s.K / ROWS_BLOCK_N));
-		if (s.C == 128)
+		if (s.C == 256)
+			hipLaunchKernelGGL((k_winograd_rows<TE, 8>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+		else if (s.C == 128)
 			hipLaunchKernelGGL((k_winograd_rows<TE, 4>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
 		else
 			hipLaunchKernelGGL((k_winograd_rows<TE, 2>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
@@ -589,20 +657,21 @@ extern "C" int avhip_conv2d_winograd_rows_plan(int dtype, const avhipConvShape *
 	const avhipConvShape &s = *shape;
 	if (rows_mode.load() == 0 || (dtype != DT_FLOAT16 && dtype != DT_BFLOAT16))
 		return AVHIP_NOT_SUPPORTED;
-	if (s.R != 3 || s.S != 3 || s.stride_h != 1 || s.stride_w != 1 || s.dil_h != 1 || s.dil_w != 1 || (s.C != 64 && s.C != 128) || s.K % ROWS_BLOCK_N != 0
-			|| s.N <= 0 || s.Ho <= 0 || s.Wo <= 0)
+	if (s.R != 3 || s.S != 3 || s.stride_h != 1 || s.stride_w != 1 || s.dil_h != 1 || s.dil_w != 1 || (s.C != 64 && s.C != 128 && s.C != 256)
+			|| s.K % ROWS_BLOCK_N != 0 || s.N <= 0 || s.Ho <= 0 || s.Wo <= 0)
 		return AVHIP_NOT_SUPPORTED;
-	const int pairs = (s.Wo + 1) / 2;
-	if (pairs > ROWS_MAX)
+	const RowsTile tile = choose_tile(s);
+	if (tile.th == 0)
 		return AVHIP_NOT_SUPPORTED;
-	const int th = choose_band(s, pairs);
-	if (th == 0)
-		return AVHIP_NOT_SUPPORTED;
-	const int64_t groups = static_cast<int64_t>(s.N) * ((s.Ho + th - 1) / th) * (s.K / ROWS_BLOCK_N);
+	const int64_t groups = static_cast<int64_t>(s.N) * tile.bands * tile.segments * (s.K / ROWS_BLOCK_N);
 	if (workgroups != nullptr)
 		workgroups[0] = groups > 0x7FFFFFFF ? 0x7FFFFFFF : static_cast<int>(groups);
 	if (rows_used != nullptr)
-		rows_used[0] = th * pairs;
+	{
+		/* GEMM rows that are output pixel pairs, averaged over the tiles of an image (tiles at the right and lower edge are partial) */
+		const int64_t useful = static_cast<int64_t>(s.Ho) * ((s.Wo + 1) / 2);
+		rows_used[0] = static_cast<int>(useful / (tile.bands * tile.segments));
+	}
 	return 0;
 }
 
