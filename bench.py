@@ -297,24 +297,26 @@ def time_calls(hip, ctx, fn, iters, warmup=3):
     return ms
 
 
-def int8_leg(hip, ctx, iters):
+def int8_leg(hip, ctx, iters, shape=(128, 20, 20, 128), filters=((3, -1), (1, 0))):
     """Config 4: N=128, 20x20, 128->128, 3x3 offset -1 and 1x1: int8 x int8 -> int32 (bit-exact path), int8 -> int8
-    requantised by a per-filter fp32 scale, and the same shapes in bf16 for the throughput ratio on equal work."""
+    requantised by a per-filter fp32 scale, and the same shapes in bf16 for the throughput ratio on equal work: through the same
+    entry point (cudaConvolutionImplicitGemmForward: the direct kernels for both types) and, as `bf16_dispatcher`, through
+    cudaConvolutionBiasActivationForward, which may pick a Winograd plan that int8 cannot have."""
     lib = cb.load_library()
     g = np.random.default_rng(SEED + 4)
     out = {}
-    shape = (128, 20, 20, 128)
+    ch = shape[3]
     x = cb.DeviceTensor.from_numpy(g.integers(-127, 128, shape, dtype=np.int8), cb.DTYPE_INT8)
-    b = cb.DeviceTensor.from_numpy(g.integers(-2 ** 15, 2 ** 15, 128).astype(np.int32), cb.DTYPE_INT32)
-    scale = cb.DeviceTensor.from_numpy(g.uniform(1e-4, 1e-3, 128).astype(np.float32), cb.DTYPE_FLOAT32)
+    b = cb.DeviceTensor.from_numpy(g.integers(-2 ** 15, 2 ** 15, ch).astype(np.int32), cb.DTYPE_INT32)
+    scale = cb.DeviceTensor.from_numpy(g.uniform(1e-4, 1e-3, ch).astype(np.float32), cb.DTYPE_FLOAT32)
     y = cb.DeviceTensor(shape, cb.DTYPE_INT32)
     q = cb.DeviceTensor(shape, cb.DTYPE_INT8)
     xb = cb.DeviceTensor.from_numpy(g.standard_normal(shape).astype(np.float32), cb.DTYPE_BFLOAT16)
-    bb = cb.DeviceTensor.from_numpy(g.uniform(-0.1, 0.1, 128).astype(np.float32), cb.DTYPE_FLOAT32)
+    bb = cb.DeviceTensor.from_numpy(g.uniform(-0.1, 0.1, ch).astype(np.float32), cb.DTYPE_FLOAT32)
     yb = cb.DeviceTensor(shape, cb.DTYPE_BFLOAT16)
-    for r, pad in ((3, -1), (1, 0)):
-        w = cb.DeviceTensor.from_numpy(g.integers(-127, 128, (128, r, r, 128), dtype=np.int8), cb.DTYPE_INT8)
-        wb = cb.DeviceTensor.from_numpy((g.standard_normal((128, r, r, 128)) * np.sqrt(2.0 / (r * r * 128))).astype(np.float32), cb.DTYPE_BFLOAT16)
+    for r, pad in filters:
+        w = cb.DeviceTensor.from_numpy(g.integers(-127, 128, (ch, r, r, ch), dtype=np.int8), cb.DTYPE_INT8)
+        wb = cb.DeviceTensor.from_numpy((g.standard_normal((ch, r, r, ch)) * np.sqrt(2.0 / (r * r * ch))).astype(np.float32), cb.DTYPE_BFLOAT16)
         conv = cb.ConvolutionDescriptor(padding=(pad, pad), dtype=cb.DTYPE_INT8)
         convb = cb.ConvolutionDescriptor(padding=(pad, pad), dtype=cb.DTYPE_BFLOAT16)
 
@@ -329,13 +331,19 @@ def int8_leg(hip, ctx, iters):
         def bf16():
             cb.check(lib.cudaConvolutionImplicitGemmForward(ctx.handle, convb.handle, None, xb.desc, xb.mem, wb.desc, wb.mem, bb.desc, bb.mem, None, 0, 0,
                                                             None, yb.desc, yb.mem, cb.ACTIVATION_RELU), "bf16 conv")
-        ops = conv_flops(128, 20, 20, 128, 128, r, r)
+
+        def bf16_dispatcher():
+            cb.check(lib.cudaConvolutionBiasActivationForward(ctx.handle, convb.handle, None, xb.desc, xb.mem, wb.desc, wb.mem, bb.desc, bb.mem, None, 0, 0,
+                                                              None, yb.desc, yb.mem, cb.ACTIVATION_RELU, 0), "bf16 conv, dispatcher")
+        ops = conv_flops(shape[0], shape[1], shape[2], ch, ch, r, r)
         rec = {}
-        for name, fn in (("int32_out", exact), ("int8_requant_out", requant), ("bf16_same_shape", bf16)):
+        for name, fn in (("int32_out", exact), ("int8_requant_out", requant), ("bf16_same_shape", bf16), ("bf16_dispatcher", bf16_dispatcher)):
             ms = time_calls(hip, ctx, fn, iters)
             rec[name] = {"us": ms * 1e3, "tops": ops / (ms * 1e-3) / 1e12}
         rec["int8_over_bf16"] = {"int32_out": rec["bf16_same_shape"]["us"] / rec["int32_out"]["us"],
                                  "int8_requant_out": rec["bf16_same_shape"]["us"] / rec["int8_requant_out"]["us"]}
+        rec["int8_over_bf16_dispatcher"] = {"int32_out": rec["bf16_dispatcher"]["us"] / rec["int32_out"]["us"],
+                                            "int8_requant_out": rec["bf16_dispatcher"]["us"] / rec["int8_requant_out"]["us"]}
         out["%dx%d" % (r, r)] = rec
         w.close()
         wb.close()
@@ -622,6 +630,8 @@ def main():
                 detail["tower_" + other] = time_tower(hip, ctx, other, max(3, args.steps // 2), 2, check=not args.no_cpu)
         detail["caller_level_two_chains_of_128"] = two_half_batch_chains(hip, args.dtype, args.steps)
         detail["int8_config4"] = int8_leg(hip, ctx, it)
+        # the same comparison on a layer large enough for the k loop to dominate the fixed cost of a launch (the shape of config 3)
+        detail["int8_at_config3_shape"] = int8_leg(hip, ctx, it, shape=(64, 56, 56, 256), filters=((3, -1),))
         detail["copy_GBs_measured"] = copy_bandwidth(hip, ctx)
         rates = detail["stream_GBs_measured"] = stream_rates(hip, ctx)
         detail["nonfused_winograd_f32_F4"] = nonfused_stages(hip, ctx, "f32", "f32", 4, it, rates=rates)

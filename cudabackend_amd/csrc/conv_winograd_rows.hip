@@ -219,22 +219,22 @@ namespace
 		const unsigned int step_stride = static_cast<unsigned int>(POSITIONS * g.filter_tiles * PHASE_SLABS * OPERAND_BYTES);
 		const __amdgpu_buffer_rsrc_t ru = make_buffer(U, static_cast<unsigned int>(STEPS) * step_stride);
 		const unsigned int b_offset = static_cast<unsigned int>((p * g.filter_tiles + kb * 4 + fh * 2) * PHASE_SLABS * OPERAND_BYTES + lane * 16);
-		/* filters are requested two steps ahead where the kernel is written out, one step ahead where it loops: the sixteen registers
-		 * of a third set do not fit there (three registers spilled cost more, 198 against 192 us on 64 x 56 x 56 x 256 -> 256, than
-		 * the shorter way ahead) */
-		constexpr int AHEAD = PHASES <= MAX_PHASES ? 2 : 1;
-		Chunk bq[AHEAD + 1][PHASE_SLABS][2];
-		auto load_b = [&](int step, Chunk (&set)[PHASE_SLABS][2]) __attribute__((always_inline))
+		/* Filters go through a ring of register sets, one set = the two filter tiles of one 16-channel slab (two slabs per step),
+		 * requested B_AHEAD slabs before they are multiplied: six sets where the kernel is written out, four where it loops (the
+		 * sixteen registers more do not fit there: three registers spilled cost more, 198 against 192 us on 64 x 56 x 56 x 256 -> 256,
+		 * than the shorter way ahead). */
+		constexpr int B_RING = PHASES <= MAX_PHASES ? 6 : 4, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
+		Chunk bq[B_RING][2];
+		auto load_b = [&](int slab, Chunk (&set)[2]) __attribute__((always_inline)) /* slab: (step, slab of the step), over the whole k walk */
 		{
+			const int step = slab / PHASE_SLABS, sl = slab - step * PHASE_SLABS;
 #pragma unroll
 			for (int tn = 0; tn < 2; tn++)
-#pragma unroll
-				for (int sl = 0; sl < PHASE_SLABS; sl++)
-				{
-					const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(ru, static_cast<int>(b_offset + (tn * PHASE_SLABS + sl) * OPERAND_BYTES),
-							static_cast<int>(step * step_stride), 0);
-					set[sl][tn].u = make_uint4(v[0], v[1], v[2], v[3]);
-				}
+			{
+				const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(ru, static_cast<int>(b_offset + tn * PHASE_SLABS * OPERAND_BYTES),
+						static_cast<int>(step * step_stride + sl * OPERAND_BYTES), 0);
+				set[tn].u = make_uint4(v[0], v[1], v[2], v[3]);
+			}
 		};
 
 		/* transform side: this work-item's (row, pair, 8 channels) of every phase */
@@ -291,9 +291,9 @@ namespace
 				*reinterpret_cast<uint4*>(dst + q * POSITION_BYTES) = __builtin_bit_cast(uint4, v[q]);
 		};
 		load_x(0); /* what the first MFMA waits for longest goes out first */
-		load_b(0, bq[0]);
-		if (AHEAD > 1)
-			load_b(1, bq[1]);
+#pragma unroll
+		for (int slab = 0; slab < B_AHEAD; slab++)
+			load_b(slab, bq[slab]);
 
 		/* V rows outside the image are zeros, in every plane and slice: the rows above the image are the first `top * pairs`
 		 * pixels of a plane, the rows below it its last `bottom * pairs` */
@@ -354,26 +354,25 @@ namespace
 				for (int i = 0; i < FILTER_ROWS; i++)
 				{
 					const int step = phase * FILTER_ROWS + i;
-					if (LOOPED || step + AHEAD < STEPS)
-					{
-						/* ahead by that many steps and not a moment later: left to itself the scheduler sinks these requests to just
-						 * before their use, to shorten the life of their registers */
-						__builtin_amdgcn_sched_barrier(0);
-						/* (a scalar offset is not part of a buffer's bounds check: steps past the last ask for the last again) */
-						const int ahead = first * FILTER_ROWS + step + AHEAD;
-						load_b(LOOPED ? (ahead < STEPS ? ahead : STEPS - 1) : ahead, bq[(step + AHEAD) % (AHEAD + 1)]);
-						__builtin_amdgcn_sched_barrier(0);
-					}
+					__builtin_amdgcn_sched_barrier(0); /* a step is one scheduling region, laid out by the groups at its end */
 					/* The next phase's V, from pixels requested a phase ago, is formed among the MFMAs of the middle step and made
 					 * visible by a barrier before the last one, so that the last step can read the first operands of the next phase
 					 * ahead like any other: no phase starts with a barrier and a bare LDS latency. */
 					const bool transform_here = i == 1 && more;
-					if (transform_here)
-						transform((phase + 1) % RING);
 					if (i == 2 && more)
 						__syncthreads();
 #pragma unroll
 					for (int sl = 0; sl < PHASE_SLABS; sl++)
+					{
+						const int slab = step * PHASE_SLABS + sl; /* within the trip */
+						if (LOOPED || slab + B_AHEAD < SLABS_TOTAL)
+						{
+							/* (a scalar offset is not part of a buffer's bounds check: slabs past the last ask for the last again) */
+							const int ahead = first * FILTER_ROWS * PHASE_SLABS + slab + B_AHEAD;
+							load_b(LOOPED ? (ahead < SLABS_TOTAL ? ahead : SLABS_TOTAL - 1) : ahead, bq[(slab + B_AHEAD) % B_RING]);
+						}
+						if (transform_here && sl == 0)
+							transform((phase + 1) % RING);
 #pragma unroll
 						for (int rt = 0; rt < 4; rt++)
 						{
@@ -390,28 +389,40 @@ namespace
 								/* filters as the rows of the MFMA tile, pixels as its columns: a lane then holds runs of four
 								 * consecutive filters of one pixel, which the fold can move as 16-byte vectors */
 								if (!LOOPED && step == 0 && sl == 0)
-									Mma<f16_t>::start(bq[step % (AHEAD + 1)][sl][tn], a[c % A_RING], acc[rt][tn]);
+									Mma<f16_t>::start(bq[slab % B_RING][tn], a[c % A_RING], acc[rt][tn]);
 								else
-									Mma<f16_t>::run(bq[step % (AHEAD + 1)][sl][tn], a[c % A_RING], acc[rt][tn]);
+									Mma<f16_t>::run(bq[slab % B_RING][tn], a[c % A_RING], acc[rt][tn]);
 							}
 						}
-					if (transform_here)
-					{
-						/* six vector instructions of the transform behind every MFMA: they issue while the matrix pipeline works */
+					}
+					/* The order of the step's instructions: the filter requests of a slab go out in front of the slab's MFMAs and not a
+					 * moment later (left to itself the scheduler sinks them to just before their use, to shorten the life of their
+					 * registers); four vector instructions of the transform behind every MFMA issue while the matrix pipeline works,
+					 * and a finished plane leaves for LDS at once. */
 #pragma unroll
-						for (int k = 0; k < 4 * 2 * PHASE_SLABS; k++)
+					for (int sl = 0; sl < PHASE_SLABS; sl++)
+					{
+						if (LOOPED || step * PHASE_SLABS + sl + B_AHEAD < SLABS_TOTAL)
+							__builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+#pragma unroll
+						for (int k = 0; k < 8; k++)
 						{
 							__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-							__builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-							if (k % 3 == 2)
-								__builtin_amdgcn_sched_group_barrier(0x200, 1, 0); /* a finished plane leaves for LDS at once */
+							if (transform_here)
+							{
+								__builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+								if (k % 4 == 3)
+									__builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+							}
 						}
+					}
+					if (transform_here)
+					{
 						__builtin_amdgcn_sched_barrier(0);
 						if (LOOPED || phase + 2 < COUNT)
 						{
 							const int next = first + phase + 2;
 							load_x(LOOPED ? (next < PHASES ? next : PHASES - 1) : next);
-							__builtin_amdgcn_sched_barrier(0);
 						}
 					}
 				}
@@ -425,7 +436,7 @@ namespace
 			run_phases(std::false_type(), 0);
 		else
 		{
-			static_assert(PHASES % RING == 0 && (RING * FILTER_ROWS) % (AHEAD + 1) == 0 && (RING * FILTER_ROWS * STEP_CHUNKS_A) % A_RING == 0,
+			static_assert(PHASES % RING == 0 && (RING * FILTER_ROWS * PHASE_SLABS) % B_RING == 0 && (RING * FILTER_ROWS * STEP_CHUNKS_A) % A_RING == 0,
 					"whole trips, and the operand rings in the same position at the start of each");
 #pragma unroll
 			for (int rt = 0; rt < 4; rt++)
@@ -482,6 +493,8 @@ namespace
 		for (int pass = 0; pass < 2; pass++)
 		{
 			__syncthreads(); /* pass 0: everyone is done with V; pass 1: with the planes of pass 0 */
+			if (pass == 0)
+				STAMP(5);
 			typedef float quad_t __attribute__((ext_vector_type(4)));
 #ifndef ROWS_KNOCK_LDS
 			/* A row of the fold buffer holds the 128 filters of a pixel as [first halves | second halves] of the 16 runs of 8
@@ -501,6 +514,8 @@ namespace
 					}
 			__syncthreads();
 #endif
+			if (pass == 0)
+				STAMP(6);
 			quad_t m[2][POSITIONS][2];
 #pragma unroll
 			for (int it = 0; it < 2; it++)
@@ -553,6 +568,8 @@ namespace
 				leave(std::false_type(), std::true_type());
 			else
 				leave(std::false_type(), std::false_type());
+			if (pass == 0)
+				STAMP(7);
 		}
 		STAMP(4);
 	}
