@@ -94,7 +94,8 @@ KERNEL_LAYER_SYMBOLS = ["avhip_winograd_weight_transform", "avhip_winograd_input
                         "avhip_set_memory", "avhip_mfma_rate_probe", "avhip_set_small_problem_threshold", "avhip_set_short_k_engine",
                         "avhip_affine_forward", "avhip_batchnorm_inference", "avhip_stream_probe", "avhip_conv2d_winograd_rows",
                         "avhip_winograd_rows_weight_transform", "avhip_winograd_rows_weight_bytes", "avhip_conv2d_winograd_rows_plan",
-                        "avhip_set_winograd_rows"]
+                        "avhip_set_winograd_rows", "avhip_conv2d_strided", "avhip_conv2d_strided_weight_layout", "avhip_conv2d_strided_weight_bytes",
+                        "avhip_conv2d_strided_plan", "avhip_set_conv_strided"]
 
 _lib = None
 

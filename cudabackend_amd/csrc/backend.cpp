@@ -481,7 +481,8 @@ namespace
 		uint64_t uid;
 		av_int64 offset;
 		int K, C, dtype, mode, m; /* m: Winograd output tile, 2 = F(2x2,3x3) for the fused kernel, 4 = F(4x4,3x3) for the non-fused plan,
-		                           * 1 = F(2,3) along rows in the operand layout of the row-Winograd kernel */
+		                           * 1 = F(2,3) along rows in the operand layout of the row-Winograd kernel, 3 = the weights themselves in the
+		                           * operand layout of the stride-2 kernel (no transform) */
 		bool operator<(const WeightKey &o) const
 		{
 			return std::tie(uid, offset, K, C, dtype, mode, m) < std::tie(o.uid, o.offset, o.K, o.C, o.dtype, o.mode, o.m);
@@ -645,6 +646,7 @@ namespace
 		const WeightKey key { owner->uid, offset, p.shape.K, p.shape.C, static_cast<int>(p.w_dtype), p.shape.mode, m };
 		const int t = m + 2;
 		const size_t bytes = m == 1 ? static_cast<size_t>(avhip_winograd_rows_weight_bytes(p.shape.K, p.shape.C))
+				: m == 3 ? static_cast<size_t>(avhip_conv2d_strided_weight_bytes(p.shape.K, p.shape.C))
 				: static_cast<size_t>(t * t) * p.shape.K * p.shape.C * size_of(mat_dtype);
 		WeightCache &cache = weight_cache();
 		std::vector<WeightEntry> victims;
@@ -712,6 +714,7 @@ namespace
 				/* the write number is read before the transform is enqueued: a write that slips in between is seen next time */
 				e.seen = owner->writes->current();
 				const int rc = m == 1 ? avhip_winograd_rows_weight_transform(ctx.stream, p.w_dtype, p.shape.mode, wm->data, e.U, p.shape.K, p.shape.C)
+						: m == 3 ? avhip_conv2d_strided_weight_layout(ctx.stream, p.w_dtype, p.shape.mode, wm->data, e.U, p.shape.K, p.shape.C)
 						: avhip_winograd_weight_transform(ctx.stream, p.w_dtype, mat_dtype, m, 3, p.shape.mode, wm->data, e.U, p.shape.K, p.shape.C);
 				status = from_launcher(rc);
 				cache.transforms++;
@@ -960,6 +963,35 @@ namespace
 			return st;
 		const int rc = avhip_conv2d_winograd_rows(c.ctx.stream, p.x_dtype, &p.shape, c.x->data, U, c.bias, c.z, c.y->data, c.alpha1, c.alpha2, c.beta,
 				activation);
+		if (rc == AVHIP_NOT_SUPPORTED)
+			return AVOCADO_STATUS_NOT_SUPPORTED;
+		touch(yMem);
+		return from_launcher(rc);
+	}
+
+	/* 3x3 stride-2 layers of 16-bit tensors through the parity-plane kernel (conv_strided.hip), weights in its operand layout from
+	 * the cache.  Worth it when its workgroups (one per compute unit, 256 filters each) cover most of the chip. */
+	bool strided_kernel_pays(const ConvCall &c, avActivationType_t activation)
+	{
+		const ConvProblem &p = c.problem;
+		if (p.y_dtype != p.x_dtype || !p.conv->padding_value_is_zero() || c.beta != 0.0 || (c.bias != nullptr && c.bias_dtype != AVOCADO_DTYPE_FLOAT32))
+			return false;
+		if (activation != AVOCADO_ACTIVATION_LINEAR && activation != AVOCADO_ACTIVATION_RELU)
+			return false;
+		int workgroups = 0, rows_used = 0;
+		if (avhip_conv2d_strided_plan(p.x_dtype, &p.shape, &workgroups, &rows_used) != 0)
+			return false;
+		return avhip_set_conv_strided(-1) == 2 || (workgroups >= 192 && rows_used >= 144);
+	}
+	avStatus_t run_strided_kernel(const ConvCall &c, avMemoryDescriptor_t wMem, avMemoryDescriptor_t yMem, avActivationType_t activation)
+	{
+		const ConvProblem &p = c.problem;
+		const void *U = nullptr;
+		WeightLease lease;
+		const avStatus_t st = cached_winograd_weights(c.ctx, p, wMem, 3, p.w_dtype, &U, lease);
+		if (st != AVOCADO_STATUS_SUCCESS)
+			return st;
+		const int rc = avhip_conv2d_strided(c.ctx.stream, p.x_dtype, &p.shape, c.x->data, U, c.bias, c.z, c.y->data, c.alpha1, c.alpha2, c.beta, activation);
 		if (rc == AVHIP_NOT_SUPPORTED)
 			return AVOCADO_STATUS_NOT_SUPPORTED;
 		touch(yMem);
@@ -1990,6 +2022,12 @@ namespace avocado
 			if (rows_winograd_pays(call, activation))
 			{
 				const avStatus_t rs = run_rows_winograd(call, wMem, yMem, activation);
+				if (rs != AVOCADO_STATUS_NOT_SUPPORTED && rs != AVOCADO_STATUS_BAD_ALLOC)
+					return rs;
+			}
+			if (strided_kernel_pays(call, activation))
+			{
+				const avStatus_t rs = run_strided_kernel(call, wMem, yMem, activation);
 				if (rs != AVOCADO_STATUS_NOT_SUPPORTED && rs != AVOCADO_STATUS_BAD_ALLOC)
 					return rs;
 			}

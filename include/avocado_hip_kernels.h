@@ -114,6 +114,22 @@ extern "C"
 	 * (tests); a negative value changes nothing.  Returns the previous value. */
 	AVHIP_API int avhip_set_winograd_rows(int mode);
 
+	/* The same formula for 3x3 stride-2 layers of 16-bit tensors (dilation 1, zero padding value, C a multiple of 64, K a multiple of
+	 * 256, beta = 0, LINEAR or RELU; AVHIP_NOT_SUPPORTED otherwise, with nothing launched): the input under a tile of output pixels
+	 * lies in LDS as four parity planes, so that a filter tap is a constant shift of consecutive plane pixels, and the filters come
+	 * straight from L2 in MFMA register layout.  Stands where the reference has cuda_convolution2dImplicitGemm,
+	 * src/conv2d_implicit_gemm.cu:303 (stride 1 only there).  U is what avhip_conv2d_strided_weight_layout wrote:
+	 * avhip_conv2d_strided_weight_bytes(K, C) bytes, the weights themselves in the order [C / 32][9][K / 32][2][64 lanes][8]. */
+	AVHIP_API int avhip_conv2d_strided(void *stream, int dtype, const avhipConvShape *shape, const void *x, const void *U, const void *bias, const void *z,
+			void *y, double alpha1, double alpha2, double beta, int activation);
+	AVHIP_API int avhip_conv2d_strided_weight_layout(void *stream, int dtype, int invert, const void *w, void *U, int K, int C);
+	AVHIP_API int64_t avhip_conv2d_strided_weight_bytes(int K, int C);
+	/* Whether avhip_conv2d_strided takes the layer (0) or not (AVHIP_NOT_SUPPORTED), its workgroups and the output pixels per
+	 * workgroup (of 224 GEMM rows); avhip_set_conv_strided: 0 declines everything, 1 (default) lets the dispatcher weigh it, 2 makes
+	 * the dispatcher take every layer it can run, negative changes nothing; returns the previous value. */
+	AVHIP_API int avhip_conv2d_strided_plan(int dtype, const avhipConvShape *shape, int *workgroups, int *rows_used);
+	AVHIP_API int avhip_set_conv_strided(int mode);
+
 	/* y = alpha1 * act(alpha2 * x + b + beta1 * z) + beta2 * z + beta3 * y.  Replaces kernel_add_bias,
 	 * src/tensor_op.cu:199-228.  x, y, z have `dtype`; b is fp32 (fp64 for fp64 tensors). */
 	AVHIP_API int avhip_add_bias(void *stream, int dtype, const void *x, const void *b, const void *z, void *y, int64_t first, int last, double alpha1,
