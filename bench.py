@@ -31,9 +31,11 @@ PEAK = {"hbm_GBs": 8000.0, "bf16": 2500.0, "f16": 2500.0, "i8": 5000.0, "f32": 1
 DT = {"bf16": cb.DTYPE_BFLOAT16, "f16": cb.DTYPE_FLOAT16, "f32": cb.DTYPE_FLOAT32, "i8": cb.DTYPE_INT8}
 SEED = 0xA70CAD0
 # HBM bytes per launch of the body convolution kernel (read + written, average over the residual and non-residual launches of a
-# pass), from the FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/conv_tile_bf16_cfg2_hbm_traffic.md.  Counters
-# cannot be read from inside this process, so the figure is carried here; it is only reported for the dtype it was taken on.
-COUNTED_TRAFFIC_BYTES = {"bf16": 39.52e6}
+# pass), from the FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/winograd_rows_bf16_cfg2_hbm_traffic.md.  Counters
+# cannot be read from inside this process, so the figure is a CONSTANT carried here, not a measurement of this run; it is only
+# reported for the dtype it was taken on.
+COUNTED_TRAFFIC_BYTES = {"bf16": 40.27e6}
+LONG_CALL_REPLAYS = 4  # graph replays per timing for side-leg calls of 50 us and more (time_calls)
 
 
 class Hip:
@@ -288,9 +290,10 @@ def time_calls(hip, ctx, fn, iters, warmup=3):
     # ratios the detail reports (int8 over bf16) are quotients of two of them
     replays = max(2, iters // 2)
     if hip.time_graph(exe, stream, 1, warmup=1) > 0.5:
-        # calls of 50 us and more: four replays of the ten calls are plenty, and rocprofv3's kernel trace of this script ends
-        # in a segmentation fault inside hipGraphLaunch when ten replays of the 0.1-0.25 ms stages of config 3 are queued at once
-        replays = min(replays, 4)
+        # calls of 50 us and more: four replays of the ten calls (40 calls per timing) are plenty.  The cap is also what keeps
+        # this script runnable under rocprofv3's kernel trace, which ended in a segmentation fault inside hipGraphLaunch, in the
+        # tracer's own frames, with ten replays of the 0.1-0.25 ms stages of config 3 queued at once; untraced runs never failed.
+        replays = min(replays, LONG_CALL_REPLAYS)
     ms = sorted(hip.time_graph(exe, stream, replays) / 10 for _ in range(3))[1]
     ctx.synchronize()
     hip.rt.hipGraphExecDestroy(exe)
@@ -660,11 +663,18 @@ def main():
                    "global_batch": 256, "entry": "cudaConvolutionBiasActivationForward"},
         "roofline": {"bound": "mfma", "achieved": head["body_conv_tflops"], "peak": peak, "unit": "TFLOP/s", "frac": head["body_conv_tflops"] / peak,
                      "traffic": COUNTED_TRAFFIC_BYTES.get(args.dtype),
+                     "traffic_source": "constant from the committed FETCH_SIZE / WRITE_SIZE counter runs (profiles/), not measured in this run",
                      "kernel": "body 3x3 conv 128->128 (k_winograd_rows for 16-bit tensors: F(2,3) along rows, 12.885 GFLOP issued to the matrix cores "
                                "for the 16.987 GFLOP of the direct form): direct-equivalent flops / ((graph-replayed pass - stem) / 20) by HIP events"},
         "cpu_baseline": cpu,
         "detail": detail,
     }
+    # the same fraction by the flops the kernel really issues (the row-wise Winograd form needs 2/3 of the direct form's multiplies)
+    if args.dtype != "f32":
+        line["roofline"]["frac_of_peak_by_issued_flops"] = line["roofline"]["frac"] * 12.885 / 16.987
+    detail["timing"] = ("towers: median of 5 timings of `steps` graph replays each (min and max in ms_per_step_groups); single layers and stages: "
+                        "median of 3 timings of a graph of 10 calls, replayed max(2, steps // 2) times, %d times when a call takes 50 us or more"
+                        % LONG_CALL_REPLAYS)
     rates = detail.get("mfma_rate_measured")
     if rates is not None:
         # the same fraction against what the matrix cores of THIS box sustain on random operands with nothing else running
