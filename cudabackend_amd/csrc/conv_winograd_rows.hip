@@ -18,20 +18,24 @@
  * B^T = [1 0 -1 0; 0 1 1 0; 0 -1 1 0; 0 1 0 -1], G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1], A^T = [1 1 1 0; 0 1 -1 -1]
  * (the one-dimensional factors of the F(2x2,3x3) tables of src/winograd_nonfused.cu:534-575, signs moved between B and A).
  *
- * Workgroup = 8 wavefronts = one band of TH output rows of one image x 128 filters; GEMM rows are (row, column pair), at most
- * 128.  Wavefront (p, half) owns plane M_p for 64 filters: 4 x 2 MFMA tiles of 32 x 32, 128 accumulator registers.
- *   A operand: V_p lives in LDS, [slice of 64 channels][p][pixel = row * pairs + pair][128 bytes + 16], fp16; filter row i is
- *              a constant shift of i * pairs pixels, so a 32-row tile always reads 32 consecutive pixels (conflict-free).
+ * Workgroup = 8 wavefronts = one tile of TH output rows x `pairs` column pairs of one image x 128 filters; GEMM rows are
+ * (row, column pair), at most 128.  Wavefront (p, half) owns plane M_p for 64 filters: 4 x 2 MFMA tiles of 32 x 32, 128
+ * accumulator registers.
+ *   A operand: V_p lives in LDS, [phase slot][p][pixel = row * pairs + pair][128 bytes + 16], fp16; filter row i is a constant
+ *              shift of i * pairs pixels, so a 32-row tile always reads 32 consecutive pixels (conflict-free).
  *              V is produced in the kernel, 32 channels per phase: every work-item loads the four pixels of one
  *              (row, pair, 8 channels), forms the four differences in packed fp16 (bf16 is converted first: exact within the
- *              fp16 range) and writes them; the next phase is transformed while the current one is multiplied.
+ *              fp16 range) and writes them; the next phase is transformed among the MFMAs of the current one.
  *   B operand: U_p[i] comes straight from global memory (L2) in MFMA register layout, written that way by the weight
  *              transform below: [phase][filter row][p][tile of 32 filters][16-channel slab][lane][16 bytes], one contiguous
- *              kilobyte per wavefront load, requested two steps ahead.  No LDS, so no barrier inside a phase.
+ *              kilobyte per wavefront load, requested several slabs ahead through a ring of register sets.  No LDS, so no
+ *              barrier inside a phase.
  *   Epilogue : the planes go through LDS (two passes of 64 rows), a work-item folds four planes into two output pixels x 8
  *              filters, applies bias / residual / ReLU and stores 16 bytes per pixel.
- * Limits: 16-bit tensors, 3x3, stride 1, dilation 1, zero padding value, C = 64 or 128, K a multiple of 128, beta = 0,
- * LINEAR or RELU, image rows of at most 256 pixels that tile into bands (see choose_band), values within the fp16 range.
+ * C = 64 and 128 run with their 2 or 4 phases written out; C = 256 loops over two trips of four phases.
+ * Limits: 16-bit tensors, 3x3, stride 1, dilation 1, zero padding value, C = 64, 128 or 256, K a multiple of 128, beta = 0,
+ * LINEAR or RELU, images that tile into at most 128 (row, pair) positions per workgroup (see choose_tile), values within the
+ * fp16 range.
  */
 #include <atomic>
 
