@@ -95,7 +95,8 @@ KERNEL_LAYER_SYMBOLS = ["avhip_winograd_weight_transform", "avhip_winograd_input
                         "avhip_affine_forward", "avhip_batchnorm_inference", "avhip_stream_probe", "avhip_conv2d_winograd_rows",
                         "avhip_winograd_rows_weight_transform", "avhip_winograd_rows_weight_bytes", "avhip_conv2d_winograd_rows_plan",
                         "avhip_set_winograd_rows", "avhip_conv2d_strided", "avhip_conv2d_strided_weight_layout", "avhip_conv2d_strided_weight_bytes",
-                        "avhip_conv2d_strided_plan", "avhip_set_conv_strided"]
+                        "avhip_conv2d_strided_plan", "avhip_set_conv_strided", "avhip_conv2d_pointwise_block", "avhip_conv2d_pointwise_block_weight_layout",
+                        "avhip_conv2d_pointwise_block_weight_bytes", "avhip_conv2d_pointwise_block_plan", "avhip_set_pointwise_block"]
 
 _lib = None
 

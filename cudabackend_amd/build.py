@@ -29,6 +29,7 @@ SOURCES = [
     "conv_winograd_fused.hip",
     "conv_winograd_rows.hip",
     "conv_strided.hip",
+    "conv_pointwise_block.hip",
     "elementwise.hip",
 ]
 HEADERS = ["common.hpp", "mfma_core.hpp", "conv_epilogue.hpp", "conv_tile.hpp", "conv_small.hpp", "conv_stem.hpp", "conv_thin.hpp", "conv_pointwise.hpp", "persistent_gemm.hpp", "resident_gemm.hpp", "../../include/avocado_hip_kernels.h", "../../include/avocado_hip_backend.h",

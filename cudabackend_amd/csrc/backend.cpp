@@ -642,11 +642,12 @@ namespace
 		if (wm == nullptr || owner == nullptr || !owner->writes)
 			return AVOCADO_STATUS_BAD_PARAM;
 		const av_int64 offset = wm->data - owner->data;
-		const av_int64 w_bytes = static_cast<av_int64>(p.shape.K) * 9 * p.shape.C * size_of(p.w_dtype);
+		const av_int64 w_bytes = static_cast<av_int64>(p.shape.K) * p.shape.R * p.shape.S * p.shape.C * size_of(p.w_dtype);
 		const WeightKey key { owner->uid, offset, p.shape.K, p.shape.C, static_cast<int>(p.w_dtype), p.shape.mode, m };
 		const int t = m + 2;
 		const size_t bytes = m == 1 ? static_cast<size_t>(avhip_winograd_rows_weight_bytes(p.shape.K, p.shape.C))
 				: m == 3 ? static_cast<size_t>(avhip_conv2d_strided_weight_bytes(p.shape.K, p.shape.C))
+				: m == 5 ? static_cast<size_t>(avhip_conv2d_pointwise_block_weight_bytes(p.shape.K, p.shape.C))
 				: static_cast<size_t>(t * t) * p.shape.K * p.shape.C * size_of(mat_dtype);
 		WeightCache &cache = weight_cache();
 		std::vector<WeightEntry> victims;
@@ -715,6 +716,7 @@ namespace
 				e.seen = owner->writes->current();
 				const int rc = m == 1 ? avhip_winograd_rows_weight_transform(ctx.stream, p.w_dtype, p.shape.mode, wm->data, e.U, p.shape.K, p.shape.C)
 						: m == 3 ? avhip_conv2d_strided_weight_layout(ctx.stream, p.w_dtype, p.shape.mode, wm->data, e.U, p.shape.K, p.shape.C)
+						: m == 5 ? avhip_conv2d_pointwise_block_weight_layout(ctx.stream, p.w_dtype, wm->data, e.U, p.shape.K, p.shape.C)
 						: avhip_winograd_weight_transform(ctx.stream, p.w_dtype, mat_dtype, m, 3, p.shape.mode, wm->data, e.U, p.shape.K, p.shape.C);
 				status = from_launcher(rc);
 				cache.transforms++;
@@ -992,6 +994,36 @@ namespace
 		if (st != AVOCADO_STATUS_SUCCESS)
 			return st;
 		const int rc = avhip_conv2d_strided(c.ctx.stream, p.x_dtype, &p.shape, c.x->data, U, c.bias, c.z, c.y->data, c.alpha1, c.alpha2, c.beta, activation);
+		if (rc == AVHIP_NOT_SUPPORTED)
+			return AVOCADO_STATUS_NOT_SUPPORTED;
+		touch(yMem);
+		return from_launcher(rc);
+	}
+
+	/* 1x1 layers of 16-bit tensors with 128 or 256 channels and a multiple of 512 filters through the pixel-block kernel
+	 * (conv_pointwise_block.hip), weights in its operand layout from the cache (kind 5).  Worth it when its workgroups (one per
+	 * compute unit) cover most of the chip and most of their 224 GEMM rows are pixels. */
+	bool pointwise_block_pays(const ConvCall &c, avActivationType_t activation)
+	{
+		const ConvProblem &p = c.problem;
+		if (p.y_dtype != p.x_dtype || c.beta != 0.0 || (c.bias != nullptr && c.bias_dtype != AVOCADO_DTYPE_FLOAT32))
+			return false;
+		if (activation != AVOCADO_ACTIVATION_LINEAR && activation != AVOCADO_ACTIVATION_RELU)
+			return false;
+		int workgroups = 0, rows_used = 0;
+		if (avhip_conv2d_pointwise_block_plan(p.x_dtype, &p.shape, &workgroups, &rows_used) != 0)
+			return false;
+		return avhip_set_pointwise_block(-1) == 2 || (workgroups >= 192 && rows_used >= 160);
+	}
+	avStatus_t run_pointwise_block(const ConvCall &c, avMemoryDescriptor_t wMem, avMemoryDescriptor_t yMem, avActivationType_t activation)
+	{
+		const ConvProblem &p = c.problem;
+		const void *U = nullptr;
+		WeightLease lease;
+		const avStatus_t st = cached_winograd_weights(c.ctx, p, wMem, 5, p.w_dtype, &U, lease);
+		if (st != AVOCADO_STATUS_SUCCESS)
+			return st;
+		const int rc = avhip_conv2d_pointwise_block(c.ctx.stream, p.x_dtype, &p.shape, c.x->data, U, c.bias, c.z, c.y->data, c.alpha1, c.alpha2, c.beta, activation);
 		if (rc == AVHIP_NOT_SUPPORTED)
 			return AVOCADO_STATUS_NOT_SUPPORTED;
 		touch(yMem);
@@ -2028,6 +2060,12 @@ namespace avocado
 			if (strided_kernel_pays(call, activation))
 			{
 				const avStatus_t rs = run_strided_kernel(call, wMem, yMem, activation);
+				if (rs != AVOCADO_STATUS_NOT_SUPPORTED && rs != AVOCADO_STATUS_BAD_ALLOC)
+					return rs;
+			}
+			if (pointwise_block_pays(call, activation))
+			{
+				const avStatus_t rs = run_pointwise_block(call, wMem, yMem, activation);
 				if (rs != AVOCADO_STATUS_NOT_SUPPORTED && rs != AVOCADO_STATUS_BAD_ALLOC)
 					return rs;
 			}

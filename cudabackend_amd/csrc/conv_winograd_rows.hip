@@ -227,7 +227,13 @@ namespace
 		 * requested B_AHEAD slabs before they are multiplied: six sets where the kernel is written out, four where it loops (the
 		 * sixteen registers more do not fit there: three registers spilled cost more, 198 against 192 us on 64 x 56 x 56 x 256 -> 256,
 		 * than the shorter way ahead). */
-		constexpr int B_RING = PHASES <= MAX_PHASES ? 6 : 4, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
+		#ifndef ROWS_LOOPED_B_RING
+#define ROWS_LOOPED_B_RING 4
+#endif
+#ifndef ROWS_LOOPED_A_RING
+#define ROWS_LOOPED_A_RING 6
+#endif
+		constexpr int B_RING = PHASES <= MAX_PHASES ? 6 : ROWS_LOOPED_B_RING, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
 		Chunk bq[B_RING][2];
 		auto load_b = [&](int slab, Chunk (&set)[2]) __attribute__((always_inline)) /* slab: (step, slab of the step), over the whole k walk */
 		{
@@ -264,6 +270,10 @@ namespace
 		uint4 raw[4];
 		auto load_x = [&](int phase) __attribute__((always_inline))
 		{
+#ifdef ROWS_KNOCK_X /* timing experiment only: no pixel requests inside the k loop (wrong results) */
+			if (phase >= 2)
+				return;
+#endif
 			/* (an out-of-range offset stays out of range with the phase added: tensors here are below 2 GiB) */
 #pragma unroll
 			for (int j = 0; j < 4; j++)
@@ -331,7 +341,7 @@ namespace
 		typename Mma<f16_t>::acc_t acc[4][2];
 		/* A operands go through a ring of six register sets: the chunk four ahead of the one being multiplied is requested from LDS,
 		 * chunk = (phase, filter row, slab, 32-row tile) in the order of use */
-		constexpr int A_RING = 6, A_AHEAD = 4, STEP_CHUNKS_A = PHASE_SLABS * 4;
+		constexpr int A_RING = PHASES <= MAX_PHASES ? 6 : ROWS_LOOPED_A_RING, A_AHEAD = A_RING - 2, STEP_CHUNKS_A = PHASE_SLABS * 4;
 		Chunk a[A_RING];
 		/* (slot: which of the ring's places in LDS holds the phase) */
 		auto read_a = [&](int slot, int i, int sl, int rt, Chunk &dst) __attribute__((always_inline))

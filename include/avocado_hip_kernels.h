@@ -130,6 +130,21 @@ extern "C"
 	AVHIP_API int avhip_conv2d_strided_plan(int dtype, const avhipConvShape *shape, int *workgroups, int *rows_used);
 	AVHIP_API int avhip_set_conv_strided(int mode);
 
+	/* 1x1 stride-1 convolution without padding of fp16 / bf16 tensors with C = 128 or 256 and a multiple of 512 filters, beta = 0,
+	 * LINEAR or RELU: blocks of up to 224 pixels resident in LDS, filters from L2 in MFMA operand layout, results stored from the
+	 * accumulators without a pass through LDS (csrc/conv_pointwise_block.hip).  Same arithmetic as the reference's implicit GEMM,
+	 * src/conv2d_implicit_gemm.cu:303, for a 1x1 filter.  U is what avhip_conv2d_pointwise_block_weight_layout wrote:
+	 * avhip_conv2d_pointwise_block_weight_bytes(K, C) bytes, the weights themselves in the order [K / 32][C / 16][64 lanes][8]. */
+	AVHIP_API int avhip_conv2d_pointwise_block(void *stream, int dtype, const avhipConvShape *shape, const void *x, const void *U, const void *bias,
+			const void *z, void *y, double alpha1, double alpha2, double beta, int activation);
+	AVHIP_API int avhip_conv2d_pointwise_block_weight_layout(void *stream, int dtype, const void *w, void *U, int K, int C);
+	AVHIP_API int64_t avhip_conv2d_pointwise_block_weight_bytes(int K, int C);
+	/* Whether avhip_conv2d_pointwise_block takes the layer (0) or not (AVHIP_NOT_SUPPORTED), its workgroups and the pixels per
+	 * workgroup (of 224 GEMM rows); avhip_set_pointwise_block: 0 declines everything, 1 (default) lets the dispatcher weigh it, 2
+	 * makes the dispatcher take it wherever it can run; a negative mode only reads.  Returns the previous mode. */
+	AVHIP_API int avhip_conv2d_pointwise_block_plan(int dtype, const avhipConvShape *shape, int *workgroups, int *rows_used);
+	AVHIP_API int avhip_set_pointwise_block(int mode);
+
 	/* y = alpha1 * act(alpha2 * x + b + beta1 * z) + beta2 * z + beta3 * y.  Replaces kernel_add_bias,
 	 * src/tensor_op.cu:199-228.  x, y, z have `dtype`; b is fp32 (fp64 for fp64 tensors). */
 	AVHIP_API int avhip_add_bias(void *stream, int dtype, const void *x, const void *b, const void *z, void *y, int64_t first, int last, double alpha1,
