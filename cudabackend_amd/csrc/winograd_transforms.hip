@@ -165,7 +165,7 @@ namespace
 	 * cost more than the transform itself).  V > 1 instances are launched only when every vector is complete and aligned:
 	 * they have no tail handling, and outside the image they load from a clamped address and select the padding value, so
 	 * the whole work-item is branch-free and all its loads are in flight together. */
-	/* BUF instances (complete vectors, zero padding value, x below 2 GiB) fetch through a buffer descriptor: a pixel outside the image is
+	/* BUF instances (complete vectors of 4, 8 or 16 bytes, zero padding value, x below 2 GiB) fetch through a buffer descriptor: a pixel outside the image is
 	 * asked for at an out-of-range offset and comes back as zeros, so every load of the work-item is unconditional.  With ordinary
 	 * loads the compiler turns "load at a clamped address, then select the padding value" back into a branch around each load,
 	 * and where the element conversion is an instruction of its own (fp16) it ends up behind the branch with a wait in front of it: the
@@ -177,7 +177,7 @@ namespace
 		typedef typename Traits<T>::compute CT;
 		constexpr int t = M + R - 1;
 		constexpr bool FULL = V > 1;
-		static_assert(!BUF || (FULL && (sizeof(T) * V == 8 || sizeof(T) * V == 16) && sizeof(IDX) == 4), "whole 8- or 16-byte vectors, 32-bit offsets");
+		static_assert(!BUF || (FULL && (sizeof(T) * V == 4 || sizeof(T) * V == 8 || sizeof(T) * V == 16) && sizeof(IDX) == 4), "whole 4-, 8- or 16-byte vectors, 32-bit offsets");
 		const IDX CV = static_cast<IDX>((C + V - 1) / V);
 		const IDX tiles = static_cast<IDX>(N) * Th * Tw;
 		/* neighbouring tiles share input pixels: consecutive runs of tiles go to one XCD, whose L2 then serves the overlap */
@@ -212,8 +212,10 @@ namespace
 					const unsigned int offset = inside ? base + static_cast<unsigned int>((ih * W + iw) * C) * static_cast<unsigned int>(sizeof(T)) : OUT_OF_RANGE;
 					if constexpr (sizeof(T) * V == 16)
 						raw[a * t + b] = __builtin_bit_cast(Pack<T, V>, __builtin_amdgcn_raw_buffer_load_b128(rx, static_cast<int>(offset), 0, 0));
-					else
+					else if constexpr (sizeof(T) * V == 8)
 						raw[a * t + b] = __builtin_bit_cast(Pack<T, V>, __builtin_amdgcn_raw_buffer_load_b64(rx, static_cast<int>(offset), 0, 0));
+					else
+						raw[a * t + b] = __builtin_bit_cast(Pack<T, V>, __builtin_amdgcn_raw_buffer_load_b32(rx, static_cast<int>(offset), 0, 0));
 				}
 #pragma unroll
 			for (int i = 0; i < t * t; i++)
@@ -490,7 +492,7 @@ namespace
 		if (V > 1 && narrow && buffered)
 		{
 			constexpr int WIDTH = VecOf<M, R, T, TM>::value;
-			if constexpr (WIDTH > 1 && (sizeof(T) * WIDTH == 8 || sizeof(T) * WIDTH == 16))
+			if constexpr (WIDTH > 1 && (sizeof(T) * WIDTH == 4 || sizeof(T) * WIDTH == 8 || sizeof(T) * WIDTH == 16))
 				hipLaunchKernelGGL((k_input_transform<M, R, T, TM, WIDTH, uint32_t, true>), grid, dim3(256), 0, s, static_cast<const T*>(x), static_cast<TM*>(Vm), N, H, W,
 						C, Th, Tw, pad_h, pad_w, padv);
 			else
