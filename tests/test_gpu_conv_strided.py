@@ -77,6 +77,7 @@ CASES = [
     dict(x=(1, 112, 112, 64), w=(256, 3, 3, 64)),                                     # 56 x 56 outputs: tiles across and down
     dict(x=(2, 30, 9, 192), w=(256, 3, 3, 192), pad=(-2, -1)),                         # six phases, asymmetric offsets, narrow image
     dict(x=(2, 8, 8, 64), w=(256, 3, 3, 64)),                                         # an image much smaller than a tile
+    dict(x=(2, 16, 16, 64), w=(256, 3, 3, 64), bias=False, relu=False),                  # no bias, no activation: the accumulators as they are
 ]
 
 
@@ -91,7 +92,7 @@ def test_through_the_dispatcher(oracle, strided_forced, dtype, case):
     assert strided_forced.avhip_conv2d_strided_plan(h.DT[dtype], C.byref(s), None, None) == 0, "the kernel must take this layer"
     x = h.rounded(oracle, g.standard_normal(xs), dtype)
     w = he(g, ws, dtype, oracle)
-    b = g.uniform(-0.1, 0.1, ws[0]).astype(np.float32).astype(np.float64)
+    b = g.uniform(-0.1, 0.1, ws[0]).astype(np.float32).astype(np.float64) if cs.get("bias", True) else None
     ys = (xs[0], s.Ho, s.Wo, ws[0])
     z = h.rounded(oracle, g.standard_normal(ys), dtype) if cs.get("z") else None
     relu = cs.get("relu", True)

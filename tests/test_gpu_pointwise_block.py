@@ -75,6 +75,7 @@ CASES = [
     dict(x=(2, 9, 7, 256), w=(1024, 1, 1, 256), z=True, relu=False, alpha1=1.1, alpha2=1.2),  # one block of 126 pixels, two filter blocks
     dict(x=(1, 5, 5, 128), w=(512, 1, 1, 128)),                                           # 25 pixels: less than one MFMA tile
     dict(x=(2, 33, 31, 256), w=(512, 1, 1, 256), relu=False),                             # 2046 pixels: ten blocks, the last one short
+    dict(x=(2, 12, 12, 128), w=(512, 1, 1, 128), bias=False, relu=False),                 # no bias, no activation: the accumulators as they are
 ]
 
 
@@ -88,7 +89,7 @@ def test_through_the_dispatcher(oracle, block_forced, dtype, case):
     assert block_forced.avhip_conv2d_pointwise_block_plan(h.DT[dtype], C.byref(s), None, None) == 0, "the kernel must take this layer"
     x = h.rounded(oracle, g.standard_normal(xs), dtype)
     w = he(g, ws, dtype, oracle)
-    b = g.uniform(-0.1, 0.1, ws[0]).astype(np.float32).astype(np.float64)
+    b = g.uniform(-0.1, 0.1, ws[0]).astype(np.float32).astype(np.float64) if cs.get("bias", True) else None
     ys = (xs[0], s.Ho, s.Wo, ws[0])
     z = h.rounded(oracle, g.standard_normal(ys), dtype) if cs.get("z") else None
     relu = cs.get("relu", True)
