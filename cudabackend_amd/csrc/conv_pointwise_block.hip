@@ -118,8 +118,12 @@ namespace
 		const int tid = threadIdx.x;
 		const int lane = tid & 63;
 		const int wave = tid >> 6;
-		const int kb = static_cast<int>(blockIdx.y);
-		const int row0 = static_cast<int>(blockIdx.x) * g.rows;
+		/* the filter blocks of a pixel block follow each other on one XCD, whose L2 then holds the pixels for the second one */
+		unsigned int block = blockIdx.x, filter_block = 0;
+		if (gridDim.y != 1)
+			xcd_tile(block, filter_block);
+		const int kb = static_cast<int>(filter_block);
+		const int row0 = static_cast<int>(block) * g.rows;
 		const int rows = g.M - row0 < g.rows ? g.M - row0 : g.rows; /* real pixels of this block */
 
 		/* the block's pixels: work-item t takes 16-byte chunk t % CHUNKS_PER_ROW of rows t / CHUNKS_PER_ROW + k * SWEEP_ROWS; rows

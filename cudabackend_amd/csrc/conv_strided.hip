@@ -128,16 +128,19 @@ namespace
 		const int lane = tid & 63;
 		const int wave = tid >> 6; /* = this wavefront's tile of 32 filters */
 
-		int n = static_cast<int>(blockIdx.x), th = 0, tw = 0;
-		if (g.tiles_h * g.tiles_w != 1)
+		/* workgroups that share input (the filter blocks of a tile; neighbouring tiles of an image) follow each other on one XCD */
+		int n = static_cast<int>(blockIdx.x), th = 0, tw = 0, kb = 0;
+		if (g.tiles_h * g.tiles_w != 1 || gridDim.y != 1)
 		{
+			unsigned int item, filter_block;
+			xcd_tile(item, filter_block);
+			kb = static_cast<int>(filter_block);
 			const int per_image = g.tiles_h * g.tiles_w;
-			n = static_cast<int>(blockIdx.x) / per_image;
-			const int tile = static_cast<int>(blockIdx.x) - n * per_image;
+			n = static_cast<int>(item) / per_image;
+			const int tile = static_cast<int>(item) - n * per_image;
 			th = tile / g.tiles_w;
 			tw = tile - th * g.tiles_w;
 		}
-		const int kb = static_cast<int>(blockIdx.y);
 		const int oh0 = th * g.TH, ow0 = tw * g.TW;
 		const int ih0 = 2 * oh0 + g.pad_h, iw0 = 2 * ow0 + g.pad_w;
 

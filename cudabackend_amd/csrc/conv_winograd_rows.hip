@@ -198,17 +198,21 @@ namespace
 		const int p = wave & 3; /* plane of this wavefront */
 		const int fh = wave >> 2; /* its half of the 128 filters */
 
-		/* (image, band, segment): the tiles of an image are neighbours in the grid; the filter block is the slow index */
-		int n = static_cast<int>(blockIdx.x), band = 0, segment = 0;
-		if (g.bands * g.segments != 1)
+		/* (image, band, segment) and filter block.  Where workgroups share input (several tiles per image: neighbouring bands
+		 * read two rows in common; several filter blocks: each reads the whole tile) they are renumbered so that the filter
+		 * blocks of a tile and then the tiles of an image follow each other on one XCD, whose L2 then serves the second reader. */
+		int n = static_cast<int>(blockIdx.x), band = 0, segment = 0, kb = 0;
+		if (g.bands * g.segments != 1 || gridDim.y != 1)
 		{
+			unsigned int item, filter_block;
+			xcd_tile(item, filter_block);
+			kb = static_cast<int>(filter_block);
 			const int per_image = g.bands * g.segments;
-			n = static_cast<int>(blockIdx.x) / per_image;
-			const int tile = static_cast<int>(blockIdx.x) - n * per_image;
+			n = static_cast<int>(item) / per_image;
+			const int tile = static_cast<int>(item) - n * per_image;
 			band = tile / g.segments;
 			segment = tile - band * g.segments;
 		}
-		const int kb = static_cast<int>(blockIdx.y);
 		const int oh0 = band * g.TH;
 		const int ow0 = segment * 2 * g.pairs;
 		const int ih0 = oh0 + g.pad_h; /* input row of V row 0 */
