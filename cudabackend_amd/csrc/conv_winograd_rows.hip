@@ -231,17 +231,24 @@ namespace
 		 * requested B_AHEAD slabs before they are multiplied: six sets where the kernel is written out, four where it loops (the
 		 * sixteen registers more do not fit there: three registers spilled cost more, 198 against 192 us on 64 x 56 x 56 x 256 -> 256,
 		 * than the shorter way ahead). */
-		#ifndef ROWS_LOOPED_B_RING
+		#ifndef ROWS_B_RING
+#define ROWS_B_RING 6 /* (4 and 8 measure the same: the way ahead is not what the requests cost) */
+#endif
+#ifndef ROWS_LOOPED_B_RING
 #define ROWS_LOOPED_B_RING 4
 #endif
 #ifndef ROWS_LOOPED_A_RING
 #define ROWS_LOOPED_A_RING 6
 #endif
-		constexpr int B_RING = PHASES <= MAX_PHASES ? 6 : ROWS_LOOPED_B_RING, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
+		constexpr int B_RING = PHASES <= MAX_PHASES ? ROWS_B_RING : ROWS_LOOPED_B_RING, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
 		Chunk bq[B_RING][2];
 		auto load_b = [&](int slab, Chunk (&set)[2]) __attribute__((always_inline)) /* slab: (step, slab of the step), over the whole k walk */
 		{
 			const int step = slab / PHASE_SLABS, sl = slab - step * PHASE_SLABS;
+#ifdef ROWS_KNOCK_B /* timing experiment only: no filter requests inside the k loop (wrong results) */
+			if (slab >= B_AHEAD)
+				return;
+#endif
 #pragma unroll
 			for (int tn = 0; tn < 2; tn++)
 			{
@@ -420,11 +427,15 @@ namespace
 #pragma unroll
 					for (int sl = 0; sl < PHASE_SLABS; sl++)
 					{
-						if (LOOPED || step * PHASE_SLABS + sl + B_AHEAD < SLABS_TOTAL)
-							__builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+						/* (the slab's two requests half a slab apart: 1 % better than back to back) */
+						const bool requests = LOOPED || step * PHASE_SLABS + sl + B_AHEAD < SLABS_TOTAL;
+						if (requests)
+							__builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
 #pragma unroll
 						for (int k = 0; k < 8; k++)
 						{
+							if (requests && k == 4)
+								__builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
 							__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 							if (transform_here)
 							{
