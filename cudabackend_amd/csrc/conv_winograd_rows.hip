@@ -228,19 +228,17 @@ namespace
 		const __amdgpu_buffer_rsrc_t ru = make_buffer(U, static_cast<unsigned int>(STEPS) * step_stride);
 		const unsigned int b_offset = static_cast<unsigned int>((p * g.filter_tiles + kb * 4 + fh * 2) * PHASE_SLABS * OPERAND_BYTES + lane * 16);
 		/* Filters go through a ring of register sets, one set = the two filter tiles of one 16-channel slab (two slabs per step),
-		 * requested B_AHEAD slabs before they are multiplied: six sets where the kernel is written out, four where it loops (the
+		 * requested B_AHEAD slabs before they are multiplied: six sets where the kernel is written out (one phase's worth, which is
+		 * what its last phase keeps in registers; rings of four and eight measured the same), four where it loops (the
 		 * sixteen registers more do not fit there: three registers spilled cost more, 198 against 192 us on 64 x 56 x 56 x 256 -> 256,
 		 * than the shorter way ahead). */
-		#ifndef ROWS_B_RING
-#define ROWS_B_RING 6 /* (4 and 8 measure the same: the way ahead is not what the requests cost) */
-#endif
-#ifndef ROWS_LOOPED_B_RING
+		#ifndef ROWS_LOOPED_B_RING
 #define ROWS_LOOPED_B_RING 4
 #endif
 #ifndef ROWS_LOOPED_A_RING
 #define ROWS_LOOPED_A_RING 6
 #endif
-		constexpr int B_RING = PHASES <= MAX_PHASES ? ROWS_B_RING : ROWS_LOOPED_B_RING, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
+		constexpr int B_RING = PHASES <= MAX_PHASES ? FILTER_ROWS * PHASE_SLABS : ROWS_LOOPED_B_RING, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
 		Chunk bq[B_RING][2];
 		auto load_b = [&](int slab, Chunk (&set)[2]) __attribute__((always_inline)) /* slab: (step, slab of the step), over the whole k walk */
 		{
@@ -369,12 +367,13 @@ namespace
 		auto run_phases = [&](auto looped, int first) __attribute__((always_inline))
 		{
 			constexpr bool LOOPED = decltype(looped)::value;
-			constexpr int COUNT = LOOPED ? RING : PHASES;
+			/* (written out, the last phase is not one of these: it walks its products row tile by row tile, see below) */
+			constexpr int COUNT = LOOPED ? RING : PHASES - 1;
 			constexpr int CHUNKS = COUNT * FILTER_ROWS * STEP_CHUNKS_A;
 #pragma unroll
 			for (int phase = 0; phase < COUNT; phase++)
 			{
-				const bool more = LOOPED || phase + 1 < COUNT; /* another phase follows */
+				const bool more = true; /* another phase follows */
 #pragma unroll
 				for (int i = 0; i < FILTER_ROWS; i++)
 				{
@@ -448,7 +447,7 @@ namespace
 					if (transform_here)
 					{
 						__builtin_amdgcn_sched_barrier(0);
-						if (LOOPED || phase + 2 < COUNT)
+						if (LOOPED || phase + 2 < PHASES)
 						{
 							const int next = first + phase + 2;
 							load_x(LOOPED ? (next < PHASES ? next : PHASES - 1) : next);
@@ -461,8 +460,153 @@ namespace
 #pragma unroll
 		for (int c = 0; c < A_AHEAD; c++)
 			read_a(0, 0, c / 4, c % 4, a[c]);
+		/* the fold buffer: [plane][row][128 filters + 4] floats, a row holding the filters as [first halves | second halves] of the 16
+		 * runs of 8 filters a work-item stores: run g, half h at word h * 64 + g * 4, so that sixteen lanes reading the same half of
+		 * sixteen runs touch 64 consecutive words (every bank once).  A lane's accumulator registers 4i..4i+3 of tile (rt, tn) are
+		 * filters fh * 64 + tn * 32 + 8i + 4 * (lane / 32) + 0..3 of GEMM row 32 rt + lane % 32: run fh * 8 + tn * 4 + i, half lane / 32. */
+		typedef float quad_t __attribute__((ext_vector_type(4)));
+		const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
+		__amdgpu_buffer_rsrc_t rz = make_buffer(nullptr, 0);
+		if (epi.z != nullptr)
+			rz = make_buffer(epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
+		const bool relu = epi.activation == ACT_RELU, has_z = epi.z != nullptr;
 		if constexpr (PHASES <= RING)
+		{
 			run_phases(std::false_type(), 0);
+			/*
+			 * The last phase, and the results out while it runs.  Its filters (six slabs, the whole ring) stay in registers and its
+			 * products are taken row tile by row tile, so that the sums of row tile 0 are final after a quarter of the phase: they go
+			 * through LDS (32 rows of four planes: the half of LDS that the last phase does not read), are folded and stored while
+			 * the matrix cores work on row tile 1, and so on.  The stores of three quarters of the tile are then under way before
+			 * the loop has ended, and what is left behind it is one quarter's hand-over instead of two passes over the whole tile.
+			 */
+			constexpr int LAST = PHASES - 1, LAST_SLAB = LAST * FILTER_ROWS * PHASE_SLABS, PASS_ROWS = 32;
+			static_assert(B_RING == FILTER_ROWS * PHASE_SLABS && POSITIONS * PASS_ROWS * FOLD_PITCH * 4 <= SLICE_BYTES, "one phase of filters in the ring; the fold buffer in one slice");
+			float *sm = reinterpret_cast<float*>(lds + ((LAST % RING) >> 1 == 0 ? SLICE_BYTES : 0));
+			STAMP(5);
+			load_b(LAST_SLAB + B_AHEAD, bq[(LAST_SLAB + B_AHEAD) % B_RING]);
+			typename FloatEpilogue<TE>::template ColumnsT<8> columns;
+			epi.request_columns(kcol, columns);
+			/* this work-item's (row, pair) of a pass: where its two output pixels go, and their residual */
+			unsigned int y_off[2][2];
+			typename FloatEpilogue<TE>::template Residual<8> residual[2][2];
+			auto place = [&](int pass) __attribute__((always_inline))
+			{
+				const int q = pass * PASS_ROWS + (tid >> 4);
+				const int r = static_cast<int>((static_cast<unsigned int>(q) * g.pairs_magic) >> 20);
+				const int pair = q - r * g.pairs;
+				const int oh = oh0 + r;
+				const bool row_ok = (q < band_rows) & (oh < g.Ho) & (kcol < g.K);
+#pragma unroll
+				for (int o = 0; o < 2; o++)
+				{
+					const int ow = ow0 + 2 * pair + o;
+					y_off[pass & 1][o] = (row_ok & (ow < g.Wo)) ? static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ : OUT_OF_RANGE;
+					union
+					{
+						uint4 u;
+						decltype(residual[0][0].raw) r8;
+					} cast;
+					cast.u = buffer_fetch<2>(rz, y_off[pass & 1][o]);
+					residual[pass & 1][o].raw = cast.r8;
+				}
+			};
+			auto fold_and_store = [&](int pass, auto with_relu, auto with_z) __attribute__((always_inline))
+			{
+				quad_t m[POSITIONS][2];
+#pragma unroll
+				for (int q = 0; q < POSITIONS; q++)
+#pragma unroll
+					for (int part = 0; part < 2; part++)
+						m[q][part] = *reinterpret_cast<const quad_t*>(sm + (q * PASS_ROWS + (tid >> 4)) * FOLD_PITCH + part * 64 + (tid & 15) * 4);
+				float out[2][8];
+#pragma unroll
+				for (int c = 0; c < 8; c++)
+				{
+					const float m0 = m[0][c >> 2][c & 3], m1 = m[1][c >> 2][c & 3], m2 = m[2][c >> 2][c & 3], m3 = m[3][c >> 2][c & 3];
+					out[0][c] = m0 + m1 + m2;
+					out[1][c] = m1 - m2 - m3;
+				}
+#pragma unroll
+				for (int o = 0; o < 2; o++)
+				{
+					const unsigned int offset = y_off[pass & 1][o];
+					epi.template store_fast<decltype(with_relu)::value, decltype(with_z)::value, 8>(out[o], columns, residual[pass & 1][o], [&](auto words) __attribute__((always_inline))
+					{
+						buffer_put<ROWS_STORE_POLICY>(ry, offset, words);
+					});
+				}
+			};
+			place(0);
+#pragma unroll
+			for (int c = 0; c < A_AHEAD; c++)
+				read_a(LAST % RING, (c / PHASE_SLABS) % FILTER_ROWS, c % PHASE_SLABS, c / (FILTER_ROWS * PHASE_SLABS), a[c % A_RING]); /* chunk = (row tile, filter row, slab) */
+			auto fold_pass = [&](int pass) __attribute__((always_inline))
+			{
+				if (relu && has_z)
+					fold_and_store(pass, std::true_type(), std::true_type());
+				else if (relu)
+					fold_and_store(pass, std::true_type(), std::false_type());
+				else if (has_z)
+					fold_and_store(pass, std::false_type(), std::true_type());
+				else
+					fold_and_store(pass, std::false_type(), std::false_type());
+			};
+#pragma unroll
+			for (int rt = 0; rt < 4; rt++)
+			{
+				/* one scheduling region: the products of row tile rt, and among them the fold and the stores of row tile rt - 1,
+				 * whose sums the barrier behind the previous region has made visible */
+				__builtin_amdgcn_sched_barrier(0);
+				if (rt > 0)
+				{
+					fold_pass(rt - 1);
+					place(rt);
+				}
+#pragma unroll
+				for (int i = 0; i < FILTER_ROWS; i++)
+#pragma unroll
+					for (int sl = 0; sl < PHASE_SLABS; sl++)
+					{
+						const int c = (rt * FILTER_ROWS + i) * PHASE_SLABS + sl, cn = c + A_AHEAD;
+						if (cn < 4 * FILTER_ROWS * PHASE_SLABS)
+							read_a(LAST % RING, (cn / PHASE_SLABS) % FILTER_ROWS, cn % PHASE_SLABS, cn / (FILTER_ROWS * PHASE_SLABS), a[cn % A_RING]);
+#pragma unroll
+						for (int tn = 0; tn < 2; tn++)
+							Mma<f16_t>::run(bq[(LAST_SLAB + i * PHASE_SLABS + sl) % B_RING][tn], a[c % A_RING], acc[rt][tn]);
+					}
+				if (rt > 0)
+					__builtin_amdgcn_sched_group_barrier(0x100, 8, 0); /* the eight reads of the fold first */
+#pragma unroll
+				for (int k = 0; k < FILTER_ROWS * PHASE_SLABS; k++)
+				{
+					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+					__builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+					if (rt > 0)
+						__builtin_amdgcn_sched_group_barrier(0x002, 12, 0);
+				}
+				__builtin_amdgcn_sched_barrier(0);
+				if (rt == 0)
+					STAMP(6);
+				if (rt == 3)
+					STAMP(7);
+				/* row tile rt is final: out through LDS (everyone has folded the previous row tile: its values were consumed above) */
+				if (rt > 0)
+					__syncthreads();
+#pragma unroll
+				for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+					for (int i = 0; i < 4; i++)
+					{
+						const typename Mma<f16_t>::acc_t &t = acc[rt][tn];
+						const quad_t run = { t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3] };
+						*reinterpret_cast<quad_t*>(sm + (p * PASS_ROWS + (lane & 31)) * FOLD_PITCH + (lane >> 5) * 64 + (fh * 8 + tn * 4 + i) * 4) = run;
+					}
+				__syncthreads();
+			}
+			fold_pass(3);
+			STAMP(3);
+		}
 		else
 		{
 			static_assert(PHASES % RING == 0 && (RING * FILTER_ROWS * PHASE_SLABS) % B_RING == 0 && (RING * FILTER_ROWS * STEP_CHUNKS_A) % A_RING == 0,
@@ -479,14 +623,11 @@ namespace
 				run_phases(std::true_type(), first);
 		}
 
+		if constexpr (PHASES > RING)
+		{
 		STAMP(3);
 		/* fold and store: two passes of 64 GEMM rows; a work-item takes (row, 8 filters) twice per pass */
 		float *sm = reinterpret_cast<float*>(lds);
-		const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
-		__amdgpu_buffer_rsrc_t rz = make_buffer(nullptr, 0);
-		if (epi.z != nullptr)
-			rz = make_buffer(epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
-		const bool relu = epi.activation == ACT_RELU, has_z = epi.z != nullptr;
 		/* per-filter constants of the epilogue (requested here and not before the k loop, where eight more live registers are eight
 		 * too many; the fold through LDS hides the latency) */
 		typename FloatEpilogue<TE>::template ColumnsT<8> columns;
@@ -524,7 +665,6 @@ namespace
 			__syncthreads(); /* pass 0: everyone is done with V; pass 1: with the planes of pass 0 */
 			if (pass == 0)
 				STAMP(5);
-			typedef float quad_t __attribute__((ext_vector_type(4)));
 #ifndef ROWS_KNOCK_LDS
 			/* A row of the fold buffer holds the 128 filters of a pixel as [first halves | second halves] of the 16 runs of 8
 			 * filters a work-item stores: run g, half h sits at word h * 64 + g * 4, so that sixteen lanes reading the same half of
@@ -599,6 +739,7 @@ namespace
 				leave(std::false_type(), std::false_type());
 			if (pass == 0)
 				STAMP(7);
+		}
 		}
 		STAMP(4);
 	}
