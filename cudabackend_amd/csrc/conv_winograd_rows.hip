@@ -30,9 +30,10 @@
  *              transform below: [phase][filter row][p][tile of 32 filters][16-channel slab][lane][16 bytes], one contiguous
  *              kilobyte per wavefront load, requested several slabs ahead through a ring of register sets.  No LDS, so no
  *              barrier inside a phase.
- *   Epilogue : the planes go through LDS (two passes of 64 rows), a work-item folds four planes into two output pixels x 8
- *              filters, applies bias / residual / ReLU and stores 16 bytes per pixel.
- * C = 64 and 128 run with their 2 or 4 phases written out; C = 256 loops over two trips of four phases.
+ *   Epilogue : runs inside the last phase.  That phase keeps its filters in registers and takes its products row tile by row
+ *              tile; a finished row tile's four planes go through LDS (32 rows), a work-item folds them into two output pixels x
+ *              8 filters, applies bias / residual / ReLU and stores 16 bytes per pixel while the next row tile is multiplied.
+ * All phases are written out (2, 4 or 8 for C = 64, 128, 256); V has four slots in LDS, a fifth phase takes the first slot again.
  * Limits: 16-bit tensors, 3x3, stride 1, dilation 1, zero padding value, C = 64, 128 or 256, K a multiple of 128, beta = 0,
  * LINEAR or RELU, images that tile into at most 128 (row, pair) positions per workgroup (see choose_tile), values within the
  * fp16 range.
@@ -78,10 +79,8 @@ namespace
 	constexpr int ROWS_BLOCK_N = 128; /* filters per workgroup */
 	constexpr int THREADS = 512;
 	constexpr int OPERAND_BYTES = 1024; /* one MFMA operand of a wavefront: 64 lanes x 16 bytes */
-	/* epilogue: [plane][64 rows][128 filters + 4] floats */
-	constexpr int FOLD_ROWS = 64;
+	/* epilogue: [plane][32 rows][128 filters + 4] floats per row tile, in the slice of LDS that the last phase does not read */
 	constexpr int FOLD_PITCH = ROWS_BLOCK_N + 4;
-	static_assert(POSITIONS * FOLD_ROWS * FOLD_PITCH * 4 <= V_BYTES, "the fold reuses the LDS of V");
 	static_assert(V_BYTES <= 160 * 1024, "LDS of a compute unit");
 
 	struct RowsGeom
@@ -228,17 +227,9 @@ namespace
 		const __amdgpu_buffer_rsrc_t ru = make_buffer(U, static_cast<unsigned int>(STEPS) * step_stride);
 		const unsigned int b_offset = static_cast<unsigned int>((p * g.filter_tiles + kb * 4 + fh * 2) * PHASE_SLABS * OPERAND_BYTES + lane * 16);
 		/* Filters go through a ring of register sets, one set = the two filter tiles of one 16-channel slab (two slabs per step),
-		 * requested B_AHEAD slabs before they are multiplied: six sets where the kernel is written out (one phase's worth, which is
-		 * what its last phase keeps in registers; rings of four and eight measured the same), four where it loops (the
-		 * sixteen registers more do not fit there: three registers spilled cost more, 198 against 192 us on 64 x 56 x 56 x 256 -> 256,
-		 * than the shorter way ahead). */
-		#ifndef ROWS_LOOPED_B_RING
-#define ROWS_LOOPED_B_RING 4
-#endif
-#ifndef ROWS_LOOPED_A_RING
-#define ROWS_LOOPED_A_RING 6
-#endif
-		constexpr int B_RING = PHASES <= MAX_PHASES ? FILTER_ROWS * PHASE_SLABS : ROWS_LOOPED_B_RING, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
+		 * requested B_AHEAD slabs before they are multiplied: six sets, one phase's worth, which is what the last phase keeps in
+		 * registers (rings of four and eight measured the same: the way ahead is not what the requests cost). */
+		constexpr int B_RING = FILTER_ROWS * PHASE_SLABS, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
 		Chunk bq[B_RING][2];
 		auto load_b = [&](int slab, Chunk (&set)[2]) __attribute__((always_inline)) /* slab: (step, slab of the step), over the whole k walk */
 		{
@@ -350,30 +341,22 @@ namespace
 		typename Mma<f16_t>::acc_t acc[4][2];
 		/* A operands go through a ring of six register sets: the chunk four ahead of the one being multiplied is requested from LDS,
 		 * chunk = (phase, filter row, slab, 32-row tile) in the order of use */
-		constexpr int A_RING = PHASES <= MAX_PHASES ? 6 : ROWS_LOOPED_A_RING, A_AHEAD = A_RING - 2, STEP_CHUNKS_A = PHASE_SLABS * 4;
+		constexpr int A_RING = 6, A_AHEAD = 4, STEP_CHUNKS_A = PHASE_SLABS * 4;
 		Chunk a[A_RING];
 		/* (slot: which of the ring's places in LDS holds the phase) */
 		auto read_a = [&](int slot, int i, int sl, int rt, Chunk &dst) __attribute__((always_inline))
 		{
 			dst.u = *reinterpret_cast<const uint4*>(lds + (slot >> 1) * SLICE_BYTES + (slot & 1) * 64 + sl * 32 + i * tap_shift + rt * 32 * PITCH + a_off);
 		};
-		/*
-		 * The phases of one trip: all PHASES of them when they fit the ring (LOOPED false: written out once, the last phase without
-		 * the work for a next one), else RING of them per trip of a loop that stays a loop (LOOPED: the same code for every trip, which
-		 * keeps the registers of a layer with 256 channels where those of one with 128 are; after the last phase it requests, transforms
-		 * and reads ahead for a phase that does not exist: it asks for the last phase again, and the slot it writes is one that nobody
-		 * reads any more).  `first`: global number of the trip's first phase.
-		 */
-		auto run_phases = [&](auto looped, int first) __attribute__((always_inline))
+		/* All phases but the last, written out (the last one walks its products row tile by row tile, see below).  With more
+		 * phases than LDS has slots a phase's V takes the slot of phase - RING, whose readers are long gone (above). */
+		auto run_phases = [&]() __attribute__((always_inline))
 		{
-			constexpr bool LOOPED = decltype(looped)::value;
-			/* (written out, the last phase is not one of these: it walks its products row tile by row tile, see below) */
-			constexpr int COUNT = LOOPED ? RING : PHASES - 1;
+			constexpr int COUNT = PHASES - 1;
 			constexpr int CHUNKS = COUNT * FILTER_ROWS * STEP_CHUNKS_A;
 #pragma unroll
 			for (int phase = 0; phase < COUNT; phase++)
 			{
-				const bool more = true; /* another phase follows */
 #pragma unroll
 				for (int i = 0; i < FILTER_ROWS; i++)
 				{
@@ -382,18 +365,18 @@ namespace
 					/* The next phase's V, from pixels requested a phase ago, is formed among the MFMAs of the middle step and made
 					 * visible by a barrier before the last one, so that the last step can read the first operands of the next phase
 					 * ahead like any other: no phase starts with a barrier and a bare LDS latency. */
-					const bool transform_here = i == 1 && more;
-					if (i == 2 && more)
+					const bool transform_here = i == 1;
+					if (i == 2)
 						__syncthreads();
 #pragma unroll
 					for (int sl = 0; sl < PHASE_SLABS; sl++)
 					{
 						const int slab = step * PHASE_SLABS + sl; /* within the trip */
-						if (LOOPED || slab + B_AHEAD < SLABS_TOTAL)
+						if (slab + B_AHEAD < SLABS_TOTAL)
 						{
 							/* (a scalar offset is not part of a buffer's bounds check: slabs past the last ask for the last again) */
-							const int ahead = first * FILTER_ROWS * PHASE_SLABS + slab + B_AHEAD;
-							load_b(LOOPED ? (ahead < SLABS_TOTAL ? ahead : SLABS_TOTAL - 1) : ahead, bq[(slab + B_AHEAD) % B_RING]);
+							const int ahead = slab + B_AHEAD;
+							load_b(ahead, bq[(slab + B_AHEAD) % B_RING]);
 						}
 						if (transform_here && sl == 0)
 							transform((phase + 1) % RING);
@@ -402,17 +385,17 @@ namespace
 						{
 							const int c = (step * PHASE_SLABS + sl) * 4 + rt;
 							const int cn = c + A_AHEAD; /* the chunk to request now */
-							if (cn < CHUNKS || LOOPED)
+							if (cn < CHUNKS)
 							{
-								const int nstep = (cn / STEP_CHUNKS_A) % (COUNT * FILTER_ROWS), nphase = cn < CHUNKS ? nstep / FILTER_ROWS : COUNT;
-								read_a(nphase % RING, cn < CHUNKS ? nstep % FILTER_ROWS : 0, (cn / 4) % PHASE_SLABS, cn % 4, a[cn % A_RING]);
+								const int nstep = cn / STEP_CHUNKS_A, nphase = nstep / FILTER_ROWS;
+								read_a(nphase % RING, nstep % FILTER_ROWS, (cn / 4) % PHASE_SLABS, cn % 4, a[cn % A_RING]);
 							}
 #pragma unroll
 							for (int tn = 0; tn < 2; tn++)
 							{
 								/* filters as the rows of the MFMA tile, pixels as its columns: a lane then holds runs of four
 								 * consecutive filters of one pixel, which the fold can move as 16-byte vectors */
-								if (!LOOPED && step == 0 && sl == 0)
+								if (step == 0 && sl == 0)
 									Mma<f16_t>::start(bq[slab % B_RING][tn], a[c % A_RING], acc[rt][tn]);
 								else
 									Mma<f16_t>::run(bq[slab % B_RING][tn], a[c % A_RING], acc[rt][tn]);
@@ -427,7 +410,7 @@ namespace
 					for (int sl = 0; sl < PHASE_SLABS; sl++)
 					{
 						/* (the slab's two requests half a slab apart: 1 % better than back to back) */
-						const bool requests = LOOPED || step * PHASE_SLABS + sl + B_AHEAD < SLABS_TOTAL;
+						const bool requests = step * PHASE_SLABS + sl + B_AHEAD < SLABS_TOTAL;
 						if (requests)
 							__builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
 #pragma unroll
@@ -447,10 +430,10 @@ namespace
 					if (transform_here)
 					{
 						__builtin_amdgcn_sched_barrier(0);
-						if (LOOPED || phase + 2 < PHASES)
+						if (phase + 2 < PHASES)
 						{
-							const int next = first + phase + 2;
-							load_x(LOOPED ? (next < PHASES ? next : PHASES - 1) : next);
+							const int next = phase + 2;
+							load_x(next);
 						}
 					}
 				}
@@ -470,9 +453,8 @@ namespace
 		if (epi.z != nullptr)
 			rz = make_buffer(epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
 		const bool relu = epi.activation == ACT_RELU, has_z = epi.z != nullptr;
-		if constexpr (PHASES <= RING)
 		{
-			run_phases(std::false_type(), 0);
+			run_phases();
 			/*
 			 * The last phase, and the results out while it runs.  Its filters (six slabs, the whole ring) stay in registers and its
 			 * products are taken row tile by row tile, so that the sums of row tile 0 are final after a quarter of the phase: they go
@@ -606,140 +588,6 @@ namespace
 			}
 			fold_pass(3);
 			STAMP(3);
-		}
-		else
-		{
-			static_assert(PHASES % RING == 0 && (RING * FILTER_ROWS * PHASE_SLABS) % B_RING == 0 && (RING * FILTER_ROWS * STEP_CHUNKS_A) % A_RING == 0,
-					"whole trips, and the operand rings in the same position at the start of each");
-#pragma unroll
-			for (int rt = 0; rt < 4; rt++)
-#pragma unroll
-				for (int tn = 0; tn < 2; tn++)
-#pragma unroll
-					for (int v = 0; v < 16; v++)
-						acc[rt][tn][v] = 0.0f;
-#pragma unroll 1
-			for (int first = 0; first < PHASES; first += RING)
-				run_phases(std::true_type(), first);
-		}
-
-		if constexpr (PHASES > RING)
-		{
-		STAMP(3);
-		/* fold and store: two passes of 64 GEMM rows; a work-item takes (row, 8 filters) twice per pass */
-		float *sm = reinterpret_cast<float*>(lds);
-		/* per-filter constants of the epilogue (requested here and not before the k loop, where eight more live registers are eight
-		 * too many; the fold through LDS hides the latency) */
-		typename FloatEpilogue<TE>::template ColumnsT<8> columns;
-		epi.request_columns(kcol, columns);
-		/* where this work-item's two rows of either pass go, and their residual, requested before the planes go through LDS */
-		unsigned int y_off[2][2][2];
-		typename FloatEpilogue<TE>::template Residual<8> residual[2][2][2];
-#pragma unroll
-		for (int pass = 0; pass < 2; pass++)
-#pragma unroll
-			for (int it = 0; it < 2; it++)
-			{
-				const int q = pass * FOLD_ROWS + (tid >> 4) + it * (THREADS / 16);
-				const int r = static_cast<int>((static_cast<unsigned int>(q) * g.pairs_magic) >> 20);
-				const int pair = q - r * g.pairs;
-				const int oh = oh0 + r;
-				const bool row_ok = (q < band_rows) & (oh < g.Ho) & (kcol < g.K);
-#pragma unroll
-				for (int o = 0; o < 2; o++)
-				{
-					const int ow = ow0 + 2 * pair + o;
-					y_off[pass][it][o] = (row_ok & (ow < g.Wo)) ? static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ : OUT_OF_RANGE;
-					union
-					{
-						uint4 u;
-						decltype(residual[0][0][0].raw) r8;
-					} cast;
-					cast.u = buffer_fetch<2>(rz, y_off[pass][it][o]);
-					residual[pass][it][o].raw = cast.r8;
-				}
-			}
-#pragma unroll
-		for (int pass = 0; pass < 2; pass++)
-		{
-			__syncthreads(); /* pass 0: everyone is done with V; pass 1: with the planes of pass 0 */
-			if (pass == 0)
-				STAMP(5);
-#ifndef ROWS_KNOCK_LDS
-			/* A row of the fold buffer holds the 128 filters of a pixel as [first halves | second halves] of the 16 runs of 8
-			 * filters a work-item stores: run g, half h sits at word h * 64 + g * 4, so that sixteen lanes reading the same half of
-			 * sixteen runs touch 64 consecutive words (every bank once).  This lane's accumulator registers 4i..4i+3 are filters
-			 * fh * 64 + tn * 32 + 8i + 4 * (lane / 32) + 0..3 of pixel (lane % 32): run fh * 8 + tn * 4 + i, half (lane / 32). */
-#pragma unroll
-			for (int rt = 0; rt < 2; rt++)
-#pragma unroll
-				for (int tn = 0; tn < 2; tn++)
-#pragma unroll
-					for (int i = 0; i < 4; i++)
-					{
-						const typename Mma<f16_t>::acc_t &t = acc[pass * 2 + rt][tn];
-						const quad_t run = { t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3] };
-						*reinterpret_cast<quad_t*>(sm + (p * FOLD_ROWS + rt * 32 + (lane & 31)) * FOLD_PITCH + (lane >> 5) * 64 + (fh * 8 + tn * 4 + i) * 4) = run;
-					}
-			__syncthreads();
-#endif
-			if (pass == 0)
-				STAMP(6);
-			quad_t m[2][POSITIONS][2];
-#pragma unroll
-			for (int it = 0; it < 2; it++)
-#pragma unroll
-				for (int q = 0; q < POSITIONS; q++)
-#pragma unroll
-					for (int part = 0; part < 2; part++)
-#ifndef ROWS_KNOCK_LDS
-						m[it][q][part] = *reinterpret_cast<const quad_t*>(sm + (q * FOLD_ROWS + (tid >> 4) + it * (THREADS / 16)) * FOLD_PITCH + part * 64 + (tid & 15) * 4);
-#else
-					{
-						const typename Mma<f16_t>::acc_t &t = acc[pass * 2 + it][part];
-						m[it][q][part] = quad_t { t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3] };
-					}
-#endif
-			auto leave = [&](auto with_relu, auto with_z) __attribute__((always_inline))
-			{
-#pragma unroll
-				for (int it = 0; it < 2; it++)
-				{
-					float out[2][8];
-#pragma unroll
-					for (int c = 0; c < 8; c++)
-					{
-						const float m0 = m[it][0][c >> 2][c & 3], m1 = m[it][1][c >> 2][c & 3], m2 = m[it][2][c >> 2][c & 3], m3 = m[it][3][c >> 2][c & 3];
-						out[0][c] = m0 + m1 + m2;
-						out[1][c] = m1 - m2 - m3;
-					}
-#pragma unroll
-					for (int o = 0; o < 2; o++)
-					{
-						const unsigned int offset = y_off[pass][it][o];
-						epi.template store_fast<decltype(with_relu)::value, decltype(with_z)::value, 8>(out[o], columns, residual[pass][it][o], [&](auto words) __attribute__((always_inline))
-						{
-#ifndef ROWS_KNOCK_STORES
-							buffer_put<ROWS_STORE_POLICY>(ry, offset, words);
-#else
-							if (offset == 12345u)
-								buffer_put<STORE_STREAM_THROUGH>(ry, offset, words);
-#endif
-						});
-					}
-				}
-			};
-			if (relu && has_z)
-				leave(std::true_type(), std::true_type());
-			else if (relu)
-				leave(std::true_type(), std::false_type());
-			else if (has_z)
-				leave(std::false_type(), std::true_type());
-			else
-				leave(std::false_type(), std::false_type());
-			if (pass == 0)
-				STAMP(7);
-		}
 		}
 		STAMP(4);
 	}
