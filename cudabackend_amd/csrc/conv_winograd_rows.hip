@@ -534,47 +534,8 @@ namespace
 				else
 					fold_and_store(pass, std::false_type(), std::false_type());
 			};
-#pragma unroll
-			for (int rt = 0; rt < 4; rt++)
+			auto hand_over = [&](int rt) __attribute__((always_inline)) /* a finished row tile's sums into the fold buffer */
 			{
-				/* one scheduling region: the products of row tile rt, and among them the fold and the stores of row tile rt - 1,
-				 * whose sums the barrier behind the previous region has made visible */
-				__builtin_amdgcn_sched_barrier(0);
-				if (rt > 0)
-				{
-					fold_pass(rt - 1);
-					place(rt);
-				}
-#pragma unroll
-				for (int i = 0; i < FILTER_ROWS; i++)
-#pragma unroll
-					for (int sl = 0; sl < PHASE_SLABS; sl++)
-					{
-						const int c = (rt * FILTER_ROWS + i) * PHASE_SLABS + sl, cn = c + A_AHEAD;
-						if (cn < 4 * FILTER_ROWS * PHASE_SLABS)
-							read_a(LAST % RING, (cn / PHASE_SLABS) % FILTER_ROWS, cn % PHASE_SLABS, cn / (FILTER_ROWS * PHASE_SLABS), a[cn % A_RING]);
-#pragma unroll
-						for (int tn = 0; tn < 2; tn++)
-							Mma<f16_t>::run(bq[(LAST_SLAB + i * PHASE_SLABS + sl) % B_RING][tn], a[c % A_RING], acc[rt][tn]);
-					}
-				if (rt > 0)
-					__builtin_amdgcn_sched_group_barrier(0x100, 8, 0); /* the eight reads of the fold first */
-#pragma unroll
-				for (int k = 0; k < FILTER_ROWS * PHASE_SLABS; k++)
-				{
-					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-					__builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-					if (rt > 0)
-						__builtin_amdgcn_sched_group_barrier(0x002, 12, 0);
-				}
-				__builtin_amdgcn_sched_barrier(0);
-				if (rt == 0)
-					STAMP(6);
-				if (rt == 3)
-					STAMP(7);
-				/* row tile rt is final: out through LDS (everyone has folded the previous row tile: its values were consumed above) */
-				if (rt > 0)
-					__syncthreads();
 #pragma unroll
 				for (int tn = 0; tn < 2; tn++)
 #pragma unroll
@@ -584,8 +545,68 @@ namespace
 						const quad_t run = { t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3] };
 						*reinterpret_cast<quad_t*>(sm + (p * PASS_ROWS + (lane & 31)) * FOLD_PITCH + (lane >> 5) * 64 + (fh * 8 + tn * 4 + i) * 4) = run;
 					}
-				__syncthreads();
+			};
+			auto products = [&](int rt, int from, int to) __attribute__((always_inline)) /* chunk slots [from, to) of row tile rt */
+			{
+#pragma unroll
+				for (int k = from; k < to; k++)
+				{
+					const int i = k / PHASE_SLABS, sl = k % PHASE_SLABS;
+					const int c = rt * FILTER_ROWS * PHASE_SLABS + k, cn = c + A_AHEAD;
+					if (cn < 4 * FILTER_ROWS * PHASE_SLABS)
+						read_a(LAST % RING, (cn / PHASE_SLABS) % FILTER_ROWS, cn % PHASE_SLABS, cn / (FILTER_ROWS * PHASE_SLABS), a[cn % A_RING]);
+#pragma unroll
+					for (int tn = 0; tn < 2; tn++)
+						Mma<f16_t>::run(bq[(LAST_SLAB + i * PHASE_SLABS + sl) % B_RING][tn], a[c % A_RING], acc[rt][tn]);
+				}
+			};
+			constexpr int SLOTS = FILTER_ROWS * PHASE_SLABS, HEAD = 2; /* chunk slots of a row tile; those that carry the previous tile's hand-over */
+#pragma unroll
+			for (int rt = 0; rt < 4; rt++)
+			{
+				/* Row tile rt in two scheduling regions.  The first slots carry, between their MFMAs, the writes of row tile rt - 1
+				 * into the fold buffer; behind the barrier that makes them visible the remaining slots carry its fold and its stores. */
+				__builtin_amdgcn_sched_barrier(0);
+				if (rt > 0)
+					hand_over(rt - 1);
+				products(rt, 0, HEAD);
+#pragma unroll
+				for (int k = 0; k < HEAD; k++)
+				{
+					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+					__builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+					if (rt > 0)
+						__builtin_amdgcn_sched_group_barrier(0x200, 8 / HEAD, 0);
+				}
+				__builtin_amdgcn_sched_barrier(0);
+				if (rt > 0)
+				{
+					__syncthreads();
+					fold_pass(rt - 1);
+					place(rt);
+				}
+				products(rt, HEAD, SLOTS);
+				if (rt > 0)
+					__builtin_amdgcn_sched_group_barrier(0x100, 8, 0); /* the eight reads of the fold first */
+#pragma unroll
+				for (int k = HEAD; k < SLOTS; k++)
+				{
+					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+					__builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+					if (rt > 0)
+						__builtin_amdgcn_sched_group_barrier(0x002, 30, 0);
+				}
+				__builtin_amdgcn_sched_barrier(0);
+				if (rt == 0)
+					STAMP(6);
+				if (rt == 3)
+					STAMP(7);
+				/* everyone has folded row tile rt - 1 (its values were consumed above) before anyone overwrites the buffer */
+				if (rt > 0)
+					__syncthreads();
 			}
+			hand_over(3);
+			__syncthreads();
 			fold_pass(3);
 			STAMP(3);
 		}
