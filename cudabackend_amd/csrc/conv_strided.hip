@@ -241,6 +241,7 @@ namespace
 			for (int v = 0; v < 16; v++)
 				acc[rt][v] = 0.0f;
 		constexpr int A_RING = 6, A_AHEAD = 4;
+		constexpr int HEAD_TAPS = 4, TAIL_TAPS = S_TAPS - HEAD_TAPS; /* of the last phase: taps walked slab by slab / row tile by row tile */
 		constexpr int PHASE_CHUNKS = S_TAPS * S_SLABS * S_ROW_TILES; /* 126 A chunks per phase */
 		static_assert(PHASE_CHUNKS % A_RING == 0 && (S_TAPS * S_SLABS) % B_RING == 0, "both operand rings stand at 0 when a phase starts");
 		Chunk a[A_RING];
@@ -254,25 +255,28 @@ namespace
 		};
 		/* One phase: 9 taps x 2 slabs x 7 MFMAs per wavefront.  SLOT: which half of LDS holds it; B_BASE: where the filter ring stands
 		 * at its start. */
-		auto run_phase = [&](auto slot_tag, auto b_base_tag, int phase, int next) __attribute__((always_inline))
+		auto run_phase = [&](auto slot_tag, auto last_tag, int phase, int next) __attribute__((always_inline))
 		{
-			constexpr int SLOT = decltype(slot_tag)::value, B_BASE = decltype(b_base_tag)::value;
+			/* LAST: the first HEAD_TAPS taps of the last phase only (no next phase to fetch; the remaining taps below) */
+			constexpr int SLOT = decltype(slot_tag)::value, B_BASE = 0;
+			constexpr bool LAST = decltype(last_tag)::value;
+			constexpr int TAPS = LAST ? HEAD_TAPS : S_TAPS, CHUNKS = TAPS * S_SLABS * S_ROW_TILES;
 			constexpr int A_BASE = 0;
 #pragma unroll
 			for (int c = 0; c < A_AHEAD; c++)
 				read_a(SLOT, c, a[(A_BASE + c) % A_RING]); /* behind the barrier of the phase: nothing could be read ahead */
 #pragma unroll
-			for (int tap = 0; tap < S_TAPS; tap++)
+			for (int tap = 0; tap < TAPS; tap++)
 			{
 				__builtin_amdgcn_sched_barrier(0);
 				/* the next phase's planes: first half requested before this phase started, second half once the first is in LDS */
-				if (tap == 3)
+				if (!LAST && tap == 3)
 				{
 					stash_x(SLOT ^ 1, 0, raw);
 					__builtin_amdgcn_sched_barrier(0);
 					load_x(next, 1, raw);
 				}
-				if (tap == 7)
+				if (!LAST && tap == 7)
 					stash_x(SLOT ^ 1, 1, raw);
 #pragma unroll
 				for (int sl = 0; sl < S_SLABS; sl++)
@@ -283,7 +287,7 @@ namespace
 					for (int rt = 0; rt < S_ROW_TILES; rt++)
 					{
 						const int c = slab * S_ROW_TILES + rt;
-						if (c + A_AHEAD < PHASE_CHUNKS)
+						if (c + A_AHEAD < CHUNKS)
 							read_a(SLOT, c + A_AHEAD, a[(A_BASE + c + A_AHEAD) % A_RING]);
 						/* filters as the rows of the MFMA tile, pixels as its columns: a lane then holds runs of four consecutive filters
 						 * of one pixel, which the hand-over can move as 16-byte vectors */
@@ -299,7 +303,7 @@ namespace
 					{
 						__builtin_amdgcn_sched_group_barrier(0x100, 1, 0); /* the LDS read four chunks ahead, in front of its MFMA */
 						__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-						if ((tap == 3 || tap == 7) && sl == 0 && k % 2 == 1 && k / 2 < HALF)
+						if (!LAST && (tap == 3 || tap == 7) && sl == 0 && k % 2 == 1 && k / 2 < HALF)
 							__builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
 					}
 				}
@@ -308,98 +312,187 @@ namespace
 		};
 		/* trips of two phases (the channel count is a multiple of 64), one per half of LDS.  The planes of phase
 		 * p + 1 are stored during phase p, into the half of LDS that phase p - 1 left at the barrier. */
-		const int last = g.phases - 1;
-		for (int phase = 0; phase < g.phases; phase += 2)
+		int phase = 0;
+		for (; phase + 2 < g.phases; phase += 2)
 		{
-			run_phase(std::integral_constant<int, 0>(), std::integral_constant<int, 0>(), phase, phase + 1);
-			load_x(phase + 2 < last ? phase + 2 : last, 0, raw);
+			run_phase(std::integral_constant<int, 0>(), std::false_type(), phase, phase + 1);
+			load_x(phase + 2, 0, raw);
 			__syncthreads();
-			run_phase(std::integral_constant<int, 1>(), std::integral_constant<int, 0>(), phase + 1, phase + 2 < last ? phase + 2 : last);
-			if (phase + 2 < g.phases)
-			{
-				load_x(phase + 3, 0, raw);
-				__syncthreads();
-			}
+			run_phase(std::integral_constant<int, 1>(), std::false_type(), phase + 1, phase + 2);
+			load_x(phase + 3, 0, raw);
+			__syncthreads();
 		}
+		run_phase(std::integral_constant<int, 0>(), std::false_type(), phase, phase + 1);
+		__syncthreads();
 		SSTAMP(3);
-
-		/* hand-over and store: two passes of 128 GEMM rows; a work-item takes (row, 8 filters) eight times per pass */
-		float *sm = reinterpret_cast<float*>(lds);
+		/*
+		 * The last phase (in the second half of LDS; the first half is free from here on), and the results out while it runs.  Its
+		 * first taps go slab by slab like any other phase.  The filters of the remaining taps are all held in registers and the
+		 * products are taken two row tiles at a time, so that the sums of row tiles 0 and 1 are final when three more pairs are
+		 * still to be multiplied: bias, residual, activation and rounding are applied in the layout of the accumulators (a lane
+		 * holds runs of four consecutive filters of one pixel), the rounded runs pass through this wavefront's own piece of the
+		 * free half of LDS (no barrier: LDS serves a wavefront's operations in order) and leave as 16-byte stores, four lanes per
+		 * pixel, among the MFMAs of the next pair.  Only the last row tile's way out is left behind the loop.
+		 */
+		run_phase(std::integral_constant<int, 1>(), std::true_type(), phase + 1, phase + 1);
+		constexpr int TAIL_SLABS = TAIL_TAPS * S_SLABS, HEAD_SLABS = HEAD_TAPS * S_SLABS;
+		Chunk bl[TAIL_SLABS];
+#pragma unroll
+		for (int j = 0; j < TAIL_SLABS; j++)
+		{
+			if (j < B_AHEAD)
+				bl[j] = bq[(HEAD_SLABS + j) % B_RING]; /* requested by the ring during the first taps */
+			else
+				load_b((phase + 1) * S_TAPS * S_SLABS + HEAD_SLABS + j, bl[j]);
+		}
 		const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
 		__amdgpu_buffer_rsrc_t rz = make_buffer(nullptr, 0);
 		if (epi.z != nullptr)
 			rz = make_buffer(epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
 		const bool relu = epi.activation == ACT_RELU, has_z = epi.z != nullptr;
-		const int kcol = kb * S_FILTERS + (tid & 31) * 8; /* a work-item always stores the same 8 filters */
-		typename FloatEpilogue<TE>::template ColumnsT<8> columns;
-		epi.request_columns(kcol, columns);
-		constexpr int SWEEPS = S_FOLD_ROWS / (S_THREADS / 32); /* 8 */
-#pragma unroll
-		for (int pass = 0; pass < 2; pass++)
+		const int half = lane >> 5;
+		const int kwave = kb * S_FILTERS + wave * 32; /* this wavefront's first filter */
+		typedef float f32x4 __attribute__((ext_vector_type(4)));
+		f32x4 bias[4]; /* of this lane's four filters in each of its four runs */
 		{
-			unsigned int y_off[SWEEPS];
-			typename FloatEpilogue<TE>::template Residual<8> residual[SWEEPS];
+			const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(epi.bias), 0, epi.bias != nullptr ? g.K * 4 : 0, 0x00020000);
 #pragma unroll
-			for (int it = 0; it < SWEEPS; it++)
+			for (int i = 0; i < 4; i++)
+				bias[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rb, (kwave + 8 * i + 4 * half) * 4, 0, 0));
+		}
+		constexpr int OUT_PITCH = 32 * static_cast<int>(SZ) + 16, OUT_BYTES = 64 * OUT_PITCH; /* [two row tiles of pixels][32 filters as stored] */
+		static_assert((S_THREADS / 64) * OUT_BYTES <= S_PHASE_BYTES, "the wavefronts' pieces fit the free half of LDS");
+		int out_put = wave * OUT_BYTES + (lane & 31) * OUT_PITCH + 4 * half * static_cast<int>(SZ);
+		asm volatile("" : "+v"(out_put));
+		int out_get = wave * OUT_BYTES + (lane >> 2) * OUT_PITCH + (lane & 3) * 16;
+		asm volatile("" : "+v"(out_get));
+		/* byte offset in y of GEMM row q of the tile (filter 0), or out of range */
+		auto y_offset = [&](int q, int filter) __attribute__((always_inline))
+		{
+			const int r = static_cast<int>((static_cast<unsigned int>(q) * g.pw_magic) >> 20), c = q - r * g.PW;
+			const int oh = oh0 + r, ow = ow0 + c;
+			const bool ok = (r < g.TH) & (c < g.TW) & (oh < g.Ho) & (ow < g.Wo);
+			return ok ? static_cast<unsigned int>((oh * g.Wo + ow) * g.K + filter) * SZ : OUT_OF_RANGE;
+		};
+		/* rounds row tile rt in the layout of the accumulators and puts it into place `at` (0 / 1) of the wavefront's piece */
+		auto round_tile = [&](int rt, int at, auto with_relu, auto with_z) __attribute__((always_inline))
+		{
+			constexpr bool RELU = decltype(with_relu)::value, HAS_Z = decltype(with_z)::value;
+			unsigned int zw[2][4] = { { 0u, 0u, 0u, 0u }, { 0u, 0u, 0u, 0u } };
+			if (HAS_Z)
 			{
-				const int q = pass * S_FOLD_ROWS + (tid >> 5) + it * (S_THREADS / 32);
-				const int r = static_cast<int>((static_cast<unsigned int>(q) * g.pw_magic) >> 20), c = q - r * g.PW;
-				const int oh = oh0 + r, ow = ow0 + c;
-				const bool ok = (q < S_ROWS) & (r < g.TH) & (c < g.TW) & (oh < g.Ho) & (ow < g.Wo) & (kcol < g.K);
-				y_off[it] = ok ? static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ : OUT_OF_RANGE;
+				/* runs (2 pair, 2 pair + 1) of the two lanes of a pixel are 32 consecutive bytes of z: 16 per lane, exchanged by the swap */
+				const int q = rt * 32 + (lane & 31);
+#pragma unroll
+				for (int pair = 0; pair < 2; pair++)
+				{
+					const u32x4_t zr = __builtin_amdgcn_raw_buffer_load_b128(rz, static_cast<int>(y_offset(q, kwave + 8 * (2 * pair + half))), 0, 2);
+					const auto s0 = __builtin_amdgcn_permlane32_swap(zr[0], zr[2], false, false);
+					const auto s1 = __builtin_amdgcn_permlane32_swap(zr[1], zr[3], false, false);
+					zw[pair][0] = s0[0]; /* run 2 pair, this lane's half */
+					zw[pair][1] = s1[0];
+					zw[pair][2] = s0[1]; /* run 2 pair + 1 */
+					zw[pair][3] = s1[1];
+				}
+			}
+#pragma unroll
+			for (int i = 0; i < 4; i++)
+			{
 				union
 				{
-					uint4 u;
-					decltype(residual[0].raw) r8;
-				} cast;
-				cast.u = buffer_fetch<2>(rz, y_off[it]);
-				residual[it].raw = cast.r8;
-			}
-			__syncthreads(); /* pass 0: everyone is done with the planes; pass 1: with the rows of pass 0 */
-			/* A row of the buffer holds the 256 filters of a pixel as [first halves | second halves] of the 32 runs of 8 filters a
-			 * work-item stores: run g, half h at word h * 128 + g * 4 (sixteen lanes reading one half of sixteen runs touch 64
-			 * consecutive words).  This lane's accumulator registers 4i .. 4i + 3 of row tile rt are filters 32 * wave + 8i + 4 *
-			 * (lane / 32) + 0..3 of pixel (lane % 32): run 4 * wave + i, half (lane / 32). */
-			typedef float quad_t __attribute__((ext_vector_type(4)));
+					Pack<TE, 4> p;
+					unsigned int w[2];
+					uint2 u;
+				} zin, out;
+				zin.w[0] = zw[i >> 1][2 * (i & 1)];
+				zin.w[1] = zw[i >> 1][2 * (i & 1) + 1];
 #pragma unroll
-			for (int rt = 0; rt < 4; rt++)
-			{
-				if (pass * 4 + rt >= S_ROW_TILES)
-					continue;
-#pragma unroll
-				for (int i = 0; i < 4; i++)
+				for (int e = 0; e < 4; e++)
 				{
-					const typename Mma<TE>::acc_t &t = acc[pass * 4 + rt];
-					const quad_t run = { t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3] };
-					*reinterpret_cast<quad_t*>(sm + (rt * 32 + (lane & 31)) * S_FOLD_PITCH + (lane >> 5) * 128 + (wave * 4 + i) * 4) = run;
+					float r = epi.alpha1 * acc[rt][4 * i + e] + bias[i][e];
+					if (HAS_Z)
+						r += epi.alpha2 * Traits<TE>::load(zin.p.v[e]);
+					out.p.v[e] = Traits<TE>::store(RELU ? __builtin_fmaxf(r, 0.0f) : r);
 				}
+				*reinterpret_cast<uint2*>(lds + out_put + at * 32 * OUT_PITCH + 8 * i * static_cast<int>(SZ)) = out.u;
 			}
-			__syncthreads();
-			auto leave = [&](auto with_relu, auto with_z) __attribute__((always_inline))
-			{
+		};
+		/* the way out of `count` row tiles from row tile rt0 on: rounded, through the wavefront's piece of LDS, stored */
+		auto leave = [&](int rt0, int count) __attribute__((always_inline))
+		{
 #pragma unroll
-				for (int it = 0; it < SWEEPS; it++)
-				{
-					const int row = (tid >> 5) + it * (S_THREADS / 32);
-					const quad_t lo = *reinterpret_cast<const quad_t*>(sm + row * S_FOLD_PITCH + (tid & 31) * 4);
-					const quad_t hi = *reinterpret_cast<const quad_t*>(sm + row * S_FOLD_PITCH + 128 + (tid & 31) * 4);
-					const float v[8] = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
-					const unsigned int offset = y_off[it];
-					epi.template store_fast<decltype(with_relu)::value, decltype(with_z)::value, 8>(v, columns, residual[it], [&](auto words) __attribute__((always_inline))
-					{
-						buffer_put<17>(ry, offset, words); /* sc0 sc1: written through as the kernel runs */
-					});
-				}
-			};
-			if (relu && has_z)
-				leave(std::true_type(), std::true_type());
-			else if (relu)
-				leave(std::true_type(), std::false_type());
-			else if (has_z)
-				leave(std::false_type(), std::true_type());
-			else
-				leave(std::false_type(), std::false_type());
+			for (int t = 0; t < count; t++)
+			{
+				if (relu && has_z)
+					round_tile(rt0 + t, t, std::true_type(), std::true_type());
+				else if (relu)
+					round_tile(rt0 + t, t, std::true_type(), std::false_type());
+				else if (has_z)
+					round_tile(rt0 + t, t, std::false_type(), std::true_type());
+				else
+					round_tile(rt0 + t, t, std::false_type(), std::false_type());
+			}
+			/* lane l: 16 bytes (l % 4) of pixel l / 4 + 16 it */
+#pragma unroll
+			for (int it = 0; it < 2 * count; it++)
+			{
+				const uint4 run = *reinterpret_cast<const uint4*>(lds + out_get + it * 16 * OUT_PITCH);
+				const unsigned int offset = y_offset(rt0 * 32 + it * 16 + (lane >> 2), kwave + (lane & 3) * 8);
+				const u32x4_t words = { run.x, run.y, run.z, run.w };
+				__builtin_amdgcn_raw_buffer_store_b128(words, ry, static_cast<int>(offset), 0, 17); /* sc0 sc1: written through as the kernel runs */
+			}
+		};
+		/* chunk n of the tail = (pair of row tiles, tap, slab, row tile of the pair) in the order of use */
+		auto tail_chunk = [&](int n, int &rt, int &tap, int &sl) __attribute__((always_inline))
+		{
+			constexpr int PER_PAIR = TAIL_SLABS * 2;
+			const int pair = n / PER_PAIR < 3 ? n / PER_PAIR : 3; /* (the fourth "pair" is row tile 6 alone) */
+			const int m = n - pair * PER_PAIR, width = pair < 3 ? 2 : 1;
+			rt = pair * 2 + m % width;
+			sl = (m / width) % S_SLABS;
+			tap = HEAD_TAPS + m / (width * S_SLABS);
+		};
+		auto read_tail = [&](int n, Chunk &dst) __attribute__((always_inline))
+		{
+			int rt, tap, sl;
+			tail_chunk(n, rt, tap, sl);
+			const int i = tap / 3, j = tap % 3;
+			const int plane = (i & 1) * 2 + (j & 1);
+			dst.u = *reinterpret_cast<const uint4*>(lds + a_base[1][i >> 1][plane >> 1] + (plane & 1) * S_PLANE_BYTES + (j >> 1) * S_PITCH + rt * 32 * S_PITCH + sl * 32);
+		};
+		constexpr int TAIL_CHUNKS = TAIL_SLABS * S_ROW_TILES;
+#pragma unroll
+		for (int n = 0; n < A_AHEAD; n++)
+			read_tail(n, a[n % A_RING]);
+#pragma unroll
+		for (int pair = 0; pair < 4; pair++)
+		{
+			/* one scheduling region: the products of a pair of row tiles, and among them the way out of the pair before */
+			__builtin_amdgcn_sched_barrier(0);
+			const int width = pair < 3 ? 2 : 1, n0 = pair * TAIL_SLABS * 2;
+			if (pair > 0)
+				leave(2 * (pair - 1), 2);
+#pragma unroll
+			for (int m = 0; m < TAIL_SLABS * width; m++)
+			{
+				const int n = n0 + m;
+				if (n + A_AHEAD < TAIL_CHUNKS)
+					read_tail(n + A_AHEAD, a[(n + A_AHEAD) % A_RING]);
+				int rt, tap, sl;
+				tail_chunk(n, rt, tap, sl);
+				Mma<TE>::run(bl[(tap - HEAD_TAPS) * S_SLABS + sl], a[n % A_RING], acc[rt]);
+			}
+#pragma unroll
+			for (int m = 0; m < TAIL_SLABS * width; m++)
+			{
+				__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+				__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+				if (pair > 0)
+					__builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+			}
 		}
+		__builtin_amdgcn_sched_barrier(0);
+		leave(6, 1);
 		SSTAMP(4);
 	}
 
