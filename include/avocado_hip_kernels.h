@@ -94,8 +94,8 @@ extern "C"
 			void *y, double alpha1, double alpha2, double beta, int activation);
 
 	/* The same formula for 16-bit tensors by Winograd F(2,3) along image rows only, in one kernel (3x3, stride 1, dilation 1,
-	 * zero padding value, C = 64 or 128, K a multiple of 128, beta = 0, LINEAR or RELU; AVHIP_NOT_SUPPORTED otherwise, with
-	 * nothing launched).  The four planes of the transformed domain stay in accumulator registers for the whole k loop, so
+	 * zero padding value, C = 64, 128 or 256, K a multiple of 128, beta = 0, LINEAR or RELU, values inside the fp16 range;
+	 * AVHIP_NOT_SUPPORTED for other layers, with nothing launched).  The four planes of the transformed domain stay in accumulator registers for the whole k loop, so
 	 * the matrix cores do two thirds of the direct kernel's work and the output transform is paid once per output.  Stands
 	 * where the reference has its fused prototype, cuda_winogradFusedForward, src/winograd_fused.cu:789 (which transforms in
 	 * both directions).  U is what avhip_winograd_rows_weight_transform wrote: avhip_winograd_rows_weight_bytes(K, C) bytes
