@@ -1737,6 +1737,21 @@ namespace avocado
 			const avStatus_t st = prepare_conv(context, config, alpha1, xDesc, xMem, wDesc, wMem, bDesc, bMem, alpha2, zDesc, zMem, beta, yDesc, yMem, call);
 			if (st != AVOCADO_STATUS_SUCCESS)
 				return st;
+			/* the two implicit-GEMM kernels that want the weights in their own layout (stride 2; 1x1 with many filters): the same
+			 * arithmetic, taken where they pay and the library's cache can hold the layout (not while the stream is capturing
+			 * with a cold cache: nothing was launched then and the general kernels take over) */
+			if (strided_kernel_pays(call, activation))
+			{
+				const avStatus_t rs = run_strided_kernel(call, wMem, yMem, activation);
+				if (rs != AVOCADO_STATUS_NOT_SUPPORTED && rs != AVOCADO_STATUS_BAD_ALLOC)
+					return rs;
+			}
+			if (pointwise_block_pays(call, activation))
+			{
+				const avStatus_t rs = run_pointwise_block(call, wMem, yMem, activation);
+				if (rs != AVOCADO_STATUS_NOT_SUPPORTED && rs != AVOCADO_STATUS_BAD_ALLOC)
+					return rs;
+			}
 			return run_implicit_gemm(call, yMem, activation, nullptr);
 		}
 
@@ -1750,6 +1765,14 @@ namespace avocado
 			const avStatus_t st = prepare_conv(context, config, alpha1, xDesc, xMem, wDesc, wMem, bDesc, bMem, alpha2, zDesc, zMem, beta, yDesc, yMem, call);
 			if (st != AVOCADO_STATUS_SUCCESS)
 				return st;
+			/* 16-bit tensors: the one-kernel Winograd that transforms along rows only, where its shapes and the layer's size allow
+			 * (a 256 x 15 x 15 x 128 -> 128 layer in bf16: 16 us against 43 us in the kernel that transforms in both directions) */
+			if (rows_winograd_pays(call, activation))
+			{
+				const avStatus_t rs = run_rows_winograd(call, wMem, yMem, activation);
+				if (rs != AVOCADO_STATUS_NOT_SUPPORTED)
+					return rs; /* (BAD_ALLOC included: the entry reports a cold cache under capture as it always did) */
+			}
 			return run_fused_winograd(call, wMem, yMem, activation);
 		}
 

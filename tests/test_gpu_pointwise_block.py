@@ -105,6 +105,28 @@ def test_through_the_dispatcher(oracle, block_forced, dtype, case):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_through_the_implicit_gemm_entry(oracle, block_forced, dtype):
+    """cudaConvolutionImplicitGemmForward takes the same kernel: it is an implicit GEMM with the weights in another order."""
+    cs = CASES[1]
+    g = h.rng(470)
+    xs, ws = cs["x"], cs["w"]
+    pad, mode = cs.get("pad", (0, 0)), cs.get("mode", 0)
+    s = shape_of(xs, ws, pad=pad)
+    x = h.rounded(oracle, g.standard_normal(xs), dtype)
+    w = he(g, ws, dtype, oracle)
+    b = g.uniform(-0.1, 0.1, ws[0]).astype(np.float32).astype(np.float64)
+    ys = (xs[0], s.Ho, s.Wo, ws[0])
+    z = h.rounded(oracle, g.standard_normal(ys), dtype)
+    before = transforms(block_forced)
+    got = h.conv_forward("implicit_gemm", x, w, ys, dtype, bias=b, z=z, activation=cb.ACTIVATION_RELU, pad=(0, 0))
+    assert transforms(block_forced) == before + 1, "the general kernels never lay weights out"
+    want = oracle.conv2d(x, w, b, z=z, pad=(0, 0), activation=oracle.RELU)
+    err = oracle.rel_l2(got, want)
+    print("through the implicit-GEMM entry %s rel-L2 = %.3e" % (dtype, err))
+    assert err < BAR
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_kernel_layer_entry(oracle, dtype):
     """avhip_conv2d_pointwise_block_weight_layout + avhip_conv2d_pointwise_block called as a foreign host would: raw device pointers."""
     lib = cb.load_library()

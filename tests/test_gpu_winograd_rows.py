@@ -198,3 +198,33 @@ def test_large_magnitudes_within_the_fp16_range(oracle, rows_forced):
     w = he(g, ws, "bf16", oracle)
     got = h.conv_forward("dispatch", x, w, xs, "bf16", activation=0)
     assert oracle.rel_l2(got, oracle.conv2d(x, w)) < BAR
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_through_the_fused_winograd_entry(oracle, rows_forced, dtype):
+    """cudaConvolutionWinogradFusedForward on 16-bit tensors takes the row-wise kernel where it can: the transformed weights it
+    caches then have the row-wise layout's size (12 K C fp16 values), not the two-dimensional one's (16 K C)."""
+    lib = rows_forced
+    g = h.rng(480)
+    xs, ws = (3, 15, 15, 128), (128, 3, 3, 128)
+    x = h.rounded(oracle, g.standard_normal(xs), dtype)
+    w = h.rounded(oracle, g.standard_normal(ws) * np.sqrt(2.0 / (9 * ws[3])), dtype)
+    b = g.uniform(-0.1, 0.1, ws[0]).astype(np.float32).astype(np.float64)
+    ys = (xs[0], xs[1], xs[2], ws[0])
+    nbytes = C.c_int64(0)
+    with h.Call() as c:
+        conv = cb.ConvolutionDescriptor(padding=(-1, -1), dtype=h.DT[dtype])
+        xt, wt, bt = c.tensor(x, dtype), c.tensor(w, dtype), c.tensor(b, "f32")
+        y = c.empty(ys, dtype)
+        assert lib.avhipGetWeightCacheState(None, C.byref(nbytes), None) == cb.STATUS_SUCCESS
+        before = nbytes.value
+        cb.check(lib.cudaConvolutionWinogradFusedForward(c.ctx.handle, conv.handle, None, xt.desc, xt.mem, wt.desc, wt.mem, bt.desc, bt.mem, None, 0, 0,
+                                                          None, y.desc, y.mem, cb.ACTIVATION_RELU), "fused Winograd entry")
+        assert lib.avhipGetWeightCacheState(None, C.byref(nbytes), None) == cb.STATUS_SUCCESS
+        assert nbytes.value - before == 12 * ws[0] * ws[3] * 2, "the new cache entry has the row-wise layout's size"
+        c.finish()
+        got = y.download()
+    want = oracle.conv2d(x, w, b, activation=oracle.RELU)
+    err = oracle.rel_l2(got, want)
+    print("through the fused-Winograd entry %s rel-L2 = %.3e" % (dtype, err))
+    assert err < BAR
