@@ -256,3 +256,46 @@ def test_weight_cache_eviction_policy():
     # a budget of zero empties the cache of what is free to go
     assert probe([10, 10, 10, 10], [4, 3, 2, 1], [0, 1, 0, 2], 0, 0) == [1, 0, 1, 0]
     assert lib.avhipWeightCachePolicyProbe(1, None, None, None, 1, 1, None) == cb.STATUS_BAD_PARAM
+
+
+class _Shape(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("N", "H", "W", "C", "K", "R", "S", "Ho", "Wo", "pad_h", "pad_w", "stride_h", "stride_w", "dil_h", "dil_w",
+                                       "mode")]
+
+
+def _shape(x, w, pad, stride=1):
+    Ho, Wo = (x[1] - 2 * pad - w[1]) // stride + 1, (x[2] - 2 * pad - w[2]) // stride + 1  # pad is the (negative) offset of the first tap
+    return _Shape(x[0], x[1], x[2], x[3], w[0], w[1], w[2], Ho, Wo, pad, pad, stride, stride, 1, 1, 0)
+
+
+def test_plans_of_the_one_kernel_convolutions():
+    """What the dispatcher weighs for the three kernels that keep their pixel operand in LDS and take the filters from L2 — the
+    number of workgroups and how many of a workgroup's GEMM rows are real — is host arithmetic: checked here on the BASELINE shapes
+    and on what each kernel must decline."""
+    lib = cb.load_library()
+    bf16, f32 = cb.DTYPE_BFLOAT16, cb.DTYPE_FLOAT32
+    groups, rows = C.c_int(0), C.c_int(0)
+
+    def plan(fn, dtype, s):
+        rc = fn(dtype, C.byref(s), C.byref(groups), C.byref(rows))
+        return (groups.value, rows.value) if rc == 0 else rc
+
+    rw = lib.avhip_conv2d_winograd_rows_plan
+    assert plan(rw, bf16, _shape((256, 15, 15, 128), (128, 3, 3, 128), -1)) == (256, 120)  # config 2: one image per workgroup, 15 rows x 8 pairs
+    assert plan(rw, bf16, _shape((64, 56, 56, 256), (256, 3, 3, 256), -1)) == (1792, 112)  # config 3: 7 bands x 2 segments x 2 filter blocks
+    assert plan(rw, bf16, _shape((128, 20, 20, 128), (128, 3, 3, 128), -1))[1] >= 100      # config 4's shape in bf16
+    assert plan(rw, f32, _shape((256, 15, 15, 128), (128, 3, 3, 128), -1)) == -1
+    assert plan(rw, bf16, _shape((256, 15, 15, 128), (64, 3, 3, 128), -1)) == -1           # filters not a multiple of 128
+    assert plan(rw, bf16, _shape((256, 15, 15, 96), (128, 3, 3, 96), -1)) == -1            # channels other than 64, 128, 256
+    assert plan(rw, bf16, _shape((256, 15, 15, 128), (128, 3, 3, 128), -1, stride=2)) == -1
+
+    st = lib.avhip_conv2d_strided_plan
+    assert plan(st, bf16, _shape((64, 56, 56, 128), (256, 3, 3, 128), -1, stride=2)) == (256, 196)  # config 5: 7 x 28 output pixels per tile
+    assert plan(st, bf16, _shape((64, 56, 56, 128), (256, 3, 3, 128), -1)) == -1
+    assert plan(st, bf16, _shape((64, 56, 56, 128), (128, 3, 3, 128), -1, stride=2)) == -1          # filters not a multiple of 256
+
+    pb = lib.avhip_conv2d_pointwise_block_plan
+    assert plan(pb, bf16, _shape((64, 28, 28, 256), (512, 1, 1, 256), 0)) == (256, 196)    # config 5: 50176 pixels in 256 equal blocks
+    assert plan(pb, bf16, _shape((8, 28, 28, 256), (1024, 1, 1, 256), 0)) == (242, 52)     # two filter blocks share the chip: 121 pixel blocks of 52
+    assert plan(pb, bf16, _shape((64, 28, 28, 64), (512, 1, 1, 64), 0)) == -1
+    assert plan(pb, bf16, _shape((64, 28, 28, 256), (512, 3, 3, 256), -1)) == -1
