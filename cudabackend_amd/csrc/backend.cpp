@@ -942,7 +942,8 @@ namespace
 
 	/* Row-wise Winograd F(2,3) for 16-bit 3x3 layers whose image bands fit a compute unit's LDS (conv_winograd_rows.hip): two
 	 * thirds of the direct kernel's MFMA work.  Worth it when its workgroups (one per compute unit, 128 filters each) cover
-	 * most of the chip and most of their 128 GEMM rows are image. */
+	 * more than half of the chip and most of their 128 GEMM rows are image (15 x 15 images, 128 -> 128, bf16: 14.3 us against
+	 * 13.2 us in the image-tile kernel at 128 images, 14.8 against 17.3 us at 160). */
 	bool rows_winograd_pays(const ConvCall &c, avActivationType_t activation)
 	{
 		const ConvProblem &p = c.problem;
@@ -953,7 +954,7 @@ namespace
 		int workgroups = 0, rows_used = 0;
 		if (avhip_conv2d_winograd_rows_plan(p.x_dtype, &p.shape, &workgroups, &rows_used) != 0)
 			return false;
-		return avhip_set_winograd_rows(-1) == 2 || (workgroups >= 192 && rows_used >= 96);
+		return avhip_set_winograd_rows(-1) == 2 || (workgroups >= 144 && rows_used >= 96);
 	}
 	avStatus_t run_rows_winograd(const ConvCall &c, avMemoryDescriptor_t wMem, avMemoryDescriptor_t yMem, avActivationType_t activation)
 	{
@@ -972,7 +973,8 @@ namespace
 	}
 
 	/* 3x3 stride-2 layers of 16-bit tensors through the parity-plane kernel (conv_strided.hip), weights in its operand layout from
-	 * the cache.  Worth it when its workgroups (one per compute unit, 256 filters each) cover most of the chip. */
+	 * the cache.  Worth it from 96 workgroups (one per compute unit, 256 filters each) on: 56 x 56 x 128 -> 256 in bf16 takes 23.5
+	 * us against 28.2 us in the gather kernel at 24 images (96 workgroups), 22.7 against 22.7 at 16. */
 	bool strided_kernel_pays(const ConvCall &c, avActivationType_t activation)
 	{
 		const ConvProblem &p = c.problem;
@@ -983,7 +985,7 @@ namespace
 		int workgroups = 0, rows_used = 0;
 		if (avhip_conv2d_strided_plan(p.x_dtype, &p.shape, &workgroups, &rows_used) != 0)
 			return false;
-		return avhip_set_conv_strided(-1) == 2 || (workgroups >= 192 && rows_used >= 144);
+		return avhip_set_conv_strided(-1) == 2 || (workgroups >= 96 && rows_used >= 144);
 	}
 	avStatus_t run_strided_kernel(const ConvCall &c, avMemoryDescriptor_t wMem, avMemoryDescriptor_t yMem, avActivationType_t activation)
 	{
@@ -1002,7 +1004,8 @@ namespace
 
 	/* 1x1 layers of 16-bit tensors with 128 or 256 channels and a multiple of 512 filters through the pixel-block kernel
 	 * (conv_pointwise_block.hip), weights in its operand layout from the cache (kind 5).  Worth it when its workgroups (one per
-	 * compute unit) cover most of the chip and most of their 224 GEMM rows are pixels. */
+	 * compute unit) cover most of the chip with at least 96 pixels each: 28 x 28 x 256 -> 512 in bf16 takes 17.0 us against 18.0
+	 * us in the short-k engine at 32 images (251 blocks of 100 pixels), 15.3 against 15.0 at 24. */
 	bool pointwise_block_pays(const ConvCall &c, avActivationType_t activation)
 	{
 		const ConvProblem &p = c.problem;
@@ -1013,7 +1016,7 @@ namespace
 		int workgroups = 0, rows_used = 0;
 		if (avhip_conv2d_pointwise_block_plan(p.x_dtype, &p.shape, &workgroups, &rows_used) != 0)
 			return false;
-		return avhip_set_pointwise_block(-1) == 2 || (workgroups >= 192 && rows_used >= 160);
+		return avhip_set_pointwise_block(-1) == 2 || (workgroups >= 192 && rows_used >= 96);
 	}
 	avStatus_t run_pointwise_block(const ConvCall &c, avMemoryDescriptor_t wMem, avMemoryDescriptor_t yMem, avActivationType_t activation)
 	{
