@@ -173,7 +173,10 @@ namespace
 			U[((((static_cast<int64_t>(phase) * FILTER_ROWS + i) * POSITIONS + p) * filter_tiles + tile) * PHASE_SLABS + slab) * 64 + lane] = out[p].u;
 	}
 
-	template<typename TE, int PHASES>
+	/* RELU, HAS_Z: the activation (ReLU or none) and whether a residual is added, fixed per instance: a branch on either inside the
+	 * last phase would cut the scheduling regions in which a row tile's fold sits between the next one's MFMAs, and one copy of the
+	 * last phase per combination behind a branch in front of it costs the register allocator its last registers. */
+	template<typename TE, int PHASES, bool RELU, bool HAS_Z>
 	__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_winograd_rows(const TE *__restrict__ x, const void *__restrict__ U,
 			RowsGeom g, FloatEpilogue<TE> epi)
 	{
@@ -322,7 +325,7 @@ namespace
 				}
 		}
 
-		const int kcol = kb * ROWS_BLOCK_N + (tid & 15) * 8; /* a work-item always stores the same 8 filters */
+		const int kcol = kb * ROWS_BLOCK_N + (tid & 15) * 4; /* a work-item always stores the same 4 filters of each half of the block */
 
 		/* MFMA operand address: lane l supplies GEMM row (l % 32) of a 32-row tile and the 8-channel half (l / 32) of a slab.  Rows
 		 * past the tile's last read whatever follows in LDS (at most 127 + 2 * pairs pixels into a plane of 137: the next plane, or
@@ -443,18 +446,23 @@ namespace
 #pragma unroll
 		for (int c = 0; c < A_AHEAD; c++)
 			read_a(0, 0, c / 4, c % 4, a[c]);
-		/* the fold buffer: [plane][row][128 filters + 4] floats, a row holding the filters as [first halves | second halves] of the 16
-		 * runs of 8 filters a work-item stores: run g, half h at word h * 64 + g * 4, so that sixteen lanes reading the same half of
-		 * sixteen runs touch 64 consecutive words (every bank once).  A lane's accumulator registers 4i..4i+3 of tile (rt, tn) are
-		 * filters fh * 64 + tn * 32 + 8i + 4 * (lane / 32) + 0..3 of GEMM row 32 rt + lane % 32: run fh * 8 + tn * 4 + i, half lane / 32. */
+		/* the fold buffer: [plane][row][128 filters + 4] floats, the filters of a row in their order.  A lane's accumulator registers
+		 * 4i..4i+3 of tile (rt, tn) are filters fh * 64 + tn * 32 + 8i + 4 * (lane / 32) + 0..3 of GEMM row 32 rt + lane % 32; the
+		 * pitch of 132 words puts sixteen consecutive rows of one such run on all 64 banks once. */
 		typedef float quad_t __attribute__((ext_vector_type(4)));
 		const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
-		__amdgpu_buffer_rsrc_t rz = make_buffer(nullptr, 0);
-		if (epi.z != nullptr)
-			rz = make_buffer(epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
-		const bool relu = epi.activation == ACT_RELU, has_z = epi.z != nullptr;
+		const __amdgpu_buffer_rsrc_t rz = make_buffer(HAS_Z ? epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K : nullptr, HAS_Z ? static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ : 0u);
+		constexpr std::integral_constant<bool, RELU> with_relu;
+		constexpr std::integral_constant<bool, HAS_Z> with_z;
 		{
 			run_phases();
+			/* The sums so far are pinned here: an MFMA has no side effect, so without a use in this block the chains of the row
+			 * tiles that the last phase takes up later may be moved down to it, their pixel operands kept alive from every phase. */
+#pragma unroll
+			for (int rt = 0; rt < 4; rt++)
+#pragma unroll
+				for (int tn = 0; tn < 2; tn++)
+					asm volatile("" : "+v"(acc[rt][tn]));
 			/*
 			 * The last phase, and the results out while it runs.  Its filters (six slabs, the whole ring) stay in registers and its
 			 * products are taken row tile by row tile, so that the sums of row tile 0 are final after a quarter of the phase: they go
@@ -467,73 +475,80 @@ namespace
 			float *sm = reinterpret_cast<float*>(lds + ((LAST % RING) >> 1 == 0 ? SLICE_BYTES : 0));
 			STAMP(5);
 			load_b(LAST_SLAB + B_AHEAD, bq[(LAST_SLAB + B_AHEAD) % B_RING]);
-			typename FloatEpilogue<TE>::template ColumnsT<8> columns;
-			epi.request_columns(kcol, columns);
-			/* this work-item's (row, pair) of a pass: where its two output pixels go, and their residual */
+			/* A work-item folds and stores, for one (row, pair) of a pass, 4 filters of each half of the workgroup's 128: sixteen
+			 * lanes then read 64 consecutive words of a fold-buffer row (every bank once) and write one whole 128-byte line of
+			 * y, and the fold holds 4 x 4 sums at a time. */
+			typename FloatEpilogue<TE>::template ColumnsT<4> columns[2];
+#pragma unroll
+			for (int h = 0; h < 2; h++)
+				epi.request_columns(kcol + h * 64, columns[h]);
 			unsigned int y_off[2][2];
-			typename FloatEpilogue<TE>::template Residual<8> residual[2][2];
-			auto place = [&](int pass) __attribute__((always_inline))
+			typedef unsigned int pair_t __attribute__((ext_vector_type(2)));
+			pair_t residual[2][2][2]; /* [pass parity][output pixel][half] */
+			auto place = [&](int pass, auto with_z) __attribute__((always_inline))
 			{
 				const int q = pass * PASS_ROWS + (tid >> 4);
 				const int r = static_cast<int>((static_cast<unsigned int>(q) * g.pairs_magic) >> 20);
 				const int pair = q - r * g.pairs;
 				const int oh = oh0 + r;
-				const bool row_ok = (q < band_rows) & (oh < g.Ho) & (kcol < g.K);
+				const bool row_ok = (q < band_rows) & (oh < g.Ho);
 #pragma unroll
 				for (int o = 0; o < 2; o++)
 				{
 					const int ow = ow0 + 2 * pair + o;
-					y_off[pass & 1][o] = (row_ok & (ow < g.Wo)) ? static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ : OUT_OF_RANGE;
-					union
+					/* the offset computed whether or not the pixel exists, and opaque: a select of a product invites a branch around
+					 * the product, and a branch here ends the scheduling region of the row tile */
+					unsigned int at = static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ;
+					asm volatile("" : "+v"(at));
+					y_off[pass & 1][o] = (row_ok & (ow < g.Wo)) ? at : OUT_OF_RANGE;
+					if constexpr (decltype(with_z)::value)
 					{
-						uint4 u;
-						decltype(residual[0][0].raw) r8;
-					} cast;
-					cast.u = buffer_fetch<2>(rz, y_off[pass & 1][o]);
-					residual[pass & 1][o].raw = cast.r8;
+#pragma unroll
+						for (int h = 0; h < 2; h++)
+							residual[pass & 1][o][h] = __builtin_bit_cast(pair_t, __builtin_amdgcn_raw_buffer_load_b64(rz, static_cast<int>(y_off[pass & 1][o]), h * 64 * SZ, 0));
+					}
 				}
 			};
 			auto fold_and_store = [&](int pass, auto with_relu, auto with_z) __attribute__((always_inline))
 			{
-				quad_t m[POSITIONS][2];
 #pragma unroll
-				for (int q = 0; q < POSITIONS; q++)
-#pragma unroll
-					for (int part = 0; part < 2; part++)
-						m[q][part] = *reinterpret_cast<const quad_t*>(sm + (q * PASS_ROWS + (tid >> 4)) * FOLD_PITCH + part * 64 + (tid & 15) * 4);
-				float out[2][8];
-#pragma unroll
-				for (int c = 0; c < 8; c++)
+				for (int h = 0; h < 2; h++)
 				{
-					const float m0 = m[0][c >> 2][c & 3], m1 = m[1][c >> 2][c & 3], m2 = m[2][c >> 2][c & 3], m3 = m[3][c >> 2][c & 3];
-					out[0][c] = m0 + m1 + m2;
-					out[1][c] = m1 - m2 - m3;
-				}
+					quad_t m[POSITIONS];
 #pragma unroll
-				for (int o = 0; o < 2; o++)
-				{
-					const unsigned int offset = y_off[pass & 1][o];
-					epi.template store_fast<decltype(with_relu)::value, decltype(with_z)::value, 8>(out[o], columns, residual[pass & 1][o], [&](auto words) __attribute__((always_inline))
+					for (int q = 0; q < POSITIONS; q++)
+						m[q] = *reinterpret_cast<const quad_t*>(sm + (q * PASS_ROWS + (tid >> 4)) * FOLD_PITCH + h * 64 + (tid & 15) * 4);
+					float out[2][4];
+#pragma unroll
+					for (int c = 0; c < 4; c++)
 					{
-						buffer_put<ROWS_STORE_POLICY>(ry, offset, words);
-					});
+						out[0][c] = m[0][c] + m[1][c] + m[2][c];
+						out[1][c] = m[1][c] - m[2][c] - m[3][c];
+					}
+#pragma unroll
+					for (int o = 0; o < 2; o++)
+					{
+						float t[4], zv[4];
+						union
+						{
+							Pack<TE, 4> e;
+							pair_t words;
+						} cast;
+						cast.words = residual[pass & 1][o][h];
+#pragma unroll
+						for (int c = 0; c < 4; c++)
+							zv[c] = decltype(with_z)::value ? Traits<TE>::load(cast.e.v[c]) : 0.0f;
+						epi.template combine<decltype(with_relu)::value, decltype(with_z)::value, 4>(t, out[o], columns[h], zv);
+#pragma unroll
+						for (int c = 0; c < 4; c++)
+							cast.e.v[c] = Traits<TE>::store(t[c]);
+						buffer_put<ROWS_STORE_POLICY>(ry, y_off[pass & 1][o] + h * 64 * SZ, cast.words);
+					}
 				}
 			};
-			place(0);
 #pragma unroll
 			for (int c = 0; c < A_AHEAD; c++)
 				read_a(LAST % RING, (c / PHASE_SLABS) % FILTER_ROWS, c % PHASE_SLABS, c / (FILTER_ROWS * PHASE_SLABS), a[c % A_RING]); /* chunk = (row tile, filter row, slab) */
-			auto fold_pass = [&](int pass) __attribute__((always_inline))
-			{
-				if (relu && has_z)
-					fold_and_store(pass, std::true_type(), std::true_type());
-				else if (relu)
-					fold_and_store(pass, std::true_type(), std::false_type());
-				else if (has_z)
-					fold_and_store(pass, std::false_type(), std::true_type());
-				else
-					fold_and_store(pass, std::false_type(), std::false_type());
-			};
 			auto hand_over = [&](int rt) __attribute__((always_inline)) /* a finished row tile's sums into the fold buffer */
 			{
 #pragma unroll
@@ -543,7 +558,7 @@ namespace
 					{
 						const typename Mma<f16_t>::acc_t &t = acc[rt][tn];
 						const quad_t run = { t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3] };
-						*reinterpret_cast<quad_t*>(sm + (p * PASS_ROWS + (lane & 31)) * FOLD_PITCH + (lane >> 5) * 64 + (fh * 8 + tn * 4 + i) * 4) = run;
+						*reinterpret_cast<quad_t*>(sm + (p * PASS_ROWS + (lane & 31)) * FOLD_PITCH + fh * 64 + tn * 32 + i * 8 + (lane >> 5) * 4) = run;
 					}
 			};
 			auto products = [&](int rt, int from, int to) __attribute__((always_inline)) /* chunk slots [from, to) of row tile rt */
@@ -561,6 +576,7 @@ namespace
 				}
 			};
 			constexpr int SLOTS = FILTER_ROWS * PHASE_SLABS, HEAD = 2; /* chunk slots of a row tile; those that carry the previous tile's hand-over */
+			place(0, with_z);
 #pragma unroll
 			for (int rt = 0; rt < 4; rt++)
 			{
@@ -582,8 +598,8 @@ namespace
 				if (rt > 0)
 				{
 					__syncthreads();
-					fold_pass(rt - 1);
-					place(rt);
+					fold_and_store(rt - 1, with_relu, with_z);
+					place(rt, with_z);
 				}
 				products(rt, HEAD, SLOTS);
 				if (rt > 0)
@@ -607,7 +623,7 @@ namespace
 			}
 			hand_over(3);
 			__syncthreads();
-			fold_pass(3);
+			fold_and_store(3, with_relu, with_z);
 			STAMP(3);
 		}
 		STAMP(4);
@@ -688,12 +704,25 @@ namespace
 		const FloatEpilogue<TE> epi { static_cast<const float*>(bias), static_cast<const TE*>(z), static_cast<TE*>(y), static_cast<float>(alpha1),
 				static_cast<float>(alpha2), 0.0f, activation, s.K, true };
 		const dim3 grid(static_cast<unsigned int>(items), static_cast<unsigned int>(s.K / ROWS_BLOCK_N));
-		if (s.C == 256)
-			hipLaunchKernelGGL((k_winograd_rows<TE, 8>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
-		else if (s.C == 128)
-			hipLaunchKernelGGL((k_winograd_rows<TE, 4>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+		auto launch = [&](auto relu, auto residual)
+		{
+			constexpr bool R = decltype(relu)::value, Z = decltype(residual)::value;
+			if (s.C == 256)
+				hipLaunchKernelGGL((k_winograd_rows<TE, 8, R, Z>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+			else if (s.C == 128)
+				hipLaunchKernelGGL((k_winograd_rows<TE, 4, R, Z>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+			else
+				hipLaunchKernelGGL((k_winograd_rows<TE, 2, R, Z>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+		};
+		const bool relu = activation == ACT_RELU, residual = z != nullptr;
+		if (relu && residual)
+			launch(std::true_type(), std::true_type());
+		else if (relu)
+			launch(std::true_type(), std::false_type());
+		else if (residual)
+			launch(std::false_type(), std::true_type());
 		else
-			hipLaunchKernelGGL((k_winograd_rows<TE, 2>), grid, dim3(THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+			launch(std::false_type(), std::false_type());
 		return 0;
 	}
 }

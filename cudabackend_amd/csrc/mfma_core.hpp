@@ -169,10 +169,11 @@ namespace avhip
 		const u32x4_t v = { words.x, words.y, words.z, words.w };
 		__builtin_amdgcn_raw_buffer_store_b128(v, rsrc, static_cast<int>(byte_offset), 0, POLICY);
 	}
+	template<int POLICY = STORE_STREAM>
 	__device__ inline void buffer_put(__amdgpu_buffer_rsrc_t rsrc, unsigned int byte_offset, unsigned int __attribute__((ext_vector_type(2))) words)
 	{
 		const u32x2_t v = { words.x, words.y };
-		__builtin_amdgcn_raw_buffer_store_b64(v, rsrc, static_cast<int>(byte_offset), 0, 2);
+		__builtin_amdgcn_raw_buffer_store_b64(v, rsrc, static_cast<int>(byte_offset), 0, POLICY);
 	}
 	template<typename TE>
 	__device__ inline uint4 splat_chunk(TE value, int valid)
