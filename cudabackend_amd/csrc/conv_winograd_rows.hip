@@ -56,6 +56,9 @@ extern "C" __attribute__((visibility("default"))) int avhip_debug_rows_stamps(vo
 #define STAMP(i) do { } while (0)
 #endif
 
+#ifndef ROWS_UNIT_VALU
+#define ROWS_UNIT_VALU 10 /* vector-ALU instructions of the fold behind every MFMA of the last phase */
+#endif
 #ifndef ROWS_STORE_POLICY
 #define ROWS_STORE_POLICY 17 /* sc0 sc1: written through as the kernel runs, no streaming hint */
 #endif
@@ -79,8 +82,6 @@ namespace
 	constexpr int ROWS_BLOCK_N = 128; /* filters per workgroup */
 	constexpr int THREADS = 512;
 	constexpr int OPERAND_BYTES = 1024; /* one MFMA operand of a wavefront: 64 lanes x 16 bytes */
-	/* epilogue: [plane][32 rows][128 filters + 4] floats per row tile, in the slice of LDS that the last phase does not read */
-	constexpr int FOLD_PITCH = ROWS_BLOCK_N + 4;
 	static_assert(V_BYTES <= 160 * 1024, "LDS of a compute unit");
 
 	struct RowsGeom
@@ -198,7 +199,7 @@ namespace
 		const int lane = tid & 63;
 		const int wave = tid >> 6;
 		const int p = wave & 3; /* plane of this wavefront */
-		const int fh = wave >> 2; /* its half of the 128 filters */
+		const int fh = wave >> 2; /* its 32 filters of either 64-filter half of the block */
 
 		/* (image, band, segment) and filter block.  Where workgroups share input (several tiles per image: neighbouring bands
 		 * read two rows in common; several filter blocks: each reads the whole tile) they are renumbered so that the filter
@@ -225,10 +226,10 @@ namespace
 		bottom = bottom > v_rows - top ? v_rows - top : bottom;
 		const int real_rows = v_rows - top - bottom;
 
-		/* B operand: this wavefront's two filter tiles of step (phase, filter row) are 4 contiguous kilobytes */
+		/* B operand: this wavefront's two filter tiles are tiles fh and 2 + fh of the block's four (its 32 filters of either 64-filter half) */
 		const unsigned int step_stride = static_cast<unsigned int>(POSITIONS * g.filter_tiles * PHASE_SLABS * OPERAND_BYTES);
 		const __amdgpu_buffer_rsrc_t ru = make_buffer(U, static_cast<unsigned int>(STEPS) * step_stride);
-		const unsigned int b_offset = static_cast<unsigned int>((p * g.filter_tiles + kb * 4 + fh * 2) * PHASE_SLABS * OPERAND_BYTES + lane * 16);
+		const unsigned int b_offset = static_cast<unsigned int>((p * g.filter_tiles + kb * 4 + fh) * PHASE_SLABS * OPERAND_BYTES + lane * 16);
 		/* Filters go through a ring of register sets, one set = the two filter tiles of one 16-channel slab (two slabs per step),
 		 * requested B_AHEAD slabs before they are multiplied: six sets, one phase's worth, which is what the last phase keeps in
 		 * registers (rings of four and eight measured the same: the way ahead is not what the requests cost). */
@@ -244,7 +245,7 @@ namespace
 #pragma unroll
 			for (int tn = 0; tn < 2; tn++)
 			{
-				const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(ru, static_cast<int>(b_offset + tn * PHASE_SLABS * OPERAND_BYTES),
+				const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(ru, static_cast<int>(b_offset + tn * 2 * PHASE_SLABS * OPERAND_BYTES),
 						static_cast<int>(step * step_stride + sl * OPERAND_BYTES), 0);
 				set[tn].u = make_uint4(v[0], v[1], v[2], v[3]);
 			}
@@ -325,7 +326,7 @@ namespace
 				}
 		}
 
-		const int kcol = kb * ROWS_BLOCK_N + (tid & 15) * 4; /* a work-item always stores the same 4 filters of each half of the block */
+				const int kcol = kb * ROWS_BLOCK_N + (tid & 15) * 4; /* a work-item always stores the same 4 filters of each half of the block */
 
 		/* MFMA operand address: lane l supplies GEMM row (l % 32) of a 32-row tile and the 8-channel half (l / 32) of a slab.  Rows
 		 * past the tile's last read whatever follows in LDS (at most 127 + 2 * pairs pixels into a plane of 137: the next plane, or
@@ -446,9 +447,8 @@ namespace
 #pragma unroll
 		for (int c = 0; c < A_AHEAD; c++)
 			read_a(0, 0, c / 4, c % 4, a[c]);
-		/* the fold buffer: [plane][row][128 filters + 4] floats, the filters of a row in their order.  A lane's accumulator registers
-		 * 4i..4i+3 of tile (rt, tn) are filters fh * 64 + tn * 32 + 8i + 4 * (lane / 32) + 0..3 of GEMM row 32 rt + lane % 32; the
-		 * pitch of 132 words puts sixteen consecutive rows of one such run on all 64 banks once. */
+		/* A lane's accumulator registers 4i..4i+3 of tile (rt, tn) are filters tn * 64 + fh * 32 + 8i + 4 * (lane / 32) + 0..3 of GEMM row
+		 * 32 rt + lane % 32. */
 		typedef float quad_t __attribute__((ext_vector_type(4)));
 		const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
 		const __amdgpu_buffer_rsrc_t rz = make_buffer(HAS_Z ? epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K : nullptr, HAS_Z ? static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ : 0u);
@@ -465,29 +465,39 @@ namespace
 					asm volatile("" : "+v"(acc[rt][tn]));
 			/*
 			 * The last phase, and the results out while it runs.  Its filters (six slabs, the whole ring) stay in registers and its
-			 * products are taken row tile by row tile, so that the sums of row tile 0 are final after a quarter of the phase: they go
-			 * through LDS (32 rows of four planes: the half of LDS that the last phase does not read), are folded and stored while
-			 * the matrix cores work on row tile 1, and so on.  The stores of three quarters of the tile are then under way before
-			 * the loop has ended, and what is left behind it is one quarter's hand-over instead of two passes over the whole tile.
+			 * products are taken unit by unit, a unit being one MFMA tile of sums: 32 GEMM rows (a row tile) by this wavefront's 32
+			 * filters of one 64-filter half of the block.  A unit is final after an eighth of the phase; in the region after it goes
+			 * into one of two fold buffers in the slice of LDS that the last phase does not read ([plane][32 rows][64 filters + 4]
+			 * floats each), in the region after that its four sums per output are read back by the work-items that will fold them,
+			 * and in the region after that it is folded and stored: a region holds the MFMAs of unit u, the four writes of unit
+			 * u - 1, the four reads of unit u - 2 and the fold of unit u - 3, none of which waits for another or for a latency
+			 * of LDS, and one barrier ends it: the writes are visible to the next region's reads, and the buffer that this
+			 * region has read is free for the next region's writes.
 			 */
-			constexpr int LAST = PHASES - 1, LAST_SLAB = LAST * FILTER_ROWS * PHASE_SLABS, PASS_ROWS = 32;
-			static_assert(B_RING == FILTER_ROWS * PHASE_SLABS && POSITIONS * PASS_ROWS * FOLD_PITCH * 4 <= SLICE_BYTES, "one phase of filters in the ring; the fold buffer in one slice");
+			constexpr int LAST = PHASES - 1, LAST_SLAB = LAST * FILTER_ROWS * PHASE_SLABS;
+			constexpr int UNIT_ROWS = 32, UNIT_FILTERS = ROWS_BLOCK_N / 2, UNIT_PITCH = UNIT_FILTERS + 4, UNIT_WORDS = POSITIONS * UNIT_ROWS * UNIT_PITCH;
+			constexpr int ROW_TILE_CHUNKS = FILTER_ROWS * PHASE_SLABS, UNITS = 8;
+			static_assert(B_RING == ROW_TILE_CHUNKS && A_RING == ROW_TILE_CHUNKS && 2 * UNIT_WORDS * 4 <= SLICE_BYTES,
+					"one phase of filters and one row tile of pixels in the rings; both fold buffers in one slice");
 			float *sm = reinterpret_cast<float*>(lds + ((LAST % RING) >> 1 == 0 ? SLICE_BYTES : 0));
 			STAMP(5);
 			load_b(LAST_SLAB + B_AHEAD, bq[(LAST_SLAB + B_AHEAD) % B_RING]);
-			/* A work-item folds and stores, for one (row, pair) of a pass, 4 filters of each half of the workgroup's 128: sixteen
-			 * lanes then read 64 consecutive words of a fold-buffer row (every bank once) and write one whole 128-byte line of
-			 * y, and the fold holds 4 x 4 sums at a time. */
+			/* the six pixel operands of row tile 0; those of row tile rt + 1 take their places as the second unit of rt lets go of them */
+#pragma unroll
+			for (int c = 0; c < ROW_TILE_CHUNKS; c++)
+				read_a(LAST % RING, c / PHASE_SLABS, c % PHASE_SLABS, 0, a[c]);
+			/* A work-item folds and stores, for one (row, pair) of a row tile, 4 filters of each half of the block: sixteen lanes
+			 * read 64 consecutive words of a fold-buffer row (every bank once) and write one whole 128-byte line of y. */
 			typename FloatEpilogue<TE>::template ColumnsT<4> columns[2];
 #pragma unroll
-			for (int h = 0; h < 2; h++)
-				epi.request_columns(kcol + h * 64, columns[h]);
+			for (int tn = 0; tn < 2; tn++)
+				epi.request_columns(kcol + tn * UNIT_FILTERS, columns[tn]);
 			unsigned int y_off[2][2];
 			typedef unsigned int pair_t __attribute__((ext_vector_type(2)));
-			pair_t residual[2][2][2]; /* [pass parity][output pixel][half] */
-			auto place = [&](int pass, auto with_z) __attribute__((always_inline))
+			pair_t residual[2][2][2]; /* [row tile parity][output pixel][half] */
+			auto place = [&](int rt) __attribute__((always_inline)) /* where the two output pixels of this work-item's (row, pair) of row tile rt go */
 			{
-				const int q = pass * PASS_ROWS + (tid >> 4);
+				const int q = rt * UNIT_ROWS + (tid >> 4);
 				const int r = static_cast<int>((static_cast<unsigned int>(q) * g.pairs_magic) >> 20);
 				const int pair = q - r * g.pairs;
 				const int oh = oh0 + r;
@@ -497,133 +507,124 @@ namespace
 				{
 					const int ow = ow0 + 2 * pair + o;
 					/* the offset computed whether or not the pixel exists, and opaque: a select of a product invites a branch around
-					 * the product, and a branch here ends the scheduling region of the row tile */
+					 * the product, and a branch here ends the scheduling region */
 					unsigned int at = static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ;
 					asm volatile("" : "+v"(at));
-					y_off[pass & 1][o] = (row_ok & (ow < g.Wo)) ? at : OUT_OF_RANGE;
-					if constexpr (decltype(with_z)::value)
+					y_off[rt & 1][o] = (row_ok & (ow < g.Wo)) ? at : OUT_OF_RANGE;
+					if constexpr (HAS_Z)
 					{
 #pragma unroll
-						for (int h = 0; h < 2; h++)
-							residual[pass & 1][o][h] = __builtin_bit_cast(pair_t, __builtin_amdgcn_raw_buffer_load_b64(rz, static_cast<int>(y_off[pass & 1][o]), h * 64 * SZ, 0));
+						for (int tn = 0; tn < 2; tn++)
+							residual[rt & 1][o][tn] = __builtin_bit_cast(pair_t, __builtin_amdgcn_raw_buffer_load_b64(rz, static_cast<int>(y_off[rt & 1][o]), tn * UNIT_FILTERS * SZ, 0));
 					}
 				}
 			};
-			auto fold_and_store = [&](int pass, auto with_relu, auto with_z) __attribute__((always_inline))
+			auto hand_over = [&](int u) __attribute__((always_inline)) /* a finished unit into its fold buffer */
 			{
+				const int rt = u >> 1, tn = u & 1;
+				float *dst = sm + tn * UNIT_WORDS + (p * UNIT_ROWS + (lane & 31)) * UNIT_PITCH + fh * 32 + (lane >> 5) * 4;
 #pragma unroll
-				for (int h = 0; h < 2; h++)
+				for (int i = 0; i < 4; i++)
 				{
-					quad_t m[POSITIONS];
+					const typename Mma<f16_t>::acc_t &t = acc[rt][tn];
+					const quad_t run = { t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3] };
+					*reinterpret_cast<quad_t*>(dst + i * 8) = run;
+				}
+			};
+			quad_t held[2][POSITIONS]; /* a unit's four sums per output filter, read from its fold buffer a region before they are folded */
+			auto fetch = [&](int u) __attribute__((always_inline))
+			{
+				const int tn = u & 1;
+				const float *src = sm + tn * UNIT_WORDS + (tid >> 4) * UNIT_PITCH + (tid & 15) * 4;
 #pragma unroll
-					for (int q = 0; q < POSITIONS; q++)
-						m[q] = *reinterpret_cast<const quad_t*>(sm + (q * PASS_ROWS + (tid >> 4)) * FOLD_PITCH + h * 64 + (tid & 15) * 4);
-					float out[2][4];
+				for (int q = 0; q < POSITIONS; q++)
+					held[tn][q] = *reinterpret_cast<const quad_t*>(src + q * UNIT_ROWS * UNIT_PITCH);
+			};
+			auto fold_and_store = [&](int u) __attribute__((always_inline))
+			{
+				const int rt = u >> 1, tn = u & 1;
+				const quad_t (&m)[POSITIONS] = held[tn];
+				float out[2][4];
+#pragma unroll
+				for (int c = 0; c < 4; c++)
+				{
+					out[0][c] = m[0][c] + m[1][c] + m[2][c];
+					out[1][c] = m[1][c] - m[2][c] - m[3][c];
+				}
+#pragma unroll
+				for (int o = 0; o < 2; o++)
+				{
+					float t[4], zv[4];
+					union
+					{
+						Pack<TE, 4> e;
+						pair_t words;
+					} cast;
+					cast.words = residual[rt & 1][o][tn];
 #pragma unroll
 					for (int c = 0; c < 4; c++)
-					{
-						out[0][c] = m[0][c] + m[1][c] + m[2][c];
-						out[1][c] = m[1][c] - m[2][c] - m[3][c];
-					}
+						zv[c] = HAS_Z ? Traits<TE>::load(cast.e.v[c]) : 0.0f;
+					epi.template combine<RELU, HAS_Z, 4>(t, out[o], columns[tn], zv);
 #pragma unroll
-					for (int o = 0; o < 2; o++)
-					{
-						float t[4], zv[4];
-						union
-						{
-							Pack<TE, 4> e;
-							pair_t words;
-						} cast;
-						cast.words = residual[pass & 1][o][h];
+					for (int c = 0; c < 4; c++)
+						cast.e.v[c] = Traits<TE>::store(t[c]);
+					buffer_put<ROWS_STORE_POLICY>(ry, y_off[rt & 1][o] + tn * UNIT_FILTERS * SZ, cast.words);
+				}
+			};
+			auto products = [&](int u) __attribute__((always_inline))
+			{
+				const int rt = u >> 1, tn = u & 1;
 #pragma unroll
-						for (int c = 0; c < 4; c++)
-							zv[c] = decltype(with_z)::value ? Traits<TE>::load(cast.e.v[c]) : 0.0f;
-						epi.template combine<decltype(with_relu)::value, decltype(with_z)::value, 4>(t, out[o], columns[h], zv);
-#pragma unroll
-						for (int c = 0; c < 4; c++)
-							cast.e.v[c] = Traits<TE>::store(t[c]);
-						buffer_put<ROWS_STORE_POLICY>(ry, y_off[pass & 1][o] + h * 64 * SZ, cast.words);
-					}
+				for (int c = 0; c < ROW_TILE_CHUNKS; c++)
+				{
+					Mma<f16_t>::run(bq[(LAST_SLAB + c) % B_RING][tn], a[c], acc[rt][tn]);
+					if (tn == 1 && rt < 3)
+						read_a(LAST % RING, c / PHASE_SLABS, c % PHASE_SLABS, rt + 1, a[c]);
 				}
 			};
 #pragma unroll
-			for (int c = 0; c < A_AHEAD; c++)
-				read_a(LAST % RING, (c / PHASE_SLABS) % FILTER_ROWS, c % PHASE_SLABS, c / (FILTER_ROWS * PHASE_SLABS), a[c % A_RING]); /* chunk = (row tile, filter row, slab) */
-			auto hand_over = [&](int rt) __attribute__((always_inline)) /* a finished row tile's sums into the fold buffer */
+			for (int u = 0; u < UNITS + 3; u++)
 			{
+				__builtin_amdgcn_sched_barrier(0);
+#ifdef ROWS_KNOCK_LAST /* timing experiments only (wrong results): 1 no hand-over writes, 2 no fold, 8 no barriers */
+				constexpr int knock = ROWS_KNOCK_LAST;
+#else
+				constexpr int knock = 0;
+#endif
+				if (u >= 3 && !(knock & 2))
+					fold_and_store(u - 3);
+				if (u >= 2 && u <= UNITS + 1 && !(knock & 2))
+					fetch(u - 2);
+				if (u >= 1 && u <= UNITS && !(knock & 1))
+					hand_over(u - 1);
+				if (u < UNITS)
+				{
+					/* (row tile rt is placed in the region of its second unit: its residual has two regions to arrive) */
+					if ((u & 1) == 1)
+						place(u >> 1);
+					products(u);
+					if (u >= 2)
+						__builtin_amdgcn_sched_group_barrier(0x100, POSITIONS, 0); /* the reads of the fold buffer first */
 #pragma unroll
-				for (int tn = 0; tn < 2; tn++)
-#pragma unroll
-					for (int i = 0; i < 4; i++)
+					for (int c = 0; c < ROW_TILE_CHUNKS; c++)
 					{
-						const typename Mma<f16_t>::acc_t &t = acc[rt][tn];
-						const quad_t run = { t[4 * i], t[4 * i + 1], t[4 * i + 2], t[4 * i + 3] };
-						*reinterpret_cast<quad_t*>(sm + (p * PASS_ROWS + (lane & 31)) * FOLD_PITCH + fh * 64 + tn * 32 + i * 8 + (lane >> 5) * 4) = run;
+						__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+						if (u >= 1 && c < 4)
+							__builtin_amdgcn_sched_group_barrier(0x200, 1, 0); /* (all four writes in front of the MFMAs measured 7 % slower over the phase) */
+						if ((u & 1) == 1 && (u >> 1) < 3)
+							__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+						__builtin_amdgcn_sched_group_barrier(0x002, ROWS_UNIT_VALU, 0);
 					}
-			};
-			auto products = [&](int rt, int from, int to) __attribute__((always_inline)) /* chunk slots [from, to) of row tile rt */
-			{
-#pragma unroll
-				for (int k = from; k < to; k++)
-				{
-					const int i = k / PHASE_SLABS, sl = k % PHASE_SLABS;
-					const int c = rt * FILTER_ROWS * PHASE_SLABS + k, cn = c + A_AHEAD;
-					if (cn < 4 * FILTER_ROWS * PHASE_SLABS)
-						read_a(LAST % RING, (cn / PHASE_SLABS) % FILTER_ROWS, cn % PHASE_SLABS, cn / (FILTER_ROWS * PHASE_SLABS), a[cn % A_RING]);
-#pragma unroll
-					for (int tn = 0; tn < 2; tn++)
-						Mma<f16_t>::run(bq[(LAST_SLAB + i * PHASE_SLABS + sl) % B_RING][tn], a[c % A_RING], acc[rt][tn]);
-				}
-			};
-			constexpr int SLOTS = FILTER_ROWS * PHASE_SLABS, HEAD = 2; /* chunk slots of a row tile; those that carry the previous tile's hand-over */
-			place(0, with_z);
-#pragma unroll
-			for (int rt = 0; rt < 4; rt++)
-			{
-				/* Row tile rt in two scheduling regions.  The first slots carry, between their MFMAs, the writes of row tile rt - 1
-				 * into the fold buffer; behind the barrier that makes them visible the remaining slots carry its fold and its stores. */
-				__builtin_amdgcn_sched_barrier(0);
-				if (rt > 0)
-					hand_over(rt - 1);
-				products(rt, 0, HEAD);
-#pragma unroll
-				for (int k = 0; k < HEAD; k++)
-				{
-					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-					__builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-					if (rt > 0)
-						__builtin_amdgcn_sched_group_barrier(0x200, 8 / HEAD, 0);
 				}
 				__builtin_amdgcn_sched_barrier(0);
-				if (rt > 0)
-				{
-					__syncthreads();
-					fold_and_store(rt - 1, with_relu, with_z);
-					place(rt, with_z);
-				}
-				products(rt, HEAD, SLOTS);
-				if (rt > 0)
-					__builtin_amdgcn_sched_group_barrier(0x100, 8, 0); /* the eight reads of the fold first */
-#pragma unroll
-				for (int k = HEAD; k < SLOTS; k++)
-				{
-					__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-					__builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-					if (rt > 0)
-						__builtin_amdgcn_sched_group_barrier(0x002, 30, 0);
-				}
-				__builtin_amdgcn_sched_barrier(0);
-				if (rt == 0)
+				if (u == 1)
 					STAMP(6);
-				if (rt == 3)
+				if (u == UNITS - 1)
 					STAMP(7);
-				/* everyone has folded row tile rt - 1 (its values were consumed above) before anyone overwrites the buffer */
-				if (rt > 0)
+				/* (behind region UNITS + 1 nothing is written any more: the last fetch and the last two folds need no barrier) */
+				if (u <= UNITS && !(knock & 8))
 					__syncthreads();
 			}
-			hand_over(3);
-			__syncthreads();
-			fold_and_store(3, with_relu, with_z);
 			STAMP(3);
 		}
 		STAMP(4);
