@@ -46,8 +46,8 @@
 /* Instrumentation, compiled in with -DWINOGRAD_ROWS_STAMPS only: work-item 0 of every workgroup records the 100 MHz wall clock at
  * the phase boundaries of the kernel and avhip_debug_rows_stamps() copies the records of the last launch to the host. */
 #ifdef WINOGRAD_ROWS_STAMPS
-__device__ unsigned long long g_rows_stamps[4096 * 8];
-#define STAMP(i) do { if (threadIdx.x == 0) g_rows_stamps[(blockIdx.x % 4096) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+__device__ unsigned long long g_rows_stamps[4096 * 32];
+#define STAMP(i) do { if (threadIdx.x == 0) g_rows_stamps[(blockIdx.x % 4096) * 32 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
 extern "C" __attribute__((visibility("default"))) int avhip_debug_rows_stamps(void *out)
 {
 	return static_cast<int>(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_rows_stamps), sizeof(g_rows_stamps)));
@@ -497,20 +497,21 @@ namespace
 			pair_t residual[2][2][2]; /* [row tile parity][output pixel][half] */
 			auto place = [&](int rt) __attribute__((always_inline)) /* where the two output pixels of this work-item's (row, pair) of row tile rt go */
 			{
-				const int q = rt * UNIT_ROWS + (tid >> 4);
-				const int r = static_cast<int>((static_cast<unsigned int>(q) * g.pairs_magic) >> 20);
-				const int pair = q - r * g.pairs;
-				const int oh = oh0 + r;
-				const bool row_ok = (q < band_rows) & (oh < g.Ho);
+				/* (24-bit multiplies, which run at the full rate of the vector ALU, four times that of 32-bit ones: the launcher takes
+				 * filter counts below 2^24 only, and an image of a tensor below 2 GiB has fewer than 2^24 pixels) */
+				const unsigned int q = static_cast<unsigned int>(rt * UNIT_ROWS + (tid >> 4));
+				const unsigned int r = __umul24(q, g.pairs_magic) >> 20;
+				const int pair = static_cast<int>(q - __umul24(r, static_cast<unsigned int>(g.pairs)));
+				const int oh = oh0 + static_cast<int>(r);
+				const bool row_ok = (static_cast<int>(q) < band_rows) & (oh < g.Ho);
+				const int ow = ow0 + 2 * pair;
+				unsigned int first = (__umul24(__umul24(static_cast<unsigned int>(oh), static_cast<unsigned int>(g.Wo)) + static_cast<unsigned int>(ow), static_cast<unsigned int>(g.K)) + static_cast<unsigned int>(kcol)) * SZ;
+				/* opaque: a select of a product invites a branch around the product, and a branch here ends the scheduling region */
+				asm volatile("" : "+v"(first));
 #pragma unroll
 				for (int o = 0; o < 2; o++)
 				{
-					const int ow = ow0 + 2 * pair + o;
-					/* the offset computed whether or not the pixel exists, and opaque: a select of a product invites a branch around
-					 * the product, and a branch here ends the scheduling region */
-					unsigned int at = static_cast<unsigned int>((oh * g.Wo + ow) * g.K + kcol) * SZ;
-					asm volatile("" : "+v"(at));
-					y_off[rt & 1][o] = (row_ok & (ow < g.Wo)) ? at : OUT_OF_RANGE;
+					y_off[rt & 1][o] = (row_ok & (ow + o < g.Wo)) ? first + o * g.K * SZ : OUT_OF_RANGE;
 					if constexpr (HAS_Z)
 					{
 #pragma unroll
@@ -621,6 +622,7 @@ namespace
 					STAMP(6);
 				if (u == UNITS - 1)
 					STAMP(7);
+				STAMP(8 + u); /* (the end of every region of the last phase) */
 				/* (behind region UNITS + 1 nothing is written any more: the last fetch and the last two folds need no barrier) */
 				if (u <= UNITS && !(knock & 8))
 					__syncthreads();
@@ -673,7 +675,7 @@ namespace
 	int launch_rows(hipStream_t st, const avhipConvShape &s, const void *x, const void *U, const void *bias, const void *z, void *y, double alpha1,
 			double alpha2, int activation)
 	{
-		if ((s.C != 64 && s.C != 128 && s.C != 256) || s.K % ROWS_BLOCK_N != 0)
+		if ((s.C != 64 && s.C != 128 && s.C != 256) || s.K % ROWS_BLOCK_N != 0 || s.K >= (1 << 24)) /* (24-bit products in the output offsets) */
 			return AVHIP_NOT_SUPPORTED;
 		if (!aligned_to(x, 16) || !aligned_to(U, 16) || !aligned_to(y, 16) || (z != nullptr && !aligned_to(z, 16)) || (bias != nullptr && !aligned_to(bias, 16)))
 			return AVHIP_NOT_SUPPORTED;
