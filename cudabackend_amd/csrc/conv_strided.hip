@@ -110,7 +110,9 @@ namespace
 		U[e] = out.u;
 	}
 
-	template<typename TE>
+	/* RELU, HAS_Z: the activation (ReLU or none) and whether a residual is added, fixed per instance: a branch on either in the tail
+	 * would cut the scheduling regions in which the way out of a pair of row tiles sits between the MFMAs of the next pair. */
+	template<typename TE, bool RELU, bool HAS_Z>
 	__global__ __launch_bounds__(S_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_conv_strided(const TE *__restrict__ x, const void *__restrict__ U,
 			StridedGeom g, FloatEpilogue<TE> epi)
 	{
@@ -363,10 +365,7 @@ namespace
 				load_b((phase + 1) * S_TAPS * S_SLABS + HEAD_SLABS + j, bl[j]);
 		}
 		const __amdgpu_buffer_rsrc_t ry = make_buffer(epi.y + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
-		__amdgpu_buffer_rsrc_t rz = make_buffer(nullptr, 0);
-		if (epi.z != nullptr)
-			rz = make_buffer(epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K, static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ);
-		const bool relu = epi.activation == ACT_RELU, has_z = epi.z != nullptr;
+		const __amdgpu_buffer_rsrc_t rz = make_buffer(HAS_Z ? epi.z + static_cast<int64_t>(n) * g.Ho * g.Wo * g.K : nullptr, HAS_Z ? static_cast<unsigned int>(g.Ho * g.Wo * g.K) * SZ : 0u);
 		const int half = lane >> 5;
 		const int kwave = kb * S_FILTERS + wave * 32; /* this wavefront's first filter */
 		typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -383,46 +382,63 @@ namespace
 		asm volatile("" : "+v"(out_put));
 		int out_get = wave * OUT_BYTES + (lane >> 2) * OUT_PITCH + (lane & 3) * 16;
 		asm volatile("" : "+v"(out_get));
-		/* byte offset in y of GEMM row q of the tile (filter 0), or out of range */
+		/* byte offset in y of GEMM row q of the tile (filter 0), or out of range (24-bit multiplies, which run at the full rate of the
+		 * vector ALU: the launcher takes filter counts below 2^24 only, and an image of a tensor below 2 GiB has fewer than 2^24 pixels) */
 		auto y_offset = [&](int q, int filter) __attribute__((always_inline))
 		{
-			const int r = static_cast<int>((static_cast<unsigned int>(q) * g.pw_magic) >> 20), c = q - r * g.PW;
+			const int r = static_cast<int>(__umul24(static_cast<unsigned int>(q), g.pw_magic) >> 20), c = q - static_cast<int>(__umul24(static_cast<unsigned int>(r), static_cast<unsigned int>(g.PW)));
 			const int oh = oh0 + r, ow = ow0 + c;
 			const bool ok = (r < g.TH) & (c < g.TW) & (oh < g.Ho) & (ow < g.Wo);
-			return ok ? static_cast<unsigned int>((oh * g.Wo + ow) * g.K + filter) * SZ : OUT_OF_RANGE;
+			/* (computed whether or not the pixel exists, and opaque: a select of a product invites a branch around the product, and a
+			 * branch here ends the scheduling region) */
+			unsigned int at = (__umul24(__umul24(static_cast<unsigned int>(oh), static_cast<unsigned int>(g.Wo)) + static_cast<unsigned int>(ow), static_cast<unsigned int>(g.K)) + static_cast<unsigned int>(filter)) * SZ;
+			asm volatile("" : "+v"(at));
+			return ok ? at : OUT_OF_RANGE;
 		};
-		/* rounds row tile rt in the layout of the accumulators and puts it into place `at` (0 / 1) of the wavefront's piece */
-		auto round_tile = [&](int rt, int at, auto with_relu, auto with_z) __attribute__((always_inline))
+		/* The way out of a pair of row tiles (rt0, rt0 + 1) in thirteen parts, each of which sits behind one MFMA of the next pair:
+		 * parts 0..7 round run i (of four) of row tile t (of two) in the layout of the accumulators and put it into the wavefront's
+		 * piece of LDS; parts 8..12 read sixteen pixels each back as 16 bytes x 4 lanes per pixel and store them.  The residual of a pair
+		 * is asked for a region ahead (fetch_z): runs (2 pair, 2 pair + 1) of the two lanes of a pixel are 32 consecutive bytes of
+		 * z, 16 per lane, exchanged by the swap. */
+		u32x4_t zraw[2][2];
+		unsigned int zw[2][4];
+		uint4 back[2];
+		auto fetch_z = [&](int rt0, int count) __attribute__((always_inline))
 		{
-			constexpr bool RELU = decltype(with_relu)::value, HAS_Z = decltype(with_z)::value;
-			unsigned int zw[2][4] = { { 0u, 0u, 0u, 0u }, { 0u, 0u, 0u, 0u } };
 			if (HAS_Z)
 			{
-				/* runs (2 pair, 2 pair + 1) of the two lanes of a pixel are 32 consecutive bytes of z: 16 per lane, exchanged by the swap */
-				const int q = rt * 32 + (lane & 31);
 #pragma unroll
-				for (int pair = 0; pair < 2; pair++)
+				for (int t = 0; t < count; t++)
+#pragma unroll
+					for (int pair = 0; pair < 2; pair++)
+						zraw[t][pair] = __builtin_amdgcn_raw_buffer_load_b128(rz, static_cast<int>(y_offset((rt0 + t) * 32 + (lane & 31), kwave + 8 * (2 * pair + half))), 0, 2);
+			}
+		};
+		auto way_out = [&](int rt0, int count, int part) __attribute__((always_inline))
+		{
+			if (part < 8)
+			{
+				const int t = part >> 2, i = part & 3, rt = rt0 + t;
+				if (t >= count)
+					return;
+				if (HAS_Z && (i & 1) == 0)
 				{
-					const u32x4_t zr = __builtin_amdgcn_raw_buffer_load_b128(rz, static_cast<int>(y_offset(q, kwave + 8 * (2 * pair + half))), 0, 2);
+					const u32x4_t zr = zraw[t][i >> 1];
 					const auto s0 = __builtin_amdgcn_permlane32_swap(zr[0], zr[2], false, false);
 					const auto s1 = __builtin_amdgcn_permlane32_swap(zr[1], zr[3], false, false);
-					zw[pair][0] = s0[0]; /* run 2 pair, this lane's half */
-					zw[pair][1] = s1[0];
-					zw[pair][2] = s0[1]; /* run 2 pair + 1 */
-					zw[pair][3] = s1[1];
+					zw[t][0] = s0[0]; /* run i, this lane's half */
+					zw[t][1] = s1[0];
+					zw[t][2] = s0[1]; /* run i + 1 */
+					zw[t][3] = s1[1];
 				}
-			}
-#pragma unroll
-			for (int i = 0; i < 4; i++)
-			{
 				union
 				{
 					Pack<TE, 4> p;
 					unsigned int w[2];
 					uint2 u;
 				} zin, out;
-				zin.w[0] = zw[i >> 1][2 * (i & 1)];
-				zin.w[1] = zw[i >> 1][2 * (i & 1) + 1];
+				zin.w[0] = HAS_Z ? zw[t][2 * (i & 1)] : 0u;
+				zin.w[1] = HAS_Z ? zw[t][2 * (i & 1) + 1] : 0u;
 #pragma unroll
 				for (int e = 0; e < 4; e++)
 				{
@@ -431,34 +447,24 @@ namespace
 						r += epi.alpha2 * Traits<TE>::load(zin.p.v[e]);
 					out.p.v[e] = Traits<TE>::store(RELU ? __builtin_fmaxf(r, 0.0f) : r);
 				}
-				*reinterpret_cast<uint2*>(lds + out_put + at * 32 * OUT_PITCH + 8 * i * static_cast<int>(SZ)) = out.u;
+				*reinterpret_cast<uint2*>(lds + out_put + t * 32 * OUT_PITCH + 8 * i * static_cast<int>(SZ)) = out.u;
+			}
+			else
+			{
+				/* lane l: 16 bytes (l % 4) of pixel l / 4 + 16 it; read back a part ahead of its store */
+				const int it = part - 8;
+				if (it < 2 * count)
+					back[it & 1] = *reinterpret_cast<const uint4*>(lds + out_get + it * 16 * OUT_PITCH);
+				if (it >= 1 && it - 1 < 2 * count)
+				{
+					const uint4 run = back[(it - 1) & 1];
+					const unsigned int offset = y_offset(rt0 * 32 + (it - 1) * 16 + (lane >> 2), kwave + (lane & 3) * 8);
+					const u32x4_t words = { run.x, run.y, run.z, run.w };
+					__builtin_amdgcn_raw_buffer_store_b128(words, ry, static_cast<int>(offset), 0, 17); /* sc0 sc1: written through as the kernel runs */
+				}
 			}
 		};
-		/* the way out of `count` row tiles from row tile rt0 on: rounded, through the wavefront's piece of LDS, stored */
-		auto leave = [&](int rt0, int count) __attribute__((always_inline))
-		{
-#pragma unroll
-			for (int t = 0; t < count; t++)
-			{
-				if (relu && has_z)
-					round_tile(rt0 + t, t, std::true_type(), std::true_type());
-				else if (relu)
-					round_tile(rt0 + t, t, std::true_type(), std::false_type());
-				else if (has_z)
-					round_tile(rt0 + t, t, std::false_type(), std::true_type());
-				else
-					round_tile(rt0 + t, t, std::false_type(), std::false_type());
-			}
-			/* lane l: 16 bytes (l % 4) of pixel l / 4 + 16 it */
-#pragma unroll
-			for (int it = 0; it < 2 * count; it++)
-			{
-				const uint4 run = *reinterpret_cast<const uint4*>(lds + out_get + it * 16 * OUT_PITCH);
-				const unsigned int offset = y_offset(rt0 * 32 + it * 16 + (lane >> 2), kwave + (lane & 3) * 8);
-				const u32x4_t words = { run.x, run.y, run.z, run.w };
-				__builtin_amdgcn_raw_buffer_store_b128(words, ry, static_cast<int>(offset), 0, 17); /* sc0 sc1: written through as the kernel runs */
-			}
-		};
+		constexpr int WAY_OUT_PARTS = 13;
 		/* chunk n of the tail = (pair of row tiles, tap, slab, row tile of the pair) in the order of use */
 		auto tail_chunk = [&](int n, int &rt, int &tap, int &sl) __attribute__((always_inline))
 		{
@@ -484,32 +490,38 @@ namespace
 #pragma unroll
 		for (int pair = 0; pair < 4; pair++)
 		{
-			/* one scheduling region: the products of a pair of row tiles, and among them the way out of the pair before */
-			__builtin_amdgcn_sched_barrier(0);
-			const int width = pair < 3 ? 2 : 1, n0 = pair * TAIL_SLABS * 2;
-			if (pair > 0)
-				leave(2 * (pair - 1), 2);
+			/* The products of a pair of row tiles, slot by slot with a fence for the scheduler between slots: one MFMA and, behind it,
+			 * the parts of the way out of the pair before that fall to the slot; the residual of this pair is asked for once those
+			 * parts no longer need the one before. */
+			const int width = pair < 3 ? 2 : 1, n0 = pair * TAIL_SLABS * 2, slots = TAIL_SLABS * width;
 #pragma unroll
-			for (int m = 0; m < TAIL_SLABS * width; m++)
+			for (int m = 0; m < slots; m++)
 			{
+				__builtin_amdgcn_sched_barrier(0);
 				const int n = n0 + m;
 				if (n + A_AHEAD < TAIL_CHUNKS)
 					read_tail(n + A_AHEAD, a[(n + A_AHEAD) % A_RING]);
 				int rt, tap, sl;
 				tail_chunk(n, rt, tap, sl);
 				Mma<TE>::run(bl[(tap - HEAD_TAPS) * S_SLABS + sl], a[n % A_RING], acc[rt]);
-			}
-#pragma unroll
-			for (int m = 0; m < TAIL_SLABS * width; m++)
-			{
-				__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-				__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 				if (pair > 0)
-					__builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+				{
+					/* (in their order: a part that reads the piece of LDS back follows the parts that wrote what it reads) */
+					const int first = slots >= WAY_OUT_PARTS ? (m < WAY_OUT_PARTS ? m : WAY_OUT_PARTS) : m * WAY_OUT_PARTS / slots;
+					const int last = slots >= WAY_OUT_PARTS ? (m < WAY_OUT_PARTS ? m + 1 : WAY_OUT_PARTS) : (m + 1) * WAY_OUT_PARTS / slots;
+#pragma unroll
+					for (int part = first; part < last; part++)
+						way_out(2 * (pair - 1), 2, part);
+				}
+				static_assert(TAIL_SLABS > 8, "the residual of a pair is asked for behind part 7 of the pair before");
+				if (m == (pair > 0 ? 8 : 0))
+					fetch_z(2 * pair, width);
 			}
 		}
 		__builtin_amdgcn_sched_barrier(0);
-		leave(6, 1);
+#pragma unroll
+		for (int part = 0; part < WAY_OUT_PARTS; part++)
+			way_out(6, 1, part);
 		SSTAMP(4);
 	}
 
@@ -542,7 +554,7 @@ namespace
 	bool strided_shape_ok(const avhipConvShape &s)
 	{
 		return s.R == 3 && s.S == 3 && s.stride_h == 2 && s.stride_w == 2 && s.dil_h == 1 && s.dil_w == 1 && s.C % 64 == 0 && s.C >= 64 && s.K % S_FILTERS == 0
-				&& s.N > 0 && s.Ho > 0 && s.Wo > 0;
+				&& s.N > 0 && s.Ho > 0 && s.Wo > 0 && s.K < (1 << 24); /* (24-bit products in the output offsets) */
 	}
 	std::atomic<int> strided_mode { 1 };
 
@@ -582,7 +594,14 @@ namespace
 		const FloatEpilogue<TE> epi { static_cast<const float*>(bias), static_cast<const TE*>(z), static_cast<TE*>(y), static_cast<float>(alpha1),
 				static_cast<float>(alpha2), 0.0f, activation, s.K, true };
 		const dim3 grid(static_cast<unsigned int>(items), static_cast<unsigned int>(s.K / S_FILTERS));
-		hipLaunchKernelGGL((k_conv_strided<TE>), grid, dim3(S_THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+		if (activation == ACT_RELU && z != nullptr)
+			hipLaunchKernelGGL((k_conv_strided<TE, true, true>), grid, dim3(S_THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+		else if (activation == ACT_RELU)
+			hipLaunchKernelGGL((k_conv_strided<TE, true, false>), grid, dim3(S_THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+		else if (z != nullptr)
+			hipLaunchKernelGGL((k_conv_strided<TE, false, true>), grid, dim3(S_THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
+		else
+			hipLaunchKernelGGL((k_conv_strided<TE, false, false>), grid, dim3(S_THREADS), 0, st, static_cast<const TE*>(x), U, g, epi);
 		return 0;
 	}
 }
