@@ -59,6 +59,9 @@ extern "C" __attribute__((visibility("default"))) int avhip_debug_rows_stamps(vo
 #ifndef ROWS_UNIT_VALU
 #define ROWS_UNIT_VALU 10 /* vector-ALU instructions of the fold behind every MFMA of the last phase */
 #endif
+#ifndef ROWS_TRANSFORM_SLOTS
+#define ROWS_TRANSFORM_SLOTS 1
+#endif
 #ifndef ROWS_STORE_POLICY
 #define ROWS_STORE_POLICY 17 /* sc0 sc1: written through as the kernel runs, no streaming hint */
 #endif
@@ -235,20 +238,22 @@ namespace
 		 * registers (rings of four and eight measured the same: the way ahead is not what the requests cost). */
 		constexpr int B_RING = FILTER_ROWS * PHASE_SLABS, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
 		Chunk bq[B_RING][2];
-		auto load_b = [&](int slab, Chunk (&set)[2]) __attribute__((always_inline)) /* slab: (step, slab of the step), over the whole k walk */
+		auto load_b_tile = [&](int slab, int tn, Chunk &into) __attribute__((always_inline)) /* slab: (step, slab of the step), over the whole k walk */
 		{
 			const int step = slab / PHASE_SLABS, sl = slab - step * PHASE_SLABS;
 #ifdef ROWS_KNOCK_B /* timing experiment only: no filter requests inside the k loop (wrong results) */
 			if (slab >= B_AHEAD)
 				return;
 #endif
+			const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(ru, static_cast<int>(b_offset + tn * 2 * PHASE_SLABS * OPERAND_BYTES),
+					static_cast<int>(step * step_stride + sl * OPERAND_BYTES), 0);
+			into.u = make_uint4(v[0], v[1], v[2], v[3]);
+		};
+		auto load_b = [&](int slab, Chunk (&set)[2]) __attribute__((always_inline))
+		{
 #pragma unroll
 			for (int tn = 0; tn < 2; tn++)
-			{
-				const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(ru, static_cast<int>(b_offset + tn * 2 * PHASE_SLABS * OPERAND_BYTES),
-						static_cast<int>(step * step_stride + sl * OPERAND_BYTES), 0);
-				set[tn].u = make_uint4(v[0], v[1], v[2], v[3]);
-			}
+				load_b_tile(slab, tn, set[tn]);
 		};
 
 		/* transform side: this work-item's (row, pair, 8 channels) of every phase */
@@ -307,6 +312,25 @@ namespace
 #pragma unroll
 			for (int q = 0; q < POSITIONS; q++)
 				*reinterpret_cast<uint4*>(dst + q * POSITION_BYTES) = __builtin_bit_cast(uint4, v[q]);
+		};
+		/* the same in eight parts, one behind each pair of MFMAs of the step that carries it, ordered so that few converted pixels
+		 * are alive at a time: d0, d2, plane 0, d1, plane 1, plane 2, d3, plane 3 */
+		Half8 td[4];
+		auto transform_part = [&](int slot, int part) __attribute__((always_inline))
+		{
+			constexpr int convert[8] = { 0, 2, -1, 1, -1, -1, 3, -1 }, plane[8] = { -1, -1, 0, -1, 1, 2, -1, 3 };
+			if (convert[part] >= 0)
+				td[convert[part]] = to_half8(raw[convert[part]], TE());
+			else
+			{
+				const int q = plane[part];
+				Half8 v;
+#pragma unroll
+				for (int e = 0; e < 4; e++)
+					v.h[e] = q == 0 ? pk_sub(td[0].h[e], td[2].h[e]) : q == 1 ? td[1].h[e] + td[2].h[e] : q == 2 ? pk_sub(td[2].h[e], td[1].h[e]) : pk_sub(td[1].h[e], td[3].h[e]);
+				char *dst = lds + (slot >> 1) * SLICE_BYTES + (slot & 1) * 64 + v_dst;
+				*reinterpret_cast<uint4*>(dst + q * POSITION_BYTES) = __builtin_bit_cast(uint4, v);
+			}
 		};
 		load_x(0); /* what the first MFMA waits for longest goes out first */
 #pragma unroll
@@ -372,6 +396,42 @@ namespace
 					const bool transform_here = i == 1;
 					if (i == 2)
 						__syncthreads();
+#if ROWS_TRANSFORM_SLOTS
+					if (transform_here)
+					{
+						/* The step that carries the transform is written slot by slot, a fence for the scheduler between slots: the
+						 * requests of the slot, two MFMAs, one part of the transform.  (Laid out by groups like the other steps the
+						 * scheduler put three quarters of the transform into one run of fifty vector instructions behind the fourth
+						 * MFMA.) */
+#pragma unroll
+						for (int sl = 0; sl < PHASE_SLABS; sl++)
+						{
+							const int slab = step * PHASE_SLABS + sl;
+#pragma unroll
+							for (int rt = 0; rt < 4; rt++)
+							{
+								__builtin_amdgcn_sched_barrier(0);
+								if (slab + B_AHEAD < SLABS_TOTAL && (rt == 0 || rt == 2))
+									load_b_tile(slab + B_AHEAD, rt >> 1, bq[(slab + B_AHEAD) % B_RING][rt >> 1]);
+								const int c = (step * PHASE_SLABS + sl) * 4 + rt;
+								const int cn = c + A_AHEAD;
+								if (cn < CHUNKS)
+								{
+									const int nstep = cn / STEP_CHUNKS_A, nphase = nstep / FILTER_ROWS;
+									read_a(nphase % RING, nstep % FILTER_ROWS, (cn / 4) % PHASE_SLABS, cn % 4, a[cn % A_RING]);
+								}
+#pragma unroll
+								for (int tn = 0; tn < 2; tn++)
+									Mma<f16_t>::run(bq[slab % B_RING][tn], a[c % A_RING], acc[rt][tn]);
+								transform_part((phase + 1) % RING, sl * 4 + rt);
+							}
+						}
+						__builtin_amdgcn_sched_barrier(0);
+						if (phase + 2 < PHASES)
+							load_x(phase + 2);
+						continue;
+					}
+#endif
 #pragma unroll
 					for (int sl = 0; sl < PHASE_SLABS; sl++)
 					{
