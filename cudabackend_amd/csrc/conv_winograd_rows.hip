@@ -204,21 +204,75 @@ namespace
 		const int p = wave & 3; /* plane of this wavefront */
 		const int fh = wave >> 2; /* its 32 filters of either 64-filter half of the block */
 
-		/* (image, band, segment) and filter block.  Where workgroups share input (several tiles per image: neighbouring bands
-		 * read two rows in common; several filter blocks: each reads the whole tile) they are renumbered so that the filter
-		 * blocks of a tile and then the tiles of an image follow each other on one XCD, whose L2 then serves the second reader. */
-		int n = static_cast<int>(blockIdx.x), band = 0, segment = 0, kb = 0;
-		if (g.bands * g.segments != 1 || gridDim.y != 1)
+		/* (image, band, segment) and filter block of workgroup number b.  Where workgroups share input (several tiles per image:
+		 * neighbouring bands read two rows in common; several filter blocks: each reads the whole tile) they are renumbered so that the
+		 * filter blocks of a tile and then the tiles of an image follow each other on one XCD, whose L2 then serves the second reader. */
+		const unsigned int filter_blocks = static_cast<unsigned int>(g.filter_tiles) / 4u;
+		const unsigned int all_blocks = static_cast<unsigned int>(g.images * g.bands * g.segments) * filter_blocks;
+		auto tile_of = [&](unsigned int b, int &n, int &band, int &segment, int &kb) __attribute__((always_inline))
 		{
-			unsigned int item, filter_block;
-			xcd_tile(item, filter_block);
-			kb = static_cast<int>(filter_block);
-			const int per_image = g.bands * g.segments;
-			n = static_cast<int>(item) / per_image;
-			const int tile = static_cast<int>(item) - n * per_image;
-			band = tile / g.segments;
-			segment = tile - band * g.segments;
-		}
+			n = static_cast<int>(b);
+			band = segment = kb = 0;
+			if (g.bands * g.segments != 1 || filter_blocks != 1)
+			{
+				const unsigned int t = xcd_block(b, all_blocks);
+				const unsigned int item = t / filter_blocks;
+				kb = static_cast<int>(t - item * filter_blocks);
+				const int per_image = g.bands * g.segments;
+				n = static_cast<int>(item) / per_image;
+				const int tile = static_cast<int>(item) - n * per_image;
+				band = tile / g.segments;
+				segment = tile - band * g.segments;
+			}
+		};
+		/* transform side: this work-item's (row, pair, 8 channels) of every phase of a tile: where its four pixels are read and where
+		 * its four planes go (what depends on the block is the same for all work-items and stays in scalar registers; a work-item
+		 * adds its own constants) */
+		auto pixels_of = [&](unsigned int b, unsigned int (&src)[4], int &dst) __attribute__((always_inline))
+		{
+			const int t_chunk = tid & 3;
+			const int t_pixel = tid >> 2;
+			const int t_row = static_cast<int>(__umul24(static_cast<unsigned int>(t_pixel), g.pairs_magic) >> 20);
+			const int t_pair = t_pixel - t_row * g.pairs;
+			const unsigned int t_base = (static_cast<unsigned int>(t_row * g.W + 2 * t_pair) * g.C + t_chunk * 8) * SZ;
+			int n, band, segment, kb;
+			tile_of(b, n, band, segment, kb);
+			const int ih0 = band * g.TH + g.pad_h, v_rows = g.TH + 2;
+			int top = -ih0 < 0 ? 0 : -ih0;
+			top = top > v_rows ? v_rows : top;
+			int bottom = ih0 + v_rows - g.H < 0 ? 0 : ih0 + v_rows - g.H;
+			bottom = bottom > v_rows - top ? v_rows - top : bottom;
+			const int real_rows = b < all_blocks ? v_rows - top - bottom : 0;
+			const int iw0 = segment * 2 * g.pairs + g.pad_w; /* column of the tile's first pixel */
+			const unsigned int origin = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(((n * g.H + ih0 + top) * g.W + iw0) * g.C * static_cast<int>(SZ)));
+			const bool t_valid = t_row < real_rows;
+#pragma unroll
+			for (int j = 0; j < 4; j++)
+			{
+				const int iw = iw0 + 2 * t_pair + j;
+				const bool inside = t_valid & (static_cast<unsigned int>(iw) < static_cast<unsigned int>(g.W));
+				src[j] = inside ? origin + t_base + static_cast<unsigned int>(j * g.C) * SZ : OUT_OF_RANGE;
+			}
+			dst = (t_valid ? (top + t_row) * g.pairs + t_pair : PIXELS_MAX) * PITCH + t_chunk * 16;
+		};
+		const __amdgpu_buffer_rsrc_t rx = make_buffer(x, static_cast<unsigned int>(g.images) * g.H * g.W * g.C * SZ);
+		uint4 raw[4];
+		auto load_x_from = [&](const unsigned int (&src)[4], int phase) __attribute__((always_inline))
+		{
+			/* (an out-of-range offset stays out of range with the phase added: tensors here are below 2 GiB) */
+#pragma unroll
+			for (int j = 0; j < 4; j++)
+			{
+				const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rx, static_cast<int>(src[j]), phase * PHASE_CHANNELS * static_cast<int>(SZ), 0);
+				raw[j] = make_uint4(v[0], v[1], v[2], v[3]);
+			}
+		};
+		/* (the ring of filter registers: see load_b) */
+		constexpr int B_RING = FILTER_ROWS * PHASE_SLABS, B_AHEAD = B_RING - 1;
+		Chunk bq[B_RING][2];
+		const unsigned int block = blockIdx.y * gridDim.x + blockIdx.x;
+		int n, band, segment, kb;
+		tile_of(block, n, band, segment, kb);
 		const int oh0 = band * g.TH;
 		const int ow0 = segment * 2 * g.pairs;
 		const int ih0 = oh0 + g.pad_h; /* input row of V row 0 */
@@ -236,18 +290,21 @@ namespace
 		/* Filters go through a ring of register sets, one set = the two filter tiles of one 16-channel slab (two slabs per step),
 		 * requested B_AHEAD slabs before they are multiplied: six sets, one phase's worth, which is what the last phase keeps in
 		 * registers (rings of four and eight measured the same: the way ahead is not what the requests cost). */
-		constexpr int B_RING = FILTER_ROWS * PHASE_SLABS, B_AHEAD = B_RING - 1, SLABS_TOTAL = STEPS * PHASE_SLABS;
-		Chunk bq[B_RING][2];
-		auto load_b_tile = [&](int slab, int tn, Chunk &into) __attribute__((always_inline)) /* slab: (step, slab of the step), over the whole k walk */
+		constexpr int SLABS_TOTAL = STEPS * PHASE_SLABS;
+		auto load_b_at = [&](unsigned int offset, int slab, int tn, Chunk &into) __attribute__((always_inline)) /* slab: (step, slab of the step), over the whole k walk */
 		{
 			const int step = slab / PHASE_SLABS, sl = slab - step * PHASE_SLABS;
+			const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(ru, static_cast<int>(offset + tn * 2 * PHASE_SLABS * OPERAND_BYTES),
+					static_cast<int>(step * step_stride + sl * OPERAND_BYTES), 0);
+			into.u = make_uint4(v[0], v[1], v[2], v[3]);
+		};
+		auto load_b_tile = [&](int slab, int tn, Chunk &into) __attribute__((always_inline))
+		{
 #ifdef ROWS_KNOCK_B /* timing experiment only: no filter requests inside the k loop (wrong results) */
 			if (slab >= B_AHEAD)
 				return;
 #endif
-			const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(ru, static_cast<int>(b_offset + tn * 2 * PHASE_SLABS * OPERAND_BYTES),
-					static_cast<int>(step * step_stride + sl * OPERAND_BYTES), 0);
-			into.u = make_uint4(v[0], v[1], v[2], v[3]);
+			load_b_at(b_offset, slab, tn, into);
 		};
 		auto load_b = [&](int slab, Chunk (&set)[2]) __attribute__((always_inline))
 		{
@@ -256,40 +313,16 @@ namespace
 				load_b_tile(slab, tn, set[tn]);
 		};
 
-		/* transform side: this work-item's (row, pair, 8 channels) of every phase */
-		const __amdgpu_buffer_rsrc_t rx = make_buffer(x, static_cast<unsigned int>(g.images) * g.H * g.W * g.C * SZ);
-		const int t_chunk = tid & 3;
-		const int t_pixel = tid >> 2;
-		const int t_row = static_cast<int>((static_cast<unsigned int>(t_pixel) * g.pairs_magic) >> 20);
-		const int t_pair = t_pixel - t_row * g.pairs;
-		const bool t_valid = t_row < real_rows;
 		unsigned int x_src[4];
-		{
-			const int ih = ih0 + top + t_row;
-			const unsigned int line = (static_cast<unsigned int>(n) * g.H + static_cast<unsigned int>(ih)) * g.W;
-#pragma unroll
-			for (int j = 0; j < 4; j++)
-			{
-				const int iw = ow0 + 2 * t_pair + g.pad_w + j;
-				const bool inside = t_valid & (static_cast<unsigned int>(iw) < static_cast<unsigned int>(g.W));
-				x_src[j] = inside ? ((line + static_cast<unsigned int>(iw)) * g.C + t_chunk * 8) * SZ : OUT_OF_RANGE;
-			}
-		}
-		const int v_dst = (t_valid ? (top + t_row) * g.pairs + t_pair : PIXELS_MAX) * PITCH + t_chunk * 16;
-		uint4 raw[4];
+		int v_dst;
+		pixels_of(block, x_src, v_dst);
 		auto load_x = [&](int phase) __attribute__((always_inline))
 		{
 #ifdef ROWS_KNOCK_X /* timing experiment only: no pixel requests inside the k loop (wrong results) */
 			if (phase >= 2)
 				return;
 #endif
-			/* (an out-of-range offset stays out of range with the phase added: tensors here are below 2 GiB) */
-#pragma unroll
-			for (int j = 0; j < 4; j++)
-			{
-				const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rx, static_cast<int>(x_src[j]), phase * PHASE_CHANNELS * static_cast<int>(SZ), 0);
-				raw[j] = make_uint4(v[0], v[1], v[2], v[3]);
-			}
+			load_x_from(x_src, phase);
 		};
 		/* B^T d for this work-item's pixels; work-items without a (row, pair) of the band write to a spare pixel, so that the
 		 * transform is straight-line code the scheduler can spread among the MFMAs */
@@ -372,9 +405,22 @@ namespace
 		constexpr int A_RING = 6, A_AHEAD = 4, STEP_CHUNKS_A = PHASE_SLABS * 4;
 		Chunk a[A_RING];
 		/* (slot: which of the ring's places in LDS holds the phase) */
-		auto read_a = [&](int slot, int i, int sl, int rt, Chunk &dst) __attribute__((always_inline))
+		/* (With more phases than slots the addresses of phase ph + 4 are those of phase ph; left to itself the compiler keeps every
+		 * sum of a base and an offset beyond the 16 bits of the instruction alive for four phases, some 26 registers at the peak.
+		 * An opaque copy of the base per phase makes them things of one phase.) */
+		int a_base[2] = { a_off, a_off };
+		auto fresh_a_base = [&](int phase) __attribute__((always_inline))
 		{
-			dst.u = *reinterpret_cast<const uint4*>(lds + (slot >> 1) * SLICE_BYTES + (slot & 1) * 64 + sl * 32 + i * tap_shift + rt * 32 * PITCH + a_off);
+			if (PHASES > RING)
+			{
+				a_base[phase & 1] = a_off;
+				asm volatile("" : "+v"(a_base[phase & 1]));
+			}
+		};
+		auto read_a = [&](int phase, int i, int sl, int rt, Chunk &dst) __attribute__((always_inline))
+		{
+			const int slot = phase % RING;
+			dst.u = *reinterpret_cast<const uint4*>(lds + (slot >> 1) * SLICE_BYTES + (slot & 1) * 64 + sl * 32 + i * tap_shift + rt * 32 * PITCH + a_base[phase & 1]);
 		};
 		/* All phases but the last, written out (the last one walks its products row tile by row tile, see below).  With more
 		 * phases than LDS has slots a phase's V takes the slot of phase - RING, whose readers are long gone (above). */
@@ -385,6 +431,7 @@ namespace
 #pragma unroll
 			for (int phase = 0; phase < COUNT; phase++)
 			{
+				fresh_a_base(phase + 1);
 #pragma unroll
 				for (int i = 0; i < FILTER_ROWS; i++)
 				{
@@ -418,7 +465,7 @@ namespace
 								if (cn < CHUNKS)
 								{
 									const int nstep = cn / STEP_CHUNKS_A, nphase = nstep / FILTER_ROWS;
-									read_a(nphase % RING, nstep % FILTER_ROWS, (cn / 4) % PHASE_SLABS, cn % 4, a[cn % A_RING]);
+									read_a(nphase, nstep % FILTER_ROWS, (cn / 4) % PHASE_SLABS, cn % 4, a[cn % A_RING]);
 								}
 #pragma unroll
 								for (int tn = 0; tn < 2; tn++)
@@ -452,7 +499,7 @@ namespace
 							if (cn < CHUNKS)
 							{
 								const int nstep = cn / STEP_CHUNKS_A, nphase = nstep / FILTER_ROWS;
-								read_a(nphase % RING, nstep % FILTER_ROWS, (cn / 4) % PHASE_SLABS, cn % 4, a[cn % A_RING]);
+								read_a(nphase, nstep % FILTER_ROWS, (cn / 4) % PHASE_SLABS, cn % 4, a[cn % A_RING]);
 							}
 #pragma unroll
 							for (int tn = 0; tn < 2; tn++)
@@ -545,7 +592,7 @@ namespace
 			/* the six pixel operands of row tile 0; those of row tile rt + 1 take their places as the second unit of rt lets go of them */
 #pragma unroll
 			for (int c = 0; c < ROW_TILE_CHUNKS; c++)
-				read_a(LAST % RING, c / PHASE_SLABS, c % PHASE_SLABS, 0, a[c]);
+				read_a(LAST, c / PHASE_SLABS, c % PHASE_SLABS, 0, a[c]);
 			/* A work-item folds and stores, for one (row, pair) of a row tile, 4 filters of each half of the block: sixteen lanes
 			 * read 64 consecutive words of a fold-buffer row (every bank once) and write one whole 128-byte line of y. */
 			typename FloatEpilogue<TE>::template ColumnsT<4> columns[2];
@@ -640,7 +687,7 @@ namespace
 				{
 					Mma<f16_t>::run(bq[(LAST_SLAB + c) % B_RING][tn], a[c], acc[rt][tn]);
 					if (tn == 1 && rt < 3)
-						read_a(LAST % RING, c / PHASE_SLABS, c % PHASE_SLABS, rt + 1, a[c]);
+						read_a(LAST, c / PHASE_SLABS, c % PHASE_SLABS, rt + 1, a[c]);
 				}
 			};
 #pragma unroll

@@ -118,6 +118,37 @@ def test_through_the_dispatcher(oracle, rows_forced, dtype, case):
     assert err < BAR
 
 
+ROUNDS_CASES = [
+    # layers of more workgroups than the device has compute units (several rounds of workgroups)
+    dict(x=(70, 28, 28, 64), w=(128, 3, 3, 64)),                                          # 280 workgroups
+    dict(x=(44, 20, 20, 128), w=(512, 3, 3, 128), z=True),                                # 2 bands x 4 filter blocks x 44 images = 352, residual
+    dict(x=(10, 56, 56, 256), w=(256, 3, 3, 256), relu=False),                            # config 3's layer on 10 images: 140 tiles x 2 filter blocks, eight phases
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("case", range(len(ROUNDS_CASES)))
+def test_several_rounds_of_workgroups(oracle, rows_forced, dtype, case):
+    cs = ROUNDS_CASES[case]
+    g = h.rng(390 + case)
+    xs, ws = cs["x"], cs["w"]
+    s = shape_of(xs, ws)
+    groups = C.c_int(0)
+    assert rows_forced.avhip_conv2d_winograd_rows_plan(h.DT[dtype], C.byref(s), C.byref(groups), None) == 0
+    assert groups.value > 256, "the case must be more than one round of workgroups on the 256 compute units of an MI355X"
+    x = h.rounded(oracle, g.standard_normal(xs), dtype)
+    w = he(g, ws, dtype, oracle)
+    b = g.uniform(-0.1, 0.1, ws[0]).astype(np.float32).astype(np.float64)
+    ys = (xs[0], s.Ho, s.Wo, ws[0])
+    z = h.rounded(oracle, g.standard_normal(ys), dtype) if cs.get("z") else None
+    relu = cs.get("relu", True)
+    got = h.conv_forward("dispatch", x, w, ys, dtype, bias=b, z=z, activation=cb.ACTIVATION_RELU if relu else 0)
+    want = oracle.conv2d(x, w, b, z=z, activation=oracle.RELU if relu else oracle.LINEAR)
+    err = oracle.rel_l2(got, want)
+    print("rows rounds %s case %d rel-L2 = %.3e" % (dtype, case, err))
+    assert err < BAR
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_kernel_layer_entry(oracle, dtype):
     """avhip_winograd_rows_weight_transform + avhip_conv2d_winograd_rows called as a foreign host would: raw device pointers."""
