@@ -34,7 +34,7 @@ SEED = 0xA70CAD0
 # pass), from the FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/winograd_rows_bf16_cfg2_hbm_traffic.md.  Counters
 # cannot be read from inside this process, so the figure is a CONSTANT carried here, not a measurement of this run; it is only
 # reported for the dtype it was taken on.
-COUNTED_TRAFFIC_BYTES = {"bf16": 40.27e6}
+COUNTED_TRAFFIC_BYTES = {"bf16": 40.22e6}
 LONG_CALL_REPLAYS = 4  # graph replays per timing for side-leg calls of 50 us and more (time_calls)
 
 
