@@ -19,8 +19,8 @@
  * (the one-dimensional factors of the F(2x2,3x3) tables of src/winograd_nonfused.cu:534-575, signs moved between B and A).
  *
  * Workgroup = 8 wavefronts = one tile of TH output rows x `pairs` column pairs of one image x 128 filters; GEMM rows are
- * (row, column pair), at most 128.  Wavefront (p, half) owns plane M_p for 64 filters: 4 x 2 MFMA tiles of 32 x 32, 128
- * accumulator registers.
+ * (row, column pair), at most 128.  Wavefront (p, fh) owns plane M_p for 64 filters (32 of either 64-filter half of the block):
+ * 4 x 2 MFMA tiles of 32 x 32, 128 accumulator registers.
  *   A operand: V_p lives in LDS, [phase slot][p][pixel = row * pairs + pair][128 bytes + 16], fp16; filter row i is a constant
  *              shift of i * pairs pixels, so a 32-row tile always reads 32 consecutive pixels (conflict-free).
  *              V is produced in the kernel, 32 channels per phase: every work-item loads the four pixels of one
@@ -30,9 +30,12 @@
  *              transform below: [phase][filter row][p][tile of 32 filters][16-channel slab][lane][16 bytes], one contiguous
  *              kilobyte per wavefront load, requested several slabs ahead through a ring of register sets.  No LDS, so no
  *              barrier inside a phase.
- *   Epilogue : runs inside the last phase.  That phase keeps its filters in registers and takes its products row tile by row
- *              tile; a finished row tile's four planes go through LDS (32 rows), a work-item folds them into two output pixels x
- *              8 filters, applies bias / residual / ReLU and stores 16 bytes per pixel while the next row tile is multiplied.
+ *   Epilogue : runs inside the last phase.  That phase keeps its filters in registers and takes its products MFMA tile by MFMA
+ *              tile (a unit); a finished unit's four planes go through one of two buffers in LDS, a work-item folds them into
+ *              two output pixels x 4 filters, applies bias / residual / ReLU and stores 8 bytes per pixel (sixteen lanes: a whole
+ *              128-byte line) while later units are multiplied: see the last phase in the kernel.
+ *   Instances: per tensor type, channel count, activation (ReLU or none) and residual (present or not): nothing about the
+ *              epilogue is decided by a branch inside the kernel.
  * All phases are written out (2, 4 or 8 for C = 64, 128, 256); V has four slots in LDS, a fifth phase takes the first slot again.
  * Limits: 16-bit tensors, 3x3, stride 1, dilation 1, zero padding value, C = 64, 128 or 256, K a multiple of 128, beta = 0,
  * LINEAR or RELU, images that tile into at most 128 (row, pair) positions per workgroup (see choose_tile), values within the
