@@ -118,6 +118,30 @@ def test_through_the_dispatcher(oracle, rows_forced, dtype, case):
     assert err < BAR
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("channels", [64, 128, 256])
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("residual", [False, True])
+def test_every_instance_of_the_kernel(oracle, rows_forced, dtype, channels, relu, residual):
+    """The kernel is instantiated per tensor type, channel count (2, 4 or 8 phases), activation and residual: every one of the 24
+    on a small layer with two bands per image and a ragged last band."""
+    g = h.rng(370 + channels + 2 * relu + residual)
+    xs, ws = (3, 19, 14, channels), (128, 3, 3, channels)
+    s = shape_of(xs, ws)
+    assert rows_forced.avhip_conv2d_winograd_rows_plan(h.DT[dtype], C.byref(s), None, None) == 0, "the kernel must take this layer"
+    x = h.rounded(oracle, g.standard_normal(xs), dtype)
+    w = he(g, ws, dtype, oracle)
+    b = g.uniform(-0.1, 0.1, ws[0]).astype(np.float32).astype(np.float64)
+    ys = (xs[0], s.Ho, s.Wo, ws[0])
+    z = h.rounded(oracle, g.standard_normal(ys), dtype) if residual else None
+    got = h.conv_forward("dispatch", x, w, ys, dtype, bias=b, z=z, alpha1=0.9, alpha2=1.3 if residual else None,
+                         activation=cb.ACTIVATION_RELU if relu else 0)
+    want = oracle.conv2d(x, w, b, z=z, alpha1=0.9, alpha2=1.3 if residual else 1.0, activation=oracle.RELU if relu else oracle.LINEAR)
+    err = oracle.rel_l2(got, want)
+    print("rows instance %s C=%d relu=%d z=%d rel-L2 = %.3e" % (dtype, channels, relu, residual, err))
+    assert err < BAR
+
+
 ROUNDS_CASES = [
     # layers of more workgroups than the device has compute units (several rounds of workgroups)
     dict(x=(70, 28, 28, 64), w=(128, 3, 3, 64)),                                          # 280 workgroups
